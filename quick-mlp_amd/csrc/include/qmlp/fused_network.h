@@ -1,0 +1,243 @@
+#pragma once
+
+#include "activation.h"
+#include "common.h"
+#include "iencoding.h"
+#include "json.h"
+#include "kernel_loader.h"
+#include "tensor.h"
+
+#include <optional>
+#include <random>
+#include <vector>
+
+QUICKMLP_NAMESPACE_BEGIN
+
+/**
+ * A fully fused coordinate MLP: input encodings, linear layers and activations in one
+ * generated kernel per pass (inference, forward with stored intermediates, adjoint),
+ * plus one batch-reduction kernel per layer for the weight gradients.
+ */
+class FusedNetwork : NonAssignable
+{
+public:
+    /** additive flags specifying what gradients to compute in the adjoint pass */
+    enum AdjointMode
+    {
+        //Compute gradients with respect to the network input
+        GRADIENTS_INPUT = 0x1,
+        //Compute gradients with respect to the network weights
+        GRADIENTS_NETWORK_WEIGHTS = 0x2,
+        //Compute gradients with respect to the input encodings
+        GRADIENTS_INPUT_ENCODINGS = 0x4,
+
+        ADJOINT_MODE_MAX_COMBINATIONS = 8
+    };
+    typedef int AdjointModeFlags;
+
+    /** Compile options, loaded from the json ("options"). */
+    struct CompileOptions
+    {
+        //Overwrites the kernel block size (threads, multiple of the wavefront size).
+        //If <=0 (the default), the library chooses.
+        int overwriteBlocksizeInference = -1;
+        int overwriteBlocksizeForward = -1;
+        int overwriteBlocksizeBackward = -1;
+        int overwriteBlocksizeWeightUpdate = -1;
+
+        // Accepted for compatibility; the LDS layouts of this implementation are
+        // bank-conflict free for 64 lanes by construction and need no skew.
+        bool skewSharedMemory = false;
+
+        // If true, the per-layer weight update kernels are launched on separate
+        // streams that fork from / join into the caller's stream.
+        bool parallelWeightUpdate = true;
+    };
+
+private:
+    struct LayerSpecification
+    {
+        //specs from Json
+        int channelsOut;
+        bool useBias;
+        //Either a single entry, used for every channel, or one per channel (unsupported in the kernels)
+        std::vector<Activation_ptr> activations;
+
+        //cached parameter for easy access
+        int channelsIn;
+        //prefix sum, offset into parameter array
+        int weightsStart;
+        int biasStart;
+    };
+
+    CompileOptions compileOptions_;
+    int channelsIn_;
+    int channelsOut_;
+    int encodedChannels_;
+    int networkInputPadding_;
+    std::vector<IEncoding_ptr> encodings_;
+    std::vector<LayerSpecification> layers_;
+
+    int numParameters_;
+    Tensor parametersInference_;
+    Tensor parametersGradients_;
+
+    struct CompiledKernel
+    {
+        KernelFunction fun;
+        int blockSize = 0;
+        int sharedMemorySize = 0;
+        int fullGrid = 0;
+    };
+    std::optional<CompiledKernel> inferenceKernel_;
+    std::optional<CompiledKernel> forwardKernel_;
+
+    struct AdjointLayerInfo
+    {
+        //channel prefix of this layer's adjoint pre-activations in the adjoint tmp memory
+        int offsetAdjOut;
+        //channel prefix of this layer's input in the forward tmp memory (encoded input for layer 0)
+        int offsetIn;
+        //channel prefix of this layer's pre-activations in the forward tmp memory
+        int offsetPre;
+
+        stream_t stream = nullptr;
+        event_t event = nullptr;
+    };
+    struct WeightUpdateKernel
+    {
+        CompiledKernel kernel;
+        int numChunks = 1;
+    };
+    struct AdjointKernel
+    {
+        CompiledKernel adjoint;
+        std::vector<WeightUpdateKernel> layers;
+        int perEntryAdjointMemoryBytes = 0;
+    };
+    std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS];
+
+    int perEntryForwardMemoryBytes_;
+    std::vector<AdjointLayerInfo> backwardInfo_;
+    event_t adjointEvent_;
+    bool streamsCreated_;
+
+public:
+    //Size of the matrix fragments: all layer widths are padded to multiples of this.
+    static constexpr int MATRIX_SIZE = 16;
+    //Wavefront size; one wavefront processes a tile of this many points and
+    //temporary memory is a multiple of that value
+    static constexpr int WARP_SIZE = 64;
+
+    //LDS available to one workgroup on the current device
+    static int MaxSharedMemoryBytes();
+
+    /**
+     * Constructs the network from the Json configuration 'cfg'. 'parent' is the folder
+     * relative to which activation files are resolved. After constructing, the
+     * configuration is immutable, so that kernels are compiled once and cached.
+     */
+    FusedNetwork(const json& cfg, const std::filesystem::path& parent);
+    ~FusedNetwork();
+
+    [[nodiscard]] const std::vector<IEncoding_ptr>& encodings() const { return encodings_; }
+    [[nodiscard]] int numEncodings() const { return static_cast<int>(encodings_.size()); }
+    [[nodiscard]] IEncoding_ptr encoding(int idx);
+
+    [[nodiscard]] int channelsIn() const { return channelsIn_; }
+    [[nodiscard]] int channelsOut() const { return channelsOut_; }
+    [[nodiscard]] Tensor::Precision precisionIn() const { return Tensor::FLOAT; }
+    [[nodiscard]] Tensor::Precision precisionOut() const { return Tensor::FLOAT; }
+    [[nodiscard]] int numLayers() const { return static_cast<int>(layers_.size()); }
+    [[nodiscard]] const CompileOptions& compileOptions() const { return compileOptions_; }
+    [[nodiscard]] bool isParallelStreams() const { return compileOptions_.parallelWeightUpdate; }
+    void setParallelStreams(bool enabled) { compileOptions_.parallelWeightUpdate = enabled; }
+
+    [[nodiscard]] int networkParameterCount() const;
+    [[nodiscard]] Tensor::Precision networkParameterPrecision(Tensor::Usage usage) const;
+
+    /**
+     * Sets the network parameters to the specified tensor: 1D, networkParameterCount()
+     * entries of type networkParameterPrecision(usage). The memory stays owned by the caller.
+     * Layout: all weight matrices in layer order (row-major (C_out, C_in), padded widths),
+     * then the bias vectors of the layers that have one.
+     */
+    void setNetworkParameter(const Tensor& tensor, Tensor::Usage usage);
+
+    /**
+     * Initializes the inference weights to U(-1/sqrt(C_in), 1/sqrt(C_in)) (the default
+     * initialization of torch.nn.Linear), drawn row-major layer by layer.
+     */
+    void initializeInferenceParameters(std::default_random_engine& rng);
+
+    /**
+     * Returns the slice of the parameters for the weight matrix (bias=false) or bias
+     * vector (bias=true) of layer 'layer'; shares memory with 'rawPtr'.
+     */
+    Tensor networkParameter(int layer, bool bias, void* rawPtr, Tensor::Precision precision);
+    Tensor networkParameter(int layer, bool bias, Tensor::Usage usage);
+
+    /**
+     * Inference.
+     * \param input (N, channelsIn) float  \param output (N, channelsOut) float
+     * \param stream the stream the kernel is enqueued on
+     */
+    void inference(const Tensor& input, Tensor& output, stream_t stream);
+
+    /** Bytes of temporary memory forward() needs for 'numElements' points. */
+    size_t forwardMemory(int numElements, AdjointModeFlags adjointFlags);
+    size_t forwardMemory(const Tensor& input, AdjointModeFlags adjointFlags);
+
+    /**
+     * Forward pass that stores intermediate results in 'tmpMemory' (forwardMemory() bytes,
+     * 16-byte aligned) for a following adjoint().
+     */
+    void forward(const Tensor& input, Tensor& output, void* tmpMemory, stream_t stream);
+
+    /** Zeros the gradients of the network weights and of the encodings. */
+    void zeroGradients();
+
+    /** Bytes of temporary memory adjoint() needs for 'numElements' points. */
+    size_t adjointMemory(int numElements, AdjointModeFlags adjointFlags);
+    size_t adjointMemory(const Tensor& input, AdjointModeFlags adjointFlags);
+
+    /**
+     * Adjoint pass following forward(). Weight and encoding gradients are added to the
+     * gradient tensors set via setNetworkParameter / IEncoding::setParameter with
+     * Usage::GRADIENTS; input gradients are added to 'adjInput'.
+     */
+    void adjoint(const Tensor& input, const Tensor& adjOutput, AdjointModeFlags adjointFlags, Tensor& adjInput,
+                 const void* tmpMemoryForward, void* tmpMemoryAdjoint, stream_t stream);
+
+    /** For debugging, clears all cached kernels. */
+    void clearCachedKernels();
+
+    /**
+     * Generates and compiles all kernels for the given adjoint flags without a GPU
+     * (flags < 0: inference and forward only). Fills the kernel disk cache.
+     */
+    void precompile(int adjointFlags);
+
+    /** The generated device source of a kernel kind: "inference", "backward", "weight_update". */
+    std::string generatedSource(const std::string& kind, int adjointFlags = 0);
+
+private:
+    void compileInferenceKernel(bool compileOnly = false);
+    void compileForwardKernel(bool compileOnly = false);
+    void compileBackwardKernel(int flags, bool compileOnly = false);
+
+    std::string forwardSource(int blockSize) const;
+    std::string backwardSource(int flags, int blockSize) const;
+    std::string weightUpdateSource(int blockSize) const;
+    std::string weightUpdateKernelName(int layer, int& numChunks) const;
+    void fillEncodingsAndActivations(std::string& codeTemplate) const;
+    int forwardBlockSize(int overwrite, bool adjoint) const;
+    int ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const;
+    int ldsParamHalves(bool adjoint) const;
+    int stageBytesPerWave() const;
+    std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);
+    void ensureStreams();
+};
+typedef std::shared_ptr<FusedNetwork> FusedNetwork_ptr;
+
+QUICKMLP_NAMESPACE_END

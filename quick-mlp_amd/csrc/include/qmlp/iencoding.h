@@ -1,0 +1,137 @@
+#pragma once
+
+#include "common.h"
+#include "json.h"
+#include "kernel_loader.h"
+#include "tensor.h"
+
+#include <functional>
+#include <optional>
+#include <sstream>
+#include <unordered_map>
+#include <vector>
+
+QUICKMLP_NAMESPACE_BEGIN
+
+/**
+ * Defines an input encoding.
+ *
+ * What the device-side implementation must provide:
+ * <code>
+ * struct NameOfEncoding
+ * {
+ *     static constexpr int NumOutputs;
+ *     template<typename I, typename O>
+ *     static __device__ void forward(const I& input, O& output [, const param-type& params ]);
+ *
+ *     template<bool EvaluateInputGradients, bool EvaluateParameterGradients, typename I, typename O, typename AdjI>
+ *     static __device__ void adjoint(const I& input, const O& adjOutput, AdjI& adjInput [, const param-type& params ]);
+ * }
+ * </code>
+ * 'input' is indexable with operator[] and yields the raw float inputs of one point;
+ * 'output' is indexable, assignable and has a typedef ValueType (float or a half type).
+ * Encodings with parameters receive them as one by-value kernel argument of the type
+ * named by parameterName(), whose bytes fillParameterMemory() produces.
+ */
+class IEncoding
+{
+public:
+    virtual ~IEncoding() = default;
+
+    [[nodiscard]] virtual json toJson() const = 0;
+    [[nodiscard]] virtual std::string id() const = 0;
+
+    /** The maximal addressed input channel, e.g. 2 for a 3D index. */
+    [[nodiscard]] virtual int maxInputChannel() const = 0;
+
+    /** The number of output channels */
+    [[nodiscard]] virtual int numOutputChannels() const = 0;
+
+    /** The qualified device type of the encoding including all template arguments. */
+    [[nodiscard]] virtual std::string qualifiedName() const = 0;
+
+    /** Appends the device code needed by qualifiedName(): includes and generated definitions. */
+    virtual void fillCode(std::stringstream& code) const = 0;
+
+    /** True iff the encoding has a parameter structure (and trainable parameters). */
+    [[nodiscard]] virtual bool hasParameters() const { return false; }
+
+    /** Fully-qualified device type of the parameter structure. */
+    [[nodiscard]] virtual std::string parameterName() const { return ""; }
+
+    [[nodiscard]] virtual Tensor::Precision parameterPrecision(Tensor::Usage usage) const { return Tensor::FLOAT; }
+
+    [[nodiscard]] virtual int parameterCount() const { return 0; }
+
+    /**
+     * Sets the underlying parameter to the specified tensor: 1D with parameterCount()
+     * entries of type parameterPrecision(usage). An undefined tensor clears it.
+     */
+    virtual void setParameter(const Tensor& tensor, Tensor::Usage usage) {}
+
+    /**
+     * Writes the bytes of the parameter structure (kernel argument) into 'dst' with a
+     * capacity of 'dstSize' bytes; returns the number of bytes written.
+     */
+    [[nodiscard]] virtual int fillParameterMemory(char* dst, int dstSize) { return 0; }
+
+    /** Zeros the gradients of this encoding's parameters (no-op without parameters). */
+    virtual void zeroGradients() {}
+
+    /**
+     * Standalone forward pass.
+     * \param input shape (B, Cin), float32
+     * \param output shape (B, >= numOutputChannels()), float32, unit stride along the channels
+     * \param parametersForward optional override of the inference parameters for this call
+     */
+    virtual void forward(const Tensor& input, Tensor& output, stream_t stream,
+                         const std::optional<const Tensor>& parametersForward);
+
+    enum AdjointMode
+    {
+        INPUT_GRADIENTS = 0x1,
+        PARAM_GRADIENTS = 0x2,
+        ALL_GRADIENTS = INPUT_GRADIENTS | PARAM_GRADIENTS
+    };
+
+    /**
+     * Standalone adjoint pass; adjInput (B, Cin) and the parameter gradients are accumulated.
+     */
+    virtual void adjoint(const Tensor& input, const Tensor& adjOutput, Tensor& adjInput, stream_t stream,
+                         const std::optional<const Tensor>& parametersForward,
+                         const std::optional<const Tensor>& parametersGradients,
+                         int adjointMode = AdjointMode::ALL_GRADIENTS);
+
+private:
+    std::optional<KernelFunction> forwardKernel_;
+    std::optional<KernelFunction> adjointKernel_[AdjointMode::ALL_GRADIENTS + 1];
+};
+typedef std::shared_ptr<IEncoding> IEncoding_ptr;
+
+/**
+ * Encodings over a bounded volume; can serve as child of other encodings.
+ */
+class IVolumetricEncoding : public IEncoding
+{
+public:
+    [[nodiscard]] virtual int ndim() const = 0;
+
+    typedef std::vector<float> BoundingBoxVector_t;
+    [[nodiscard]] virtual BoundingBoxVector_t boundingBoxMin() const = 0;
+    [[nodiscard]] virtual BoundingBoxVector_t boundingBoxSize() const = 0;
+    [[nodiscard]] virtual BoundingBoxVector_t boundingBoxInvSize() const = 0;
+};
+
+class EncodingFactory
+{
+private:
+    EncodingFactory();
+    typedef std::function<IEncoding_ptr(const json&)> factory_t;
+    std::unordered_map<std::string, factory_t> encodings_;
+
+public:
+    static EncodingFactory& Instance();
+    IEncoding_ptr create(const json& cfg);
+};
+
+QUICKMLP_NAMESPACE_END

@@ -1,0 +1,105 @@
+#pragma once
+// Device-side basics shared by every runtime-compiled QuickMLP kernel (gfx950, wave64).
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <qmlp/kernels/tensor.h>
+
+#define QUICKMLP_KERNEL_NAMESPACE ::qmlp::kernel
+#define QUICKMLP_KERNEL_NAMESPACE_BEGIN namespace qmlp { namespace kernel {
+#define QUICKMLP_KERNEL_NAMESPACE_END }}
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+typedef _Float16 f16;
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// One wavefront works on a tile of 64 points: NT column tiles of 16 points each.
+// Lane l = 16*g + r. In an MFMA accumulator tile the lane holds output rows
+// 4g..4g+3 (channels) of column r; column r of column-tile nt is point 4*r + nt
+// of the 64-point tile, so that one lane owns 4 consecutive points per channel.
+constexpr int WAVE_SIZE = 64;
+constexpr int TILE_POINTS = 64;
+constexpr int NT = 4;
+
+__device__ __forceinline__ half hZERO() { return __half_raw{static_cast<f16>(0)}; }
+__device__ __forceinline__ half2 h2ZERO() { return __half2{hZERO(), hZERO()}; }
+
+__device__ __forceinline__ half toHalf(f16 v) { return __half_raw{v}; }
+__device__ __forceinline__ f16 fromHalf(half v) { return static_cast<__half_raw>(v).data; }
+
+/** Templated casting between float and half datatypes */
+template <typename Dst, typename Src> __device__ __forceinline__ Dst fcast(const Src& src);
+template <> __device__ __forceinline__ float fcast<float, half>(const half& src) { return __half2float(src); }
+template <> __device__ __forceinline__ float fcast<float, float>(const float& src) { return src; }
+template <> __device__ __forceinline__ half fcast<half, half>(const half& src) { return src; }
+template <> __device__ __forceinline__ half fcast<half, float>(const float& src) { return __float2half(src); }
+template <> __device__ __forceinline__ float fcast<float, f16>(const f16& src) { return static_cast<float>(src); }
+template <> __device__ __forceinline__ f16 fcast<f16, float>(const float& src) { return static_cast<f16>(src); }
+template <> __device__ __forceinline__ f16 fcast<f16, f16>(const f16& src) { return src; }
+
+/**
+ * Orders LDS traffic between the lanes of one wavefront: everything written before
+ * is visible to every lane's reads after. Waves run their tile loops independently,
+ * so a workgroup barrier must not be used inside them.
+ */
+__device__ __forceinline__ void waveLdsSync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+/** Row of the per-wave staging area that holds point p (0..63) of the tile. Points
+ *  4r+nt (fixed nt) of the 16 lanes r land in 16 consecutive rows, which together with
+ *  an odd multiple of 16 bytes as row stride makes the tile reads bank-conflict free. */
+__device__ __forceinline__ int stageRow(int p) { return ((p & 3) << 4) | (p >> 2); }
+
+__device__ __forceinline__ f16x8 concat(f16x4 a, f16x4 b)
+{
+    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+__device__ __forceinline__ f16x4 toF16(f32x4 v)
+{
+    f16x4 o;
+    o[0] = static_cast<f16>(v[0]);
+    o[1] = static_cast<f16>(v[1]);
+    o[2] = static_cast<f16>(v[2]);
+    o[3] = static_cast<f16>(v[3]);
+    return o;
+}
+
+template <typename Act>
+__device__ __forceinline__ f16x4 activationForward(f16x4 v)
+{
+    f16x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = fromHalf(Act::forward(toHalf(v[i])));
+    return o;
+}
+
+template <typename Act>
+__device__ __forceinline__ f16x8 activationForward(f16x8 v)
+{
+    f16x8 o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = fromHalf(Act::forward(toHalf(v[i])));
+    return o;
+}
+
+/** One row of a strided 2-D tensor. */
+template <typename T>
+struct RowAccessor
+{
+    T* p;
+    int stride;
+    __device__ __forceinline__ T& operator[](int i) const { return p[static_cast<long long>(i) * stride]; }
+};
+
+QUICKMLP_KERNEL_NAMESPACE_END

@@ -1,0 +1,64 @@
+// Template of the standalone encoding kernels (fp32 in, fp32 out). Everything in
+// $$..$$ is replaced by the host before compilation.
+// Replaces src_cpp/include/qmlp/kernels/encoding_kernels.cuh:26-62 of the reference.
+
+#include <qmlp/kernels/common.h>
+#include <qmlp/kernels/arrays.h>
+
+$$INCLUDES$$
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+__global__ void EncodingForwardKernel(
+    long long numel,
+    const Tensor2Read<float> inputs,  //shape (numel, Cin)
+    Tensor2RW<float> outputs          //shape (numel, Cout), unit stride along the channels
+    $$ENCODING_PARAMETERS$$)
+{
+    for (long long index = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; index < numel;
+         index += static_cast<long long>(blockDim.x) * gridDim.x)
+    {
+        const StridedArray<const float> encodingInput{inputs.data_ + index * inputs.strides_[0], inputs.strides_[1]};
+        WrappedArray<float> encodingOutput{outputs.data_ + index * outputs.strides_[0]};
+        $$CALL_ENCODINGS_FORWARD$$
+    }
+}
+
+__global__ void EncodingAdjointKernel(
+    long long numel,
+    const Tensor2Read<float> inputs,      //shape (numel, Cin)
+    const Tensor2Read<float> adjOutputs,  //shape (numel, Cout)
+    Tensor2RW<float> adjInputs            //shape (numel, Cin), accumulated
+    $$ENCODING_PARAMETERS$$)
+{
+    for (long long index = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; index < numel;
+         index += static_cast<long long>(blockDim.x) * gridDim.x)
+    {
+        const StridedArray<const float> encodingInput{inputs.data_ + index * inputs.strides_[0], inputs.strides_[1]};
+        const StridedArray<const float> encodingAdjOutput{adjOutputs.data_ + index * adjOutputs.strides_[0], adjOutputs.strides_[1]};
+        StridedArray<float> encodingAdjInput{adjInputs.data_ + index * adjInputs.strides_[0], adjInputs.strides_[1]};
+        $$CALL_ENCODINGS_ADJOINT$$
+    }
+}
+
+// Test aid: table offsets and interpolation weights of every corner of every level.
+__global__ void EncodingCornersKernel(
+    long long numel,
+    const Tensor2Read<float> inputs,  //shape (numel, Cin)
+    unsigned* __restrict__ indices,   //shape (numel, perPoint)
+    float* __restrict__ weights,      //shape (numel, perPoint)
+    int perPoint
+    $$ENCODING_PARAMETERS$$)
+{
+    for (long long index = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; index < numel;
+         index += static_cast<long long>(blockDim.x) * gridDim.x)
+    {
+        const StridedArray<const float> encodingInput{inputs.data_ + index * inputs.strides_[0], inputs.strides_[1]};
+        unsigned* cornerIndices = indices + index * perPoint;
+        float* cornerWeights = weights + index * perPoint;
+        (void)encodingInput; (void)cornerIndices; (void)cornerWeights;
+        $$CALL_ENCODINGS_CORNERS$$
+    }
+}
+
+QUICKMLP_KERNEL_NAMESPACE_END

@@ -1,0 +1,206 @@
+#pragma once
+// One fully-connected layer of the fused network on a 64-point wavefront tile.
+//
+// Every layer is the contraction  Y^T (C_out x points) = W (C_out x C_in) * X^T (C_in x points)
+// on the matrix cores: A = a 16-row tile of W, B = activations of 16 points,
+// fp16 operands, fp32 accumulation (v_mfma_f32_16x16x32_f16; an odd trailing
+// 16-channel tile is paired with a zero tile). The accumulator layout (lane 16g+r
+// holds channels 4g..4g+3 of point column r) is exactly the layout the next
+// layer's B operand needs once the contraction index is permuted accordingly: a
+// k-block of 32 channels built from the 16-channel tiles t0,t1 assigns to lane
+// group g the channels 16*t0+4g+{0..3} and 16*t1+4g+{0..3}. Because only the
+// weights have to follow that permutation (done once while staging them into LDS),
+// activations stay in registers from the first to the last layer.
+//
+// Only one MFMA shape is used on purpose: with the ROCm 7.2 compiler at -O3, a
+// v_mfma_f32_16x16x16_f16 accumulating onto the result of the v_mfma_f32_16x16x32_f16
+// issued right before it was observed to deliver wrong accumulator elements 0 and 1
+// on gfx950 (fewer of them when MFMAs were padded with wait states).
+//
+// Replaces Layer<...>::inference / ::adjoint of the reference
+// (src_cpp/include/qmlp/kernels/layer.cuh:86-266), which round-trips the activations
+// through shared memory between layers and accumulates in half precision.
+
+#include <qmlp/kernels/common.h>
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+__device__ __forceinline__ f32x4 mfma32(f16x8 a, f16x8 b, f32x4 c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+/**
+ * \tparam CIN padded input channels (multiple of 16)
+ * \tparam COUT padded output channels (multiple of 16)
+ * \tparam BIAS layer has a bias vector
+ * \tparam Activation struct with static half forward(half), half adjoint(half x, half adjz)
+ */
+template <int CIN, int COUT, bool BIAS, typename Activation>
+struct Layer
+{
+    static constexpr int KT = CIN / 16;     // 16-channel tiles of the input
+    static constexpr int MT = COUT / 16;    // 16-channel tiles of the output
+    // forward operand order: per output tile m, ceil(KT/2) blocks of 64 lanes x 8 halves;
+    // if KT is odd the upper 4 halves of the last block are zero
+    static constexpr int F_KB = (KT + 1) / 2;
+    static constexpr int F_MSTRIDE = F_KB * 512;
+    static constexpr int F_LDS_HALVES = MT * F_MSTRIDE;
+    // adjoint (transposed) operand order: per input tile, ceil(MT/2) blocks
+    static constexpr int A_KB = (MT + 1) / 2;
+    static constexpr int A_MSTRIDE = A_KB * 512;
+    static constexpr int A_LDS_HALVES = KT * A_MSTRIDE;
+
+    /**
+     * Copies the row-major (COUT, CIN) weight matrix into LDS in forward operand
+     * order. Called by all threads of the block; 'W' must be 8-byte aligned.
+     */
+    __device__ static void stageForward(const f16* __restrict__ W, f16* __restrict__ dst, int tid, int nthreads)
+    {
+        // one unit = 4 consecutive halves of a weight row
+        constexpr int UNITS = F_LDS_HALVES / 4;
+        for (int u = tid; u < UNITS; u += nthreads) {
+            const int m = u / (F_MSTRIDE / 4);
+            int rest = u - m * (F_MSTRIDE / 4);
+            const int kb = rest / 128;
+            rest -= kb * 128;
+            const int lane = rest >> 1;
+            const int tile = 2 * kb + (rest & 1);
+            const int g = lane >> 4, r = lane & 15;
+            f16x4 v = {0, 0, 0, 0};
+            if (tile < KT) v = *reinterpret_cast<const f16x4*>(W + (16 * m + r) * CIN + 16 * tile + 4 * g);
+            *reinterpret_cast<f16x4*>(dst + 4 * u) = v;
+        }
+    }
+
+    /**
+     * Copies the weight matrix into LDS in adjoint operand order (A = tiles of W^T).
+     */
+    __device__ static void stageAdjoint(const f16* __restrict__ W, f16* __restrict__ dst, int tid, int nthreads)
+    {
+        constexpr int N = A_LDS_HALVES;
+        for (int e = tid; e < N; e += nthreads) {
+            const int mi = e / A_MSTRIDE;
+            int rest = e - mi * A_MSTRIDE;
+            const int kb = rest / 512;
+            rest -= kb * 512;
+            const int lane = rest >> 3;
+            const int slot = rest & 7;
+            const int tile = 2 * kb + (slot >> 2);
+            const int j = slot & 3;
+            const int g = lane >> 4, r = lane & 15;
+            dst[e] = tile < MT ? W[(16 * tile + 4 * g + j) * CIN + 16 * mi + r] : static_cast<f16>(0);
+        }
+    }
+
+    /**
+     * Forward pass of the layer for one 64-point tile.
+     * \param w LDS weights in forward operand order
+     * \param bias LDS bias vector (COUT halves) or nullptr
+     * \param x input activations: x[nt][t] = channels 16t+4g+{0..3} of point 4r+nt
+     * \param y output activations in the same layout
+     * \param preTile [STORE] where the pre-activations of this tile go: (COUT, 64) halves,
+     *        channel-major, so that both the adjoint pass (per channel, 4 points of one
+     *        lane) and the weight update (per channel, 8 consecutive points) read it
+     *        with wide loads
+     */
+    template <bool STORE>
+    __device__ __forceinline__ static void forward(const f16* __restrict__ w, const f16* __restrict__ bias,
+                                                   const f16x4 (&x)[NT][KT], f16x4 (&y)[NT][MT],
+                                                   f16* __restrict__ preTile, int lane)
+    {
+        const int g = lane >> 4, r = lane & 15;
+        const f16x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            f32x4 acc[NT];
+            if constexpr (BIAS) {
+                const f16x4 b = *reinterpret_cast<const f16x4*>(bias + 16 * m + 4 * g);
+                const f32x4 bf = {static_cast<float>(b[0]), static_cast<float>(b[1]),
+                                  static_cast<float>(b[2]), static_cast<float>(b[3])};
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = bf;
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int kb = 0; kb < F_KB; ++kb) {
+                const f16x8 a = *reinterpret_cast<const f16x8*>(w + m * F_MSTRIDE + kb * 512 + lane * 8);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const f16x4 hi = (2 * kb + 1 < KT) ? x[nt][(2 * kb + 1 < KT) ? 2 * kb + 1 : 0] : zero4;
+                    acc[nt] = mfma32(a, concat(x[nt][2 * kb], hi), acc[nt]);
+                }
+            }
+            f16x4 p[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) p[nt] = toF16(acc[nt]);
+            if constexpr (STORE) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f16x4 v = {p[0][i], p[1][i], p[2][i], p[3][i]};
+                    *reinterpret_cast<f16x4*>(preTile + (16 * m + 4 * g + i) * TILE_POINTS + 4 * r) = v;
+                }
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) y[nt][m] = activationForward<Activation>(p[nt]);
+        }
+    }
+
+    /**
+     * Adjoint pass of the layer for one 64-point tile.
+     * \param wT LDS weights in adjoint operand order
+     * \param dy in: adjoint of the layer output (after the activation);
+     *           out: adjoint of the pre-activation, zeroed for points outside the batch
+     * \param dx adjoint of the layer input (only written if COMPUTE_DX)
+     * \param preTile pre-activations stored by forward<true>
+     * \param dpreTile [STORE_DPRE] receives the pre-activation adjoints, same layout
+     * \param validMask bit nt set iff point 4r+nt of this lane is inside the batch
+     */
+    template <bool STORE_DPRE, bool COMPUTE_DX>
+    __device__ __forceinline__ static void adjoint(const f16* __restrict__ wT, f16x4 (&dy)[NT][MT],
+                                                   f16x4 (&dx)[NT][KT], const f16* __restrict__ preTile,
+                                                   f16* __restrict__ dpreTile, int validMask, int lane)
+    {
+        const int g = lane >> 4, r = lane & 15;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16x4 pre = *reinterpret_cast<const f16x4*>(preTile + (16 * m + 4 * g + i) * TILE_POINTS + 4 * r);
+                f16x4 d;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const half a = Activation::adjoint(toHalf(pre[nt]), toHalf(dy[nt][m][i]));
+                    d[nt] = ((validMask >> nt) & 1) ? fromHalf(a) : static_cast<f16>(0);
+                    dy[nt][m][i] = d[nt];
+                }
+                if constexpr (STORE_DPRE)
+                    *reinterpret_cast<f16x4*>(dpreTile + (16 * m + 4 * g + i) * TILE_POINTS + 4 * r) = d;
+            }
+        }
+        if constexpr (COMPUTE_DX) {
+            const f16x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+            for (int mi = 0; mi < KT; ++mi) {
+                f32x4 acc[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kb = 0; kb < A_KB; ++kb) {
+                    const f16x8 a = *reinterpret_cast<const f16x8*>(wT + mi * A_MSTRIDE + kb * 512 + lane * 8);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const f16x4 hi = (2 * kb + 1 < MT) ? dy[nt][(2 * kb + 1 < MT) ? 2 * kb + 1 : 0] : zero4;
+                        acc[nt] = mfma32(a, concat(dy[nt][2 * kb], hi), acc[nt]);
+                    }
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) dx[nt][mi] = toF16(acc[nt]);
+            }
+        }
+    }
+};
+
+QUICKMLP_KERNEL_NAMESPACE_END

@@ -1,0 +1,136 @@
+// Template of the fused adjoint kernel. The host code generator replaces everything
+// in $$..$$ before the source is handed to the runtime compiler.
+//
+// Per 64-point wavefront tile: dL/dy is loaded straight into the accumulator layout
+// of the matrix cores, each layer (last to first) applies the activation adjoint on
+// the stored pre-activations and contracts with the transposed weights
+// (dX = W^T dpre, the same MFMA path as the forward pass with the weight tiles
+// staged transposed), optionally storing dpre for the weight update. The adjoint of
+// the encoded input finally goes through the LDS staging rows to one lane per point,
+// which accumulates input gradients and scatter-adds grid gradients with hardware
+// fp32 atomics.
+//
+// Replaces NetworkKernelBackward of the reference
+// (src_cpp/include/qmlp/kernels/network_backward.cuh:33-114). Unlike the reference it
+// never reads dL/dy beyond the real output channels: padded channels are zero.
+
+#include <qmlp/kernels/common.h>
+#include <qmlp/kernels/arrays.h>
+#include <qmlp/kernels/layer.h>
+
+$$INCLUDES$$
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+namespace activations
+{
+$$DEFINE_ACTIVATIONS$$
+}
+
+__global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
+    int numel,
+    const Tensor2Read<float> inputs,      //shape (numel, Cin)
+    const Tensor2Read<float> adjOutputs,  //shape (numel, Cout)
+    Tensor2RW<float> adjInputs,           //shape (numel, Cin), accumulated; unused without input gradients
+    const half* __restrict__ networkParametersH,
+    const half* __restrict__ forwardTmpMemoryH,  //written by the forward kernel
+    half* __restrict__ adjointTmpMemoryH         //receives dpre if weight gradients are requested
+    $$ENCODING_PARAMETERS$$)
+{
+    constexpr int NUM_INPUTS = $$NUM_INPUTS$$;
+    constexpr int ENCODED_CHANNELS = $$ENCODED_CHANNELS$$;
+    constexpr int CHANNELS_IN = $$CHANNELS_IN$$;
+    constexpr int CHANNELS_OUT = $$CHANNELS_OUT$$;
+    constexpr int KT0 = CHANNELS_IN / 16;
+    constexpr int MTL = CHANNELS_OUT / 16;
+    constexpr int STAGE_STRIDE = CHANNELS_IN + 8;
+    constexpr int LDS_PARAM_HALVES = $$LDS_PARAM_HALVES$$;
+    constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
+    constexpr bool HAS_INPUT_GRADIENTS = $$HAS_INPUT_GRADIENTS$$;
+    constexpr bool HAS_NETWORK_GRADIENTS = $$HAS_NETWORK_GRADIENTS$$;
+    constexpr bool HAS_ENCODING_GRADIENTS = $$HAS_ENCODING_GRADIENTS$$;
+    // the adjoint of the encoded input is only needed if something sits behind it
+    constexpr bool NEEDS_ENCODING_ADJOINT = HAS_INPUT_GRADIENTS || HAS_ENCODING_GRADIENTS;
+    (void)ENCODED_CHANNELS; (void)NUM_INPUTS; (void)KT0; (void)STAGE_STRIDE;
+
+    const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
+    const f16* __restrict__ forwardTmpMemory = reinterpret_cast<const f16*>(forwardTmpMemoryH);
+    f16* __restrict__ adjointTmpMemory = reinterpret_cast<f16*>(adjointTmpMemoryH);
+
+    extern __shared__ __align__(16) unsigned char sMemory[];
+    f16* sParams = reinterpret_cast<f16*>(sMemory);
+    const int wave = threadIdx.x / WAVE_SIZE;
+    const int lane = threadIdx.x % WAVE_SIZE;
+    const int g = lane >> 4, r = lane & 15;
+    f16* sStage = sParams + LDS_PARAM_HALVES + wave * (TILE_POINTS * STAGE_STRIDE);
+    (void)sStage;
+
+    // stage the transposed weights in operand order
+$$STAGE_PARAMETERS$$
+    __syncthreads();
+
+    const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
+    const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
+    const int actualChannelsOut = adjOutputs.sizes_[1];
+    for (int tile = blockIdx.x * WAVES + wave; tile < numTiles; tile += gridDim.x * WAVES)
+    {
+        // dL/dy -> accumulator layout (fp32 -> fp16), zero outside batch / real channels
+        f16x4 dyOut[NT][MTL];
+        int validMask = 0;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int p = tile * TILE_POINTS + 4 * r + nt;
+            const bool pv = p < numel;
+            validMask |= pv ? (1 << nt) : 0;
+#pragma unroll
+            for (int m = 0; m < MTL; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int c = 16 * m + 4 * g + i;
+                    float v = 0.f;
+                    if (pv && c < actualChannelsOut)
+                        v = adjOutputs.data_[static_cast<long long>(p) * adjOutputs.strides_[0]
+                                             + static_cast<long long>(c) * adjOutputs.strides_[1]];
+                    dyOut[nt][m][i] = static_cast<f16>(v);
+                }
+        }
+
+        // layers, last to first
+$$CALL_NETWORK_LAYERS$$
+
+        if constexpr (NEEDS_ENCODING_ADJOINT) {
+            // adjoint of the encoded input: registers -> one staging row per point
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int t = 0; t < KT0; ++t)
+                    *reinterpret_cast<f16x4*>(sStage + (16 * nt + r) * STAGE_STRIDE + 16 * t + 4 * g) = dxIn[nt][t];
+            waveLdsSync();
+
+            const int index = tile * TILE_POINTS + lane;
+            if (index < numel) {
+                StaticArray<float, NUM_INPUTS> encodingInput;
+#pragma unroll
+                for (int i = 0; i < NUM_INPUTS; ++i)
+                    encodingInput[i] = inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
+                                                    + static_cast<long long>(i) * inputs.strides_[1]];
+                StaticArray<float, NUM_INPUTS> adjEncodingInput;
+#pragma unroll
+                for (int i = 0; i < NUM_INPUTS; ++i) adjEncodingInput[i] = 0.f;
+                WrappedArray<const f16> adjEncodingOutput{sStage + stageRow(lane) * STAGE_STRIDE};
+
+$$CALL_ENCODINGS$$
+
+                if constexpr (HAS_INPUT_GRADIENTS) {
+#pragma unroll
+                    for (int i = 0; i < NUM_INPUTS; ++i)
+                        adjInputs.data_[static_cast<long long>(index) * adjInputs.strides_[0]
+                                        + static_cast<long long>(i) * adjInputs.strides_[1]] += adjEncodingInput[i];
+                }
+            }
+            waveLdsSync();
+        }
+    }
+}
+
+QUICKMLP_KERNEL_NAMESPACE_END

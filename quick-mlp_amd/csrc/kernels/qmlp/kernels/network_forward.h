@@ -1,0 +1,138 @@
+// Template of the fused forward / inference kernel. The host code generator replaces
+// everything in $$..$$ before the source is handed to the runtime compiler.
+//
+// One wavefront owns a tile of 64 points: each lane first evaluates all input
+// encodings of one point into a row of the wave's LDS staging area (fp16), then the
+// wave reads the rows back as matrix-core B operands and runs every layer with the
+// activations kept in registers. Weights (and biases) are staged into LDS once per
+// workgroup, already permuted into operand order.
+//
+// Replaces NetworkKernelInferenceAndForward of the reference
+// (src_cpp/include/qmlp/kernels/network_forward.cuh:34-114).
+
+#include <qmlp/kernels/common.h>
+#include <qmlp/kernels/arrays.h>
+#include <qmlp/kernels/layer.h>
+
+$$INCLUDES$$
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+namespace activations
+{
+$$DEFINE_ACTIVATIONS$$
+}
+
+/**
+ * \tparam STORE false: inference. true: additionally stores, per 64-point tile and
+ *   channel-major, the encoded network input and the pre-activations of every layer
+ *   into forwardTmpMemory for the adjoint pass.
+ */
+template <bool STORE>
+__global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForward(
+    int numel,
+    const Tensor2Read<float> inputs,  //shape (numel, Cin)
+    Tensor2RW<float> outputs,         //shape (numel, Cout)
+    const half* __restrict__ networkParametersH,
+    half* __restrict__ forwardTmpMemoryH
+    $$ENCODING_PARAMETERS$$)
+{
+    constexpr int NUM_INPUTS = $$NUM_INPUTS$$;            // raw input channels
+    constexpr int ENCODED_CHANNELS = $$ENCODED_CHANNELS$$;  // sum of encoding outputs
+    constexpr int CHANNELS_IN = $$CHANNELS_IN$$;          // padded to a multiple of 16
+    constexpr int CHANNELS_OUT = $$CHANNELS_OUT$$;        // padded width of the last layer
+    constexpr int KT0 = CHANNELS_IN / 16;
+    constexpr int MTL = CHANNELS_OUT / 16;
+    constexpr int STAGE_STRIDE = CHANNELS_IN + 8;         // halves; odd multiple of 16 bytes
+    constexpr int LDS_PARAM_HALVES = $$LDS_PARAM_HALVES$$;
+    constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
+
+    const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
+    f16* __restrict__ forwardTmpMemory = reinterpret_cast<f16*>(forwardTmpMemoryH);
+
+    extern __shared__ __align__(16) unsigned char sMemory[];
+    f16* sParams = reinterpret_cast<f16*>(sMemory);
+    const int wave = threadIdx.x / WAVE_SIZE;
+    const int lane = threadIdx.x % WAVE_SIZE;
+    const int g = lane >> 4, r = lane & 15;
+    f16* sStage = sParams + LDS_PARAM_HALVES + wave * (TILE_POINTS * STAGE_STRIDE);
+
+    // stage the weights in operand order, then the biases
+$$STAGE_PARAMETERS$$
+    __syncthreads();
+
+    const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
+    const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
+    (void)numel64;
+    for (int tile = blockIdx.x * WAVES + wave; tile < numTiles; tile += gridDim.x * WAVES)
+    {
+        const int index = tile * TILE_POINTS + lane;
+        const bool valid = index < numel;
+
+        // encodings: one point per lane into its staging row
+        {
+            f16* rowPtr = sStage + stageRow(lane) * STAGE_STRIDE;
+            WrappedArray<f16> encodingOutput{rowPtr};
+            if (valid) {
+                StaticArray<float, NUM_INPUTS> encodingInput;
+#pragma unroll
+                for (int i = 0; i < NUM_INPUTS; ++i)
+                    encodingInput[i] = inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
+                                                    + static_cast<long long>(i) * inputs.strides_[1]];
+$$CALL_ENCODINGS$$
+#pragma unroll
+                for (int c = ENCODED_CHANNELS; c < CHANNELS_IN; ++c) rowPtr[c] = static_cast<f16>(0);
+            } else {
+                // rows outside the batch are zero so that no NaN enters the matrix cores
+#pragma unroll
+                for (int c = 0; c < CHANNELS_IN; ++c) rowPtr[c] = static_cast<f16>(0);
+            }
+        }
+        waveLdsSync();
+
+        // B operands of the first layer
+        f16x4 x0[NT][KT0];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int t = 0; t < KT0; ++t)
+                x0[nt][t] = *reinterpret_cast<const f16x4*>(sStage + (16 * nt + r) * STAGE_STRIDE + 16 * t + 4 * g);
+        waveLdsSync();   // the staging rows may be overwritten by the next tile
+
+        if constexpr (STORE) {
+            // encoded input, channel-major per tile, for the weight update of layer 0
+            f16* encTile = forwardTmpMemory + static_cast<long long>(tile) * (CHANNELS_IN * TILE_POINTS);
+#pragma unroll
+            for (int t = 0; t < KT0; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f16x4 v = {x0[0][t][i], x0[1][t][i], x0[2][t][i], x0[3][t][i]};
+                    *reinterpret_cast<f16x4*>(encTile + (16 * t + 4 * g + i) * TILE_POINTS + 4 * r) = v;
+                }
+        }
+
+        // layers
+$$CALL_NETWORK_LAYERS$$
+
+        // output: lane holds channels 16m+4g+i of the points 4r+nt
+        const int actualChannelsOut = outputs.sizes_[1];
+#pragma unroll
+        for (int m = 0; m < MTL; ++m)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = 16 * m + 4 * g + i;
+                if (c < actualChannelsOut) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const int p = tile * TILE_POINTS + 4 * r + nt;
+                        if (p < numel)
+                            outputs.data_[static_cast<long long>(p) * outputs.strides_[0]
+                                          + static_cast<long long>(c) * outputs.strides_[1]]
+                                = static_cast<float>(xOut[nt][m][i]);
+                    }
+                }
+            }
+    }
+}
+
+QUICKMLP_KERNEL_NAMESPACE_END

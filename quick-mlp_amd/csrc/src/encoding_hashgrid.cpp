@@ -1,0 +1,242 @@
+#include <qmlp/encoding_hashgrid.h>
+
+#include <qmlp/qmlp.h>
+
+#include <cmath>
+#include <cstring>
+#include <functional>
+
+QUICKMLP_NAMESPACE_BEGIN
+
+static std::vector<float> vectorOrUnit(const std::vector<float>& vx, int d, float v)
+{
+    if (vx.empty()) return std::vector<float>(d, v);
+    CHECK_ERROR(static_cast<int>(vx.size()) == d,
+                "If a bounding box vector is specified, its dimension must match the configured dimension. Expected ",
+                d, ", actual ", vx.size());
+    return vx;
+}
+
+static std::vector<float> invert(const std::vector<float>& vx)
+{
+    std::vector<float> o(vx.size());
+    for (size_t i = 0; i < vx.size(); ++i) o[i] = 1.f / vx[i];
+    return o;
+}
+
+static LayerCombinationMode parseCombinationMode(const json& j)
+{
+    const std::string s = j.get<std::string>();
+    if (s == "concat" || s == "cat") return LayerCombinationMode::CONCAT;
+    if (s == "add") return LayerCombinationMode::ADD;
+    throw configuration_error("Unknown combination_mode '%s', expected 'concat' or 'add'", s.c_str());
+}
+
+static Tensor::Precision parsePrecision(const json& cfg)
+{
+    const std::string s = cfg.value<std::string>("parameter_precision", "float");
+    if (s == "float" || s == "float32") return Tensor::FLOAT;
+    if (s == "half" || s == "float16") return Tensor::HALF;
+    throw configuration_error("Unknown parameter_precision '%s', expected 'float' or 'half'", s.c_str());
+}
+
+EncodingHashGrid::EncodingHashGrid(int start_channel, int dimension, int num_levels, int num_features_per_level,
+                                   int log2_hashmap_size, int min_resolution, int max_resolution,
+                                   LayerCombinationMode combination_mode,
+                                   const std::vector<float>& bounding_box_min,
+                                   const std::vector<float>& bounding_box_size,
+                                   Tensor::Precision parameter_precision)
+    : startChannel_(start_channel)
+    , dimension_(dimension)
+    , numLevels_(num_levels)
+    , numFeaturesPerLevel_(num_features_per_level)
+    , log2HashmapSize_(log2_hashmap_size)
+    , hashmapSize_(log2_hashmap_size > 0 ? 1 << log2_hashmap_size : -1)
+    , minResolution_(min_resolution)
+    , maxResolution_(max_resolution)
+    , combinationMode_(combination_mode)
+    , boundingBoxMin_(vectorOrUnit(bounding_box_min, dimension, -0.5f))
+    , boundingBoxSize_(vectorOrUnit(bounding_box_size, dimension, 1.0f))
+    , boundingBoxInvSize_(invert(boundingBoxSize_))
+    , parameterPrecision_(parameter_precision)
+{
+    CHECK_ERROR(start_channel >= 0, "start_in must be non-negative but is ", start_channel);
+    CHECK_ERROR(dimension >= 1 && dimension <= 6, "Expected 'dimension' to be in [1,6], but got ", dimension);
+    CHECK_ERROR(num_levels > 0, "num_levels must be positive but is ", num_levels);
+    CHECK_ERROR(num_features_per_level > 0, "num_features_per_level must be positive but is ", num_features_per_level);
+    CHECK_ERROR(log2_hashmap_size < 31, "log2_hashmap_size must be below 31 but is ", log2_hashmap_size);
+    CHECK_ERROR(min_resolution > 0, "min_resolution must be positive but is ", min_resolution);
+    CHECK_ERROR(max_resolution >= min_resolution, "max_resolution must be larger than min_resolution");
+    CHECK_ERROR(parameter_precision == Tensor::FLOAT || parameter_precision == Tensor::HALF,
+                "the grid parameters are stored as float or half");
+
+    // Level table: geometric progression of resolutions, evaluated in double precision.
+    numParameters_ = 0;
+    double levelScale = 1;
+    if (num_levels > 1)
+        levelScale = std::exp((std::log(max_resolution) - std::log(min_resolution)) / (num_levels - 1));
+
+    long long total = 0;
+    for (int l = 0; l < num_levels; ++l) {
+        const int resolution = static_cast<int>(std::floor(min_resolution * (std::pow(levelScale, l))));
+        // saturating R^D so that huge fine levels simply count as "too large to be dense"
+        size_t requiredCells = 1;
+        bool overflow = false;
+        for (int d = 0; d < dimension; ++d) {
+            if (requiredCells > (size_t(1) << 40)) overflow = true;
+            requiredCells *= static_cast<size_t>(resolution);
+        }
+        if (!overflow && (hashmapSize_ < 0 || requiredCells <= static_cast<size_t>(hashmapSize_))) {
+            layers_.push_back({static_cast<int>(total), resolution, 0, false});
+            total += static_cast<long long>(requiredCells) * num_features_per_level;
+            QuickMLP::Instance().getLogger()->debug("HashGrid layer %d is dense. Resolution=%d", l, resolution);
+        } else {
+            CHECK_ERROR(hashmapSize_ > 0, "HashGrid level ", l, " with resolution ", resolution,
+                        " is too large for a dense grid and no hash map size is configured");
+            layers_.push_back({static_cast<int>(total), resolution, hashmapSize_, true});
+            total += static_cast<long long>(hashmapSize_) * num_features_per_level;
+            QuickMLP::Instance().getLogger()->debug(
+                "HashGrid layer %d is sparse and will be hashed. Resolution=%d, hashmap size=%d", l, resolution,
+                hashmapSize_);
+        }
+        CHECK_ERROR(total < (1ll << 31), "The HashGrid needs more than 2^31 parameters, which the 32-bit offsets cannot address");
+    }
+    numParameters_ = static_cast<int>(total);
+}
+
+EncodingHashGrid::EncodingHashGrid(const json& cfg)
+    : EncodingHashGrid(cfg.at("start_in").get<int>(), cfg.at("n_in").get<int>(), cfg.at("n_levels").get<int>(),
+                       cfg.at("n_features_per_level").get<int>(), cfg.at("log2_hashmap_size").get<int>(),
+                       cfg.at("min_resolution").get<int>(), cfg.at("max_resolution").get<int>(),
+                       parseCombinationMode(cfg.at("combination_mode")),
+                       cfg.value("bounding_box_min", std::vector<float>()),
+                       cfg.value("bounding_box_size", std::vector<float>()), parsePrecision(cfg))
+{}
+
+json EncodingHashGrid::toJson() const
+{
+    return json::object({
+        {"id", id()},
+        {"start_in", startChannel_},
+        {"n_in", dimension_},
+        {"n_levels", numLevels_},
+        {"n_features_per_level", numFeaturesPerLevel_},
+        {"log2_hashmap_size", log2HashmapSize_},
+        {"min_resolution", minResolution_},
+        {"max_resolution", maxResolution_},
+        {"combination_mode", combinationMode_ == LayerCombinationMode::CONCAT ? "concat" : "add"},
+        {"bounding_box_min", json(boundingBoxMin_)},
+        {"bounding_box_size", json(boundingBoxSize_)},
+        {"parameter_precision", parameterPrecision_ == Tensor::HALF ? "half" : "float"},
+    });
+}
+
+std::string EncodingHashGrid::ID() { return "HashGrid"; }
+
+std::string EncodingHashGrid::id() const { return ID(); }
+
+int EncodingHashGrid::maxInputChannel() const { return startChannel_ + dimension_ - 1; }
+
+int EncodingHashGrid::numOutputChannels() const
+{
+    switch (combinationMode_) {
+    case LayerCombinationMode::CONCAT: return numLevels_ * numFeaturesPerLevel_;
+    case LayerCombinationMode::ADD: return numFeaturesPerLevel_;
+    default: throw std::runtime_error("Unknown enum");
+    }
+}
+
+std::string EncodingHashGrid::configName() const
+{
+    // the generated configuration struct is a pure function of these values
+    std::string key = format("%d_%d_%d_%d_%d_%d_%d_%d_%d", startChannel_, dimension_, numLevels_, numFeaturesPerLevel_,
+                             log2HashmapSize_, minResolution_, maxResolution_,
+                             static_cast<int>(combinationMode_), static_cast<int>(parameterPrecision_));
+    return "HashGridCfg_" + format("%zx", std::hash<std::string>()(key));
+}
+
+std::string EncodingHashGrid::qualifiedName() const
+{
+    return "qmlp::kernel::EncodingHashGrid<qmlp::kernel::" + configName() + ">";
+}
+
+void EncodingHashGrid::fillCode(std::stringstream& code) const
+{
+    const std::string name = configName();
+    code << KernelLoader::MainFile("qmlp/kernels/encoding_hashgrid.h");
+    code << "#ifndef QMLP_DEFINED_" << name << "\n#define QMLP_DEFINED_" << name << "\n";
+    code << "namespace qmlp { namespace kernel {\n";
+    code << "struct " << name << "\n{\n";
+    code << "    static constexpr int Start = " << startChannel_ << ";\n";
+    code << "    static constexpr int Dim = " << dimension_ << ";\n";
+    code << "    static constexpr int Levels = " << numLevels_ << ";\n";
+    code << "    static constexpr int Features = " << numFeaturesPerLevel_ << ";\n";
+    code << "    static constexpr bool Concat = "
+         << (combinationMode_ == LayerCombinationMode::CONCAT ? "true" : "false") << ";\n";
+    code << "    static constexpr bool ResolutionFactor = true;\n";
+    code << "    typedef " << (parameterPrecision_ == Tensor::HALF ? "f16" : "float") << " table_t;\n";
+    auto emit = [&](const char* type, const char* field, auto getter) {
+        code << "    static constexpr " << type << " " << field << "[" << numLevels_ << "] = {";
+        for (int l = 0; l < numLevels_; ++l) code << (l ? ", " : "") << getter(layers_[l]);
+        code << "};\n";
+    };
+    emit("int", "resolution", [](const HashGridLayerConfig& c) { return std::to_string(c.resolution); });
+    emit("int", "memoryOffset", [](const HashGridLayerConfig& c) { return std::to_string(c.memoryOffset); });
+    emit("unsigned", "hashGridSize",
+         [](const HashGridLayerConfig& c) { return std::to_string(c.hashed ? c.hashGridSize : 1) + "u"; });
+    emit("bool", "hashed", [](const HashGridLayerConfig& c) { return std::string(c.hashed ? "true" : "false"); });
+    code << "};\n}}\n#endif\n";
+}
+
+bool EncodingHashGrid::hasParameters() const { return true; }
+
+std::string EncodingHashGrid::parameterName() const
+{
+    return format("qmlp::kernel::HashGridParams<%s, %d>",
+                  parameterPrecision_ == Tensor::HALF ? "qmlp::kernel::f16" : "float", ndim());
+}
+
+Tensor::Precision EncodingHashGrid::parameterPrecision(Tensor::Usage usage) const
+{
+    return usage == Tensor::INFERENCE ? parameterPrecision_ : Tensor::FLOAT;
+}
+
+int EncodingHashGrid::parameterCount() const { return numParameters_; }
+
+void EncodingHashGrid::setParameter(const Tensor& tensor, Tensor::Usage usage)
+{
+    if (tensor.defined()) {
+        CHECK_DTYPE(tensor, parameterPrecision(usage));
+        CHECK_DIM(tensor, 1);
+        CHECK_SIZE(tensor, 0, parameterCount());
+        CHECK_ERROR(tensor.stride(0) == 1, "The grid parameters must be contiguous");
+        CHECK_ERROR(reinterpret_cast<uintptr_t>(tensor.rawPtr()) % 16 == 0,
+                    "The grid parameters must be aligned to 16 bytes");
+    }
+    if (usage == Tensor::INFERENCE)
+        parametersForward_ = tensor;
+    else
+        parametersGradients_ = tensor;
+}
+
+int EncodingHashGrid::fillParameterMemory(char* dst, int dstSize)
+{
+    // mirrors qmlp::kernel::HashGridParams<T, D>: two pointers, then 2*D floats
+    const int needed = static_cast<int>(2 * sizeof(void*) + 2 * dimension_ * sizeof(float));
+    CHECK_ERROR(dstSize >= needed, "parameter buffer too small");
+    const void* fwd = parametersForward_.defined() ? parametersForward_.rawPtr() : nullptr;
+    void* bwd = parametersGradients_.defined() ? parametersGradients_.rawPtr() : nullptr;
+    std::memcpy(dst, &fwd, sizeof(void*));
+    std::memcpy(dst + sizeof(void*), &bwd, sizeof(void*));
+    std::memcpy(dst + 2 * sizeof(void*), boundingBoxMin_.data(), dimension_ * sizeof(float));
+    std::memcpy(dst + 2 * sizeof(void*) + dimension_ * sizeof(float), boundingBoxInvSize_.data(),
+                dimension_ * sizeof(float));
+    return roundUp(needed, 8);
+}
+
+void EncodingHashGrid::zeroGradients()
+{
+    if (parametersGradients_.defined()) parametersGradients_.zero_();
+}
+
+QUICKMLP_NAMESPACE_END

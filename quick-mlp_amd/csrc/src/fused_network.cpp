@@ -1,0 +1,881 @@
+#include <qmlp/fused_network.h>
+
+#include <qmlp/encoding_identity.h>
+#include <qmlp/qmlp.h>
+
+#include "qmlp_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <sstream>
+#include <unordered_set>
+
+QUICKMLP_NAMESPACE_BEGIN
+
+namespace {
+constexpr int TILE_POINTS = 64;          // points per wavefront tile
+constexpr int DEFAULT_BLOCK_SIZE = 256;  // 4 wavefronts
+constexpr int STAGE_PAD = 8;             // halves of padding per staging row
+
+int gfx950LdsBytes() { return 160 * 1024; }
+} // namespace
+
+int FusedNetwork::MaxSharedMemoryBytes()
+{
+    static const int value = [] {
+        int count = 0;
+        qmlp_hip_device_count(&count);
+        if (count == 0) return gfx950LdsBytes();
+        qmlp_hip_device_props props;
+        QMLP_HIP_CALL(qmlp_hip_get_device_props(0, &props));
+        if (props.wave_size != FusedNetwork::WARP_SIZE)
+            throw configuration_error("The wavefront size of the device is %d, but the kernels are written for %d",
+                                      props.wave_size, FusedNetwork::WARP_SIZE);
+        QuickMLP::Instance().getLogger()->debug("LDS per workgroup on the current device in bytes: %d",
+                                                props.lds_bytes_per_block);
+        return props.lds_bytes_per_block;
+    }();
+    return value;
+}
+
+FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
+    : channelsIn_(cfg.at("num_inputs").get<int>())
+    , channelsOut_(cfg.at("num_outputs").get<int>())
+    , encodedChannels_(0)
+    , networkInputPadding_(0)
+    , numParameters_(0)
+    , perEntryForwardMemoryBytes_(0)
+    , adjointEvent_(nullptr)
+    , streamsCreated_(false)
+{
+    auto loader = QuickMLP::Instance().kernelLoader();
+    auto logger = QuickMLP::Instance().getLogger();
+
+    if (channelsIn_ <= 0) throw configuration_error("num_inputs must be positive, but is %d", channelsIn_);
+    if (channelsOut_ <= 0) throw configuration_error("num_outputs must be positive, but is %d", channelsOut_);
+
+    //compile options
+    if (cfg.contains("options")) {
+        const json& options = cfg.at("options");
+        compileOptions_.overwriteBlocksizeInference =
+            options.value("overwrite_blocksize_inference", compileOptions_.overwriteBlocksizeInference);
+        compileOptions_.overwriteBlocksizeForward =
+            options.value("overwrite_blocksize_forward", compileOptions_.overwriteBlocksizeForward);
+        compileOptions_.overwriteBlocksizeBackward =
+            options.value("overwrite_blocksize_backward", compileOptions_.overwriteBlocksizeBackward);
+        compileOptions_.overwriteBlocksizeWeightUpdate =
+            options.value("overwrite_blocksize_weight_update", compileOptions_.overwriteBlocksizeWeightUpdate);
+        compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
+        compileOptions_.parallelWeightUpdate =
+            options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
+    }
+
+    //activations
+    const json& activationSpecs = cfg.at("activation_specification");
+    auto activationFactory = ActivationFactory(activationSpecs, parent, loader);
+
+    //encodings
+    const json& encodingSpecs = cfg.at("encodings");
+    if (!encodingSpecs.is_array()) throw configuration_error("Illegal type for 'encodings', array expected");
+    for (const auto& ecfg : encodingSpecs) {
+        auto enc = EncodingFactory::Instance().create(ecfg);
+        if (enc->maxInputChannel() >= channelsIn_)
+            throw configuration_error("Input channels for encoding '%s' out of bounds (num channels=%d)",
+                                      enc->id().c_str(), channelsIn_);
+        encodedChannels_ += enc->numOutputChannels();
+        encodings_.push_back(enc);
+    }
+    if (encodings_.empty()) {
+        // no encoding given: the raw inputs are the network input
+        encodings_.push_back(std::make_shared<EncodingIdentity>(0, channelsIn_));
+        encodedChannels_ = channelsIn_;
+    }
+
+    //hidden layers
+    const json& networkSpecs = cfg.at("network");
+    if (!networkSpecs.is_array()) throw configuration_error("Expected a json-array for the network configuration");
+    if (networkSpecs.empty()) throw configuration_error("Empty network!");
+
+    // The first layer consumes the concatenated encoding outputs.
+    int prevInput = encodedChannels_;
+    for (const auto& e : networkSpecs) {
+        try {
+            LayerSpecification specs;
+            specs.channelsIn = prevInput;
+            specs.channelsOut = e.at("n_out").get<int>();
+            specs.useBias = e.at("bias").get<bool>();
+            specs.weightsStart = specs.biasStart = 0;
+            if (specs.channelsOut <= 0) throw configuration_error("n_out must be positive, but is %d", specs.channelsOut);
+
+            //either a single activation for all channels or one activation per channel
+            const json& ae = e.at("activation");
+            if (ae.is_string()) {
+                specs.activations.push_back(activationFactory.get(ae.get<std::string>()));
+            } else if (ae.is_array()) {
+                if (static_cast<int>(ae.size()) != specs.channelsOut)
+                    throw configuration_error(
+                        "If you specify individual activations per channel, then the number of activations (%d) must match the number of output channels (%d)",
+                        static_cast<int>(ae.size()), specs.channelsOut);
+                for (const auto& e2 : ae) {
+                    if (!e2.is_string()) throw configuration_error("Per-channel activations must be specified as a string");
+                    specs.activations.push_back(activationFactory.get(e2.get<std::string>()));
+                }
+            } else {
+                throw configuration_error("Unknown type for the activations, expected string or array");
+            }
+
+            prevInput = specs.channelsOut;
+            layers_.push_back(specs);
+        } catch (...) {
+            std::throw_with_nested(configuration_error("Parser error when processing network layer %d",
+                                                       static_cast<int>(layers_.size())));
+        }
+    }
+    if (channelsOut_ != prevInput)
+        throw configuration_error(
+            "The channel count of the last layer (%d) does not match the number of outputs specified at the top of the config file (%d)",
+            prevInput, channelsOut_);
+
+    //padding: every width becomes a multiple of the matrix size
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        const int currentIn = layers_[i].channelsIn;
+        const int paddedIn = roundUp(currentIn, MATRIX_SIZE);
+        if (currentIn == paddedIn) continue;
+        if (i == 0) {
+            networkInputPadding_ = paddedIn - currentIn;
+            layers_[i].channelsIn = paddedIn;
+            logger->warn("need to pad the network input channels from the encodings (%d channels)"
+                         " to the next multiple of the matrix size (%d). "
+                         "These extra channels are padded with zeros and are thus wasted. Consider increasing the input encoding.",
+                         currentIn, paddedIn);
+        } else {
+            layers_[i].channelsIn = paddedIn;
+            layers_[i - 1].channelsOut = paddedIn;
+            logger->warn("The hidden channels between layer %d and %d is currently specified to be "
+                         "%d channels wide. Matrix multiplications, however, are always performed in multiples of %d "
+                         "channels. The network has been automatically increased in size to fit %d channels. "
+                         "Consider updating the network specification to reflect this.",
+                         static_cast<int>(i) - 1, static_cast<int>(i), currentIn, MATRIX_SIZE, paddedIn);
+        }
+    }
+    {
+        const int currentOut = layers_.rbegin()->channelsOut;
+        const int paddedOut = roundUp(currentOut, MATRIX_SIZE);
+        if (currentOut != paddedOut) {
+            layers_.rbegin()->channelsOut = paddedOut;
+            logger->debug("the last layer's output (%d channels) is padded to %d channels", currentOut, paddedOut);
+        }
+    }
+
+    //prefix sum for the offsets of weight + bias: first all weights, then all biases
+    numParameters_ = 0;
+    for (auto& specs : layers_) {
+        specs.weightsStart = numParameters_;
+        numParameters_ += specs.channelsIn * specs.channelsOut;
+    }
+    for (auto& specs : layers_) {
+        if (specs.useBias) {
+            specs.biasStart = numParameters_;
+            numParameters_ += specs.channelsOut;
+        } else {
+            specs.biasStart = 0;
+        }
+    }
+
+    //tmp memory layout (channel prefixes; multiplied by the padded batch size at run time)
+    backwardInfo_.resize(layers_.size());
+    int offsetAdjOut = 0;
+    int offsetFwd = layers_[0].channelsIn;   // region 0 of the forward tmp memory: the encoded input
+    int offsetIn = 0;
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        backwardInfo_[i].offsetAdjOut = offsetAdjOut;
+        backwardInfo_[i].offsetIn = offsetIn;
+        backwardInfo_[i].offsetPre = offsetFwd;
+        offsetIn = offsetFwd;
+        offsetAdjOut += layers_[i].channelsOut;
+        offsetFwd += layers_[i].channelsOut;
+    }
+    perEntryForwardMemoryBytes_ = offsetFwd * static_cast<int>(sizeof(half));
+}
+
+FusedNetwork::~FusedNetwork()
+{
+    for (auto& info : backwardInfo_) {
+        if (info.stream) qmlp_hip_stream_destroy(info.stream);
+        if (info.event) qmlp_hip_event_destroy(info.event);
+    }
+    if (adjointEvent_) qmlp_hip_event_destroy(adjointEvent_);
+}
+
+void FusedNetwork::ensureStreams()
+{
+    if (streamsCreated_) return;
+    for (auto& info : backwardInfo_) {
+        qmlp_hip_stream s = nullptr;
+        qmlp_hip_event e = nullptr;
+        QMLP_HIP_CALL(qmlp_hip_stream_create(&s));
+        QMLP_HIP_CALL(qmlp_hip_event_create(&e, 0));
+        info.stream = static_cast<stream_t>(s);
+        info.event = static_cast<event_t>(e);
+    }
+    qmlp_hip_event e = nullptr;
+    QMLP_HIP_CALL(qmlp_hip_event_create(&e, 0));
+    adjointEvent_ = static_cast<event_t>(e);
+    streamsCreated_ = true;
+}
+
+IEncoding_ptr FusedNetwork::encoding(int idx)
+{
+    if (idx < 0 || idx >= static_cast<int>(encodings_.size())) throw std::runtime_error("Array index out of bounds");
+    return encodings_[idx];
+}
+
+int FusedNetwork::networkParameterCount() const { return numParameters_; }
+
+Tensor::Precision FusedNetwork::networkParameterPrecision(Tensor::Usage usage) const
+{
+    switch (usage) {
+    case Tensor::INFERENCE: return Tensor::HALF;
+    case Tensor::GRADIENTS: return Tensor::FLOAT;
+    default: throw std::runtime_error("Unknown usage");
+    }
+}
+
+void FusedNetwork::setNetworkParameter(const Tensor& tensor, Tensor::Usage usage)
+{
+    if (tensor.defined()) {
+        if (tensor.ndim() != 1 || tensor.sizes()[0] != numParameters_)
+            throw std::runtime_error(format("Illegal tensor shape, 1D tensor with %d entries required", numParameters_));
+        if (tensor.precision() != networkParameterPrecision(usage))
+            throw std::runtime_error("Wrong data type for the parameter. See parameterPrecision() for the expected format");
+        if (tensor.stride(0) != 1) throw std::runtime_error("The network parameters must be contiguous");
+        if (reinterpret_cast<uintptr_t>(tensor.rawPtr()) % 16 != 0)
+            throw std::runtime_error("The network parameters must be aligned to 16 bytes");
+    }
+    switch (usage) {
+    case Tensor::INFERENCE: parametersInference_ = tensor; break;
+    case Tensor::GRADIENTS: parametersGradients_ = tensor; break;
+    }
+}
+
+void FusedNetwork::initializeInferenceParameters(std::default_random_engine& rng)
+{
+    if (!parametersInference_.defined())
+        throw std::runtime_error("Inference parameters not defined, call setNetworkParameter(...) first");
+
+    std::vector<half> dataHost(static_cast<size_t>(parametersInference_.numel()), static_cast<half>(0));
+    for (int layer = 0; layer < numLayers(); ++layer) {
+        const auto& l = layers_[layer];
+        const float bound = 1.0f / std::sqrt(static_cast<float>(l.channelsIn));
+        std::uniform_real_distribution<float> distr1(-bound, +bound);
+        Tensor weights = networkParameter(layer, false, dataHost.data(), Tensor::HALF);
+        for (int32_t i = 0; i < weights.size(0); ++i)
+            for (int32_t j = 0; j < weights.size(1); ++j)
+                weights.dataPtr<half>()[weights.idx({i, j})] = static_cast<half>(distr1(rng));
+        if (l.useBias) {
+            Tensor bias = networkParameter(layer, true, dataHost.data(), Tensor::HALF);
+            for (int32_t i = 0; i < bias.size(0); ++i) bias.dataPtr<half>()[bias.idx({i})] = static_cast<half>(distr1(rng));
+        }
+    }
+    parametersInference_.copyFromHost(dataHost.data(), dataHost.size() * sizeof(half));
+}
+
+Tensor FusedNetwork::networkParameter(int layer, bool bias, void* rawPtr, Tensor::Precision precision)
+{
+    if (layer < 0 || layer >= static_cast<int>(layers_.size())) throw std::runtime_error("Layer index out of bounds");
+    const auto& l = layers_[layer];
+    int8_t* data = static_cast<int8_t*>(rawPtr);
+    const int bytesPerEntry = Tensor::BytesPerEntry[precision];
+    if (bias) {
+        if (!l.useBias) return {};
+        return Tensor(data + static_cast<ptrdiff_t>(bytesPerEntry) * l.biasStart, precision, {l.channelsOut}, {1});
+    }
+    //row-major
+    return Tensor(data + static_cast<ptrdiff_t>(bytesPerEntry) * l.weightsStart, precision,
+                  {l.channelsOut, l.channelsIn}, {l.channelsIn, 1});
+}
+
+Tensor FusedNetwork::networkParameter(int layer, bool bias, Tensor::Usage usage)
+{
+    auto& p = usage == Tensor::INFERENCE ? parametersInference_ : parametersGradients_;
+    return networkParameter(layer, bias, p.rawPtr(), p.precision());
+}
+
+// ------------------------------------------------------------------ code generation
+
+void FusedNetwork::fillEncodingsAndActivations(std::string& codeTemplate) const
+{
+    std::stringstream encodingIncludes;
+    std::stringstream encodingParameters;
+    for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
+        const auto& e = encodings_[encodingIdx];
+        e->fillCode(encodingIncludes);
+        encodingIncludes << "\n";
+        if (e->hasParameters())
+            encodingParameters << ",\n    const " << e->parameterName() << " cEncoding" << encodingIdx;
+    }
+    replaceAll(codeTemplate, "$$INCLUDES$$", encodingIncludes.str());
+    replaceAll(codeTemplate, "$$ENCODING_PARAMETERS$$", encodingParameters.str());
+
+    std::stringstream activationDefinitions;
+    std::unordered_set<std::string> activationIDs;
+    for (const auto& l : layers_)
+        for (const auto& a : l.activations)
+            if (activationIDs.insert(a->id()).second) activationDefinitions << a->code() << "\n";
+    replaceAll(codeTemplate, "$$DEFINE_ACTIVATIONS$$", activationDefinitions.str());
+
+    replaceAll(codeTemplate, "$$NUM_INPUTS$$", std::to_string(channelsIn_));
+    replaceAll(codeTemplate, "$$ENCODED_CHANNELS$$", std::to_string(encodedChannels_));
+    replaceAll(codeTemplate, "$$CHANNELS_IN$$", std::to_string(layers_.begin()->channelsIn));
+    replaceAll(codeTemplate, "$$CHANNELS_OUT$$", std::to_string(layers_.rbegin()->channelsOut));
+}
+
+int FusedNetwork::ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const
+{
+    // Weights sit in LDS in matrix-core operand order, contraction width padded to 32
+    // channels (forward: C_in, adjoint: C_out); the biases follow (forward only).
+    weightOffsets.assign(layers_.size(), 0);
+    biasOffsets.assign(layers_.size(), 0);
+    int n = 0;
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        const auto& l = layers_[i];
+        weightOffsets[i] = n;
+        n += adjoint ? l.channelsIn * roundUp(l.channelsOut, 32) : l.channelsOut * roundUp(l.channelsIn, 32);
+    }
+    if (!adjoint) {
+        for (size_t i = 0; i < layers_.size(); ++i) {
+            if (!layers_[i].useBias) continue;
+            biasOffsets[i] = n;
+            n += layers_[i].channelsOut;
+        }
+    }
+    return roundUp(n, 8);
+}
+
+int FusedNetwork::ldsParamHalves(bool adjoint) const
+{
+    std::vector<int> w, b;
+    return ldsLayout(adjoint, w, b);
+}
+
+int FusedNetwork::stageBytesPerWave() const
+{
+    return TILE_POINTS * (layers_[0].channelsIn + STAGE_PAD) * static_cast<int>(sizeof(half));
+}
+
+int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint) const
+{
+    int blockSize = DEFAULT_BLOCK_SIZE;
+    if (overwrite > 0) {
+        if (overwrite % WARP_SIZE != 0 || overwrite > 1024)
+            throw configuration_error("The block size must be a multiple of %d and at most 1024, but is %d", WARP_SIZE,
+                                      overwrite);
+        blockSize = overwrite;
+    }
+    const int maxLds = MaxSharedMemoryBytes();
+    const int paramBytes = ldsParamHalves(adjoint) * static_cast<int>(sizeof(half));
+    if (paramBytes + stageBytesPerWave() > maxLds)
+        throw configuration_error("The network is too large for the fused kernels: its %d parameters plus one staging "
+                                  "tile need %d bytes of LDS, the device offers %d",
+                                  numParameters_, paramBytes + stageBytesPerWave(), maxLds);
+    while (paramBytes + (blockSize / WARP_SIZE) * stageBytesPerWave() > maxLds) blockSize -= WARP_SIZE;
+    return blockSize;
+}
+
+static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
+{
+    std::stringstream ss;
+    for (size_t i = 0; i < layerTypes.size(); ++i) ss << "    typedef " << layerTypes[i] << " Layer" << i << ";\n";
+    return ss.str();
+}
+
+std::string FusedNetwork::forwardSource(int blockSize) const
+{
+    auto kl = QuickMLP::Instance().kernelLoader();
+    std::string code = kl->findFile("qmlp/kernels/network_forward.h").value();
+    fillEncodingsAndActivations(code);
+    replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
+    std::vector<int> ldsW, ldsB;
+    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(false, ldsW, ldsB)));
+
+    std::vector<std::string> layerTypes;
+    for (const auto& l : layers_) {
+        if (l.activations.size() > 1) throw std::runtime_error("Individual activations per channel are not implemented yet");
+        layerTypes.push_back(format("Layer<%d, %d, %s, activations::%s>", l.channelsIn, l.channelsOut,
+                                    l.useBias ? "true" : "false", l.activations[0]->id().c_str()));
+    }
+
+    std::stringstream stage;
+    stage << layerTypedefs(layerTypes);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        const auto& l = layers_[i];
+        stage << "    Layer" << i << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + "
+              << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
+        if (l.useBias)
+            stage << "    for (int i = threadIdx.x; i < " << l.channelsOut << "; i += blockDim.x) sParams["
+                  << ldsB[i] << " + i] = networkParameters[" << l.biasStart << " + i];\n";
+    }
+    replaceAll(code, "$$STAGE_PARAMETERS$$", stage.str());
+
+    std::stringstream callEncodings;
+    int encodingOffset = 0;
+    for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
+        const auto& e = encodings_[encodingIdx];
+        callEncodings << "                {\n                    auto encodingOutputK = encodingOutput + " << encodingOffset
+                      << ";\n                    " << e->qualifiedName() << "::forward(encodingInput, encodingOutputK";
+        if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
+        callEncodings << ");\n                }\n";
+        encodingOffset += e->numOutputChannels();
+    }
+    replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
+
+    std::stringstream callLayers;
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        const auto& l = layers_[i];
+        callLayers << "        f16x4 x" << (i + 1) << "[NT][Layer" << i << "::MT];\n";
+        callLayers << "        Layer" << i << "::template forward<STORE>(sParams + " << ldsW[i] << ", ";
+        if (l.useBias)
+            callLayers << "sParams + " << ldsB[i];
+        else
+            callLayers << "nullptr";
+        callLayers << ", x" << i << ", x" << (i + 1) << ",\n            STORE ? forwardTmpMemory + ("
+                   << backwardInfo_[i].offsetPre << "ll * numel64 + static_cast<long long>(tile) * ("
+                   << l.channelsOut << " * TILE_POINTS)) : nullptr, lane);\n";
+    }
+    callLayers << "        auto& xOut = x" << layers_.size() << ";\n";
+    replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
+    return code;
+}
+
+std::string FusedNetwork::backwardSource(int flags, int blockSize) const
+{
+    const bool hasInputGradients = flags & GRADIENTS_INPUT;
+    const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
+    const bool hasEncodingGradients = flags & GRADIENTS_INPUT_ENCODINGS;
+
+    auto kl = QuickMLP::Instance().kernelLoader();
+    std::string code = kl->findFile("qmlp/kernels/network_backward.h").value();
+    fillEncodingsAndActivations(code);
+    replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
+    replaceAll(code, "$$HAS_INPUT_GRADIENTS$$", hasInputGradients ? "true" : "false");
+    replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
+    replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
+    std::vector<int> ldsW, ldsB;
+    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(true, ldsW, ldsB)));
+
+    std::vector<std::string> layerTypes;
+    for (const auto& l : layers_) {
+        if (l.activations.size() > 1) throw std::runtime_error("Individual activations per channel are not implemented yet");
+        layerTypes.push_back(format("Layer<%d, %d, %s, activations::%s>", l.channelsIn, l.channelsOut,
+                                    l.useBias ? "true" : "false", l.activations[0]->id().c_str()));
+    }
+
+    // the first layer's transposed weights are only needed when something consumes dX0
+    const bool needsEncodingAdjoint = hasInputGradients || hasEncodingGradients;
+    std::stringstream stage;
+    stage << layerTypedefs(layerTypes);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        if (i == 0 && !needsEncodingAdjoint) continue;
+        const auto& l = layers_[i];
+        stage << "    Layer" << i << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + "
+              << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
+    }
+    replaceAll(code, "$$STAGE_PARAMETERS$$", stage.str());
+
+    std::stringstream callLayers;
+    const int L = static_cast<int>(layers_.size());
+    for (int i = L - 1; i >= 0; --i) {
+        const auto& l = layers_[i];
+        const std::string dy = (i == L - 1) ? std::string("dyOut") : "dx" + std::to_string(i + 1);
+        callLayers << "        f16x4 dx" << i << "[NT][Layer" << i << "::KT];\n";
+        callLayers << "        Layer" << i << "::template adjoint<HAS_NETWORK_GRADIENTS, "
+                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << ">(sParams + " << ldsW[i] << ", " << dy
+                   << ", dx" << i << ",\n            forwardTmpMemory + (" << backwardInfo_[i].offsetPre
+                   << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut << " * TILE_POINTS)),\n"
+                   << "            HAS_NETWORK_GRADIENTS ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut
+                   << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut
+                   << " * TILE_POINTS)) : nullptr,\n            validMask, lane);\n";
+    }
+    callLayers << "        auto& dxIn = dx0;\n        (void)dxIn;\n";
+    replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
+
+    std::stringstream callEncodings;
+    int encodingOffset = 0;
+    for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
+        const auto& e = encodings_[encodingIdx];
+        callEncodings << "                {\n                    auto adjEncodingOutputK = adjEncodingOutput + "
+                      << encodingOffset << ";\n                    " << e->qualifiedName() << "::template adjoint<"
+                      << (hasInputGradients ? "true" : "false") << ", "
+                      << ((hasEncodingGradients && e->hasParameters()) ? "true" : "false")
+                      << ">(encodingInput, adjEncodingOutputK, adjEncodingInput";
+        if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
+        callEncodings << ");\n                }\n";
+        encodingOffset += e->numOutputChannels();
+    }
+    replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
+    return code;
+}
+
+std::string FusedNetwork::weightUpdateSource(int blockSize) const
+{
+    auto kl = QuickMLP::Instance().kernelLoader();
+    std::string code = kl->findFile("qmlp/kernels/network_weight_update.h").value();
+    std::stringstream activationDefinitions;
+    std::unordered_set<std::string> activationIDs;
+    for (const auto& l : layers_)
+        for (const auto& a : l.activations)
+            if (activationIDs.insert(a->id()).second) activationDefinitions << a->code() << "\n";
+    replaceAll(code, "$$DEFINE_ACTIVATIONS$$", activationDefinitions.str());
+    replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
+    return code;
+}
+
+std::string FusedNetwork::weightUpdateKernelName(int layer, int& numChunks) const
+{
+    const auto& l = layers_[layer];
+    const int kt = l.channelsIn / MATRIX_SIZE, mt = l.channelsOut / MATRIX_SIZE;
+    // at most 16 accumulator tiles (64 VGPRs) per wave
+    int moChunk = 1;
+    for (int c = 1; c <= mt; ++c)
+        if (mt % c == 0 && c * kt <= 16) moChunk = c;
+    numChunks = mt / moChunk;
+    std::string inputActivation = "qmlp::kernel::activations::passthrough_";
+    if (layer > 0) {
+        const auto& prev = layers_[layer - 1].activations;
+        if (prev.size() > 1) throw std::runtime_error("Individual activations per channel are not implemented yet");
+        inputActivation = "qmlp::kernel::activations::" + prev[0]->id();
+    }
+    return format("qmlp::kernel::WeightUpdateKernel<%d, %d, %s, %s, %d>", l.channelsIn, l.channelsOut,
+                  l.useBias ? "true" : "false", inputActivation.c_str(), moChunk);
+}
+
+std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFlags)
+{
+    if (kind == "inference" || kind == "forward") return forwardSource(forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false));
+    if (kind == "backward") return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true));
+    if (kind == "weight_update") return weightUpdateSource(DEFAULT_BLOCK_SIZE);
+    throw std::runtime_error("unknown kernel kind '" + kind + "'");
+}
+
+// ------------------------------------------------------------------ compilation
+
+static int loaderFlags(bool compileOnly)
+{
+    int flags = QuickMLP::Instance().getCompileFlags();
+    if (compileOnly) flags |= KernelLoader::CompileOnly;
+    return flags;
+}
+
+void FusedNetwork::compileInferenceKernel(bool compileOnly)
+{
+    if (inferenceKernel_.has_value() && !compileOnly) return;
+    auto kl = QuickMLP::Instance().kernelLoader();
+    CompiledKernel ck;
+    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeInference, false);
+    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half)) + (ck.blockSize / WARP_SIZE) * stageBytesPerWave();
+    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<false>", forwardSource(ck.blockSize),
+                           loaderFlags(compileOnly)).value();
+    if (compileOnly) return;
+    ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
+    QuickMLP::Instance().getLogger()->debug("inference kernel: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
+                                            ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(), ck.fun.scratchBytes(), ck.fullGrid);
+    inferenceKernel_ = std::move(ck);
+}
+
+void FusedNetwork::compileForwardKernel(bool compileOnly)
+{
+    if (forwardKernel_.has_value() && !compileOnly) return;
+    auto kl = QuickMLP::Instance().kernelLoader();
+    CompiledKernel ck;
+    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false);
+    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half)) + (ck.blockSize / WARP_SIZE) * stageBytesPerWave();
+    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<true>", forwardSource(ck.blockSize),
+                           loaderFlags(compileOnly)).value();
+    if (compileOnly) return;
+    ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
+    QuickMLP::Instance().getLogger()->debug("forward kernel: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
+                                            ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(), ck.fun.scratchBytes(), ck.fullGrid);
+    forwardKernel_ = std::move(ck);
+}
+
+void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
+{
+    if (flags <= 0 || flags >= ADJOINT_MODE_MAX_COMBINATIONS) throw std::runtime_error("At least one derivative must be enabled");
+    if (backwardKernel_[flags].has_value() && !compileOnly) return;
+    const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
+    auto kl = QuickMLP::Instance().kernelLoader();
+    auto logger = QuickMLP::Instance().getLogger();
+
+    AdjointKernel ak;
+    ak.adjoint.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
+    ak.adjoint.sharedMemorySize =
+        ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (ak.adjoint.blockSize / WARP_SIZE) * stageBytesPerWave();
+    ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", backwardSource(flags, ak.adjoint.blockSize),
+                                   loaderFlags(compileOnly)).value();
+    if (!compileOnly) {
+        ak.adjoint.fullGrid = ak.adjoint.fun.fullGridSize(ak.adjoint.blockSize, ak.adjoint.sharedMemorySize);
+        logger->debug("backward kernel (flags %d): block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d", flags,
+                      ak.adjoint.blockSize, ak.adjoint.sharedMemorySize, ak.adjoint.fun.numVgprs(),
+                      ak.adjoint.fun.scratchBytes(), ak.adjoint.fullGrid);
+    }
+    int adjointChannels = 0;
+    for (const auto& l : layers_) adjointChannels += l.channelsOut;
+    ak.perEntryAdjointMemoryBytes = hasNetworkGradients ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
+
+    if (hasNetworkGradients) {
+        int blockSize = DEFAULT_BLOCK_SIZE;
+        if (compileOptions_.overwriteBlocksizeWeightUpdate > 0) {
+            blockSize = compileOptions_.overwriteBlocksizeWeightUpdate;
+            if (blockSize % WARP_SIZE != 0 || blockSize > 1024)
+                throw configuration_error("The block size must be a multiple of %d and at most 1024, but is %d", WARP_SIZE, blockSize);
+        }
+        const std::string source = weightUpdateSource(blockSize);
+        ak.layers.resize(layers_.size());
+        for (size_t layer = 0; layer < layers_.size(); ++layer) {
+            auto& wk = ak.layers[layer];
+            const std::string name = weightUpdateKernelName(static_cast<int>(layer), wk.numChunks);
+            const auto& l = layers_[layer];
+            const int moChunk = l.channelsOut / MATRIX_SIZE / wk.numChunks;
+            const int tiles = moChunk * (l.channelsIn / MATRIX_SIZE) + (l.useBias ? moChunk : 0);
+            wk.kernel.blockSize = blockSize;
+            wk.kernel.sharedMemorySize = tiles * 256 * static_cast<int>(sizeof(float));
+            if (wk.kernel.sharedMemorySize > MaxSharedMemoryBytes())
+                throw configuration_error("Layer %d too large for block-wise weight update!", static_cast<int>(layer));
+            wk.kernel.fun = kl->getKernel(name, source, loaderFlags(compileOnly)).value();
+            if (!compileOnly) {
+                wk.kernel.fullGrid = wk.kernel.fun.fullGridSize(blockSize, wk.kernel.sharedMemorySize);
+                logger->debug("weight update kernel layer %d: %s, LDS %d bytes, %d VGPRs, full grid %d",
+                              static_cast<int>(layer), name.c_str(), wk.kernel.sharedMemorySize,
+                              wk.kernel.fun.numVgprs(), wk.kernel.fullGrid);
+            }
+        }
+    }
+    if (!compileOnly) backwardKernel_[flags] = std::move(ak);
+}
+
+void FusedNetwork::precompile(int adjointFlags)
+{
+    compileInferenceKernel(true);
+    compileForwardKernel(true);
+    if (adjointFlags > 0) compileBackwardKernel(adjointFlags, true);
+}
+
+// ------------------------------------------------------------------ launches
+
+std::vector<char> FusedNetwork::encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage)
+{
+    storage.clear();
+    storage.reserve(encodings_.size());
+    for (auto& e : encodings_) {
+        if (!e->hasParameters()) continue;
+        storage.emplace_back(1024);
+        int n = e->fillParameterMemory(storage.back().data(), static_cast<int>(storage.back().size()));
+        (void)n;
+        args.push_back(storage.back().data());
+    }
+    return {};
+}
+
+void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t stream)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(output, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    CHECK_SIZE(output, 1, channelsOut());
+    int numel = input.size(0);
+    CHECK_SIZE(output, 0, numel);
+    CHECK_DTYPE(input, precisionIn());
+    CHECK_DTYPE(output, precisionOut());
+    CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
+    if (numel == 0) return;
+
+    compileInferenceKernel();
+    const auto& ck = inferenceKernel_.value();
+
+    const int waves = ck.blockSize / WARP_SIZE;
+    const int numTiles = divUp(numel, TILE_POINTS);
+    const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+    auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
+    const half* networkParams = parametersInference_.dataPtr<half>();
+    half* tmpMemory = nullptr;
+    std::vector<void*> args = {&numel, &inputAcc, &outputAcc, &networkParams, &tmpMemory};
+    std::vector<std::vector<char>> storage;
+    encodingArguments(args, storage);
+    ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+}
+
+size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlags)
+{
+    (void)adjointFlags;
+    numElements = roundUp(numElements, WARP_SIZE);
+    return static_cast<size_t>(perEntryForwardMemoryBytes_) * static_cast<size_t>(numElements);
+}
+
+size_t FusedNetwork::forwardMemory(const Tensor& input, AdjointModeFlags adjointFlags)
+{
+    CHECK_DIM(input, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    return forwardMemory(input.size(0), adjointFlags);
+}
+
+void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory, stream_t stream)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(output, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    CHECK_SIZE(output, 1, channelsOut());
+    int numel = input.size(0);
+    CHECK_SIZE(output, 0, numel);
+    CHECK_DTYPE(input, precisionIn());
+    CHECK_DTYPE(output, precisionOut());
+    CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
+    if (numel == 0) return;
+    CHECK_ERROR(tmpMemory != nullptr, "forward() needs temporary memory of forwardMemory() bytes");
+    CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemory) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
+
+    compileForwardKernel();
+    const auto& ck = forwardKernel_.value();
+
+    const int waves = ck.blockSize / WARP_SIZE;
+    const int numTiles = divUp(numel, TILE_POINTS);
+    const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+    auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
+    const half* networkParams = parametersInference_.dataPtr<half>();
+    half* tmpMemoryHalf = static_cast<half*>(tmpMemory);
+    std::vector<void*> args = {&numel, &inputAcc, &outputAcc, &networkParams, &tmpMemoryHalf};
+    std::vector<std::vector<char>> storage;
+    encodingArguments(args, storage);
+    ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+}
+
+void FusedNetwork::zeroGradients()
+{
+    if (parametersGradients_.defined()) parametersGradients_.zero_();
+    for (auto& e : encodings_) e->zeroGradients();
+}
+
+size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlags)
+{
+    if (adjointFlags <= 0 || adjointFlags >= ADJOINT_MODE_MAX_COMBINATIONS)
+        throw std::runtime_error("At least one derivative must be enabled");
+    int adjointChannels = 0;
+    for (const auto& l : layers_) adjointChannels += l.channelsOut;
+    const int perEntry = (adjointFlags & GRADIENTS_NETWORK_WEIGHTS) ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
+    numElements = roundUp(numElements, WARP_SIZE);
+    return static_cast<size_t>(perEntry) * static_cast<size_t>(numElements);
+}
+
+size_t FusedNetwork::adjointMemory(const Tensor& input, AdjointModeFlags adjointFlags)
+{
+    CHECK_DIM(input, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    return adjointMemory(input.size(0), adjointFlags);
+}
+
+void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, AdjointModeFlags adjointFlags,
+                           Tensor& adjInput, const void* tmpMemoryForward, void* tmpMemoryAdjoint, stream_t stream)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(adjOutput, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    CHECK_SIZE(adjOutput, 1, channelsOut());
+    int numel = input.size(0);
+    CHECK_SIZE(adjOutput, 0, numel);
+    CHECK_DTYPE(input, precisionIn());
+    CHECK_DTYPE(adjOutput, precisionOut());
+    if (adjointFlags <= 0 || adjointFlags >= ADJOINT_MODE_MAX_COMBINATIONS)
+        throw std::runtime_error("At least one derivative must be enabled");
+
+    const bool hasInputGradients = adjointFlags & GRADIENTS_INPUT;
+    const bool hasNetworkGradients = adjointFlags & GRADIENTS_NETWORK_WEIGHTS;
+    const bool hasEncodingGradients = adjointFlags & GRADIENTS_INPUT_ENCODINGS;
+
+    if (hasInputGradients) {
+        CHECK_ERROR(adjInput.defined(), "Input gradients requested, but adjInput is undefined");
+        CHECK_DIM(adjInput, 2);
+        CHECK_SIZE(adjInput, 1, channelsIn());
+        CHECK_SIZE(adjInput, 0, numel);
+        CHECK_DTYPE(adjInput, precisionIn());
+    }
+    if (hasNetworkGradients)
+        CHECK_ERROR(parametersGradients_.defined(),
+                    "Network gradients requested, but no gradient tensor was set via setNetworkParameter(..., GRADIENTS)");
+    CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
+    if (numel == 0) return;
+    CHECK_ERROR(tmpMemoryForward != nullptr, "adjoint() needs the temporary memory written by forward()");
+    if (hasNetworkGradients) {
+        CHECK_ERROR(tmpMemoryAdjoint != nullptr, "adjoint() needs temporary memory of adjointMemory() bytes");
+        CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemoryAdjoint) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
+    }
+    (void)hasEncodingGradients;
+
+    compileBackwardKernel(adjointFlags);
+    auto& ak = backwardKernel_[adjointFlags].value();
+
+    const int numTiles = divUp(numel, TILE_POINTS);
+    const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
+    {
+        const auto& ck = ak.adjoint;
+        const int waves = ck.blockSize / WARP_SIZE;
+        const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+        auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+        auto adjOutputAcc = adjOutput.accessor<kernel::Tensor2Read<float>>();
+        kernel::Tensor2RW<float> adjInputAcc;
+        std::memset(&adjInputAcc, 0, sizeof(adjInputAcc));
+        if (hasInputGradients) adjInputAcc = adjInput.accessor<kernel::Tensor2RW<float>>();
+        const half* networkParams = parametersInference_.dataPtr<half>();
+        const half* forwardTmpMemory = static_cast<const half*>(tmpMemoryForward);
+        half* adjointTmpMemory = static_cast<half*>(tmpMemoryAdjoint);
+        std::vector<void*> args = {&numel, &inputAcc, &adjOutputAcc, &adjInputAcc, &networkParams,
+                                   &forwardTmpMemory, &adjointTmpMemory};
+        std::vector<std::vector<char>> storage;
+        encodingArguments(args, storage);
+        ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+    }
+
+    if (!hasNetworkGradients) return;
+
+    const bool parallel = compileOptions_.parallelWeightUpdate && layers_.size() > 1;
+    if (parallel) {
+        ensureStreams();
+        QMLP_HIP_CALL(qmlp_hip_event_record(adjointEvent_, stream));
+    }
+    for (size_t layer = 0; layer < layers_.size(); ++layer) {
+        const auto& ls = layers_[layer];
+        const auto& ali = backwardInfo_[layer];
+        const auto& wk = ak.layers[layer];
+
+        float* gradBase = parametersGradients_.dataPtr<float>();
+        float* outAdjWeights = gradBase + ls.weightsStart;
+        float* outAdjBias = ls.useBias ? gradBase + ls.biasStart : nullptr;
+        const half* aIn = static_cast<const half*>(tmpMemoryAdjoint) + static_cast<ptrdiff_t>(ali.offsetAdjOut) * numel64;
+        const half* bIn = static_cast<const half*>(tmpMemoryForward) + static_cast<ptrdiff_t>(ali.offsetIn) * numel64;
+
+        stream_t layerStream = stream;
+        if (parallel) {
+            layerStream = ali.stream;
+            QMLP_HIP_CALL(qmlp_hip_stream_wait_event(ali.stream, adjointEvent_));
+        }
+        const int waves = wk.kernel.blockSize / WARP_SIZE;
+        const int slices = std::max(1, std::min(divUp(numTiles, waves), std::max(1, wk.kernel.fullGrid / wk.numChunks)));
+        int numTilesArg = numTiles;
+        void* args[] = {&numTilesArg, &outAdjWeights, &outAdjBias, &aIn, &bIn};
+        wk.kernel.fun.launch(slices * wk.numChunks, wk.kernel.blockSize, wk.kernel.sharedMemorySize, layerStream, args);
+        if (parallel) {
+            QMLP_HIP_CALL(qmlp_hip_event_record(ali.event, ali.stream));
+            QMLP_HIP_CALL(qmlp_hip_stream_wait_event(stream, ali.event));
+        }
+    }
+}
+
+void FusedNetwork::clearCachedKernels()
+{
+    inferenceKernel_ = {};
+    forwardKernel_ = {};
+    for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i) backwardKernel_[i] = {};
+}
+
+QUICKMLP_NAMESPACE_END

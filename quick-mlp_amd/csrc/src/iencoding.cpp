@@ -1,0 +1,181 @@
+#include <qmlp/iencoding.h>
+
+#include <qmlp/encoding_hashgrid.h>
+#include <qmlp/encoding_identity.h>
+#include <qmlp/qmlp.h>
+
+#include <cstring>
+
+QUICKMLP_NAMESPACE_BEGIN
+
+namespace {
+
+// Kernel arguments of the standalone kernels: fixed ones plus the optional parameter struct.
+struct ArgPack
+{
+    std::vector<void*> ptrs;
+    std::vector<char> paramBytes;
+};
+
+std::string standaloneSource(const IEncoding& e, const std::string& callForward, const std::string& callAdjoint,
+                             const std::string& callCorners = "")
+{
+    auto kl = QuickMLP::Instance().kernelLoader();
+    std::string codeTemplate = kl->findFile("qmlp/kernels/encoding_kernels.h").value();
+    std::stringstream includes;
+    e.fillCode(includes);
+    includes << "\n";
+    replaceAll(codeTemplate, "$$INCLUDES$$", includes.str());
+    replaceAll(codeTemplate, "$$ENCODING_PARAMETERS$$",
+               e.hasParameters() ? ", const " + e.parameterName() + " cEncoding" : std::string());
+    replaceAll(codeTemplate, "$$CALL_ENCODINGS_FORWARD$$", callForward);
+    replaceAll(codeTemplate, "$$CALL_ENCODINGS_ADJOINT$$", callAdjoint);
+    replaceAll(codeTemplate, "$$CALL_ENCODINGS_CORNERS$$", callCorners);
+    return codeTemplate;
+}
+
+} // namespace
+
+void IEncoding::forward(const Tensor& input, Tensor& output, stream_t stream,
+                        const std::optional<const Tensor>& parametersForward)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(output, 2);
+    CHECK_DTYPE(input, Tensor::FLOAT);
+    CHECK_DTYPE(output, Tensor::FLOAT);
+    CHECK_SIZE(output, 0, input.size(0));
+    CHECK_ERROR(input.size(1) > maxInputChannel());
+    CHECK_ERROR(output.size(1) >= numOutputChannels());
+    CHECK_ERROR(output.strides()[1] == 1, "The output stride along the channels must be 1");
+    long long numel = input.size(0);
+    if (numel == 0) return;
+
+    if (!forwardKernel_.has_value()) {
+        std::stringstream call;
+        call << qualifiedName() << "::forward(encodingInput, encodingOutput";
+        if (hasParameters()) call << ", cEncoding";
+        call << ");\n";
+        std::string source = standaloneSource(*this, call.str(), "");
+        forwardKernel_ = QuickMLP::Instance().kernelLoader()->getKernel(
+            "qmlp::kernel::EncodingForwardKernel", source, QuickMLP::Instance().getCompileFlags()).value();
+    }
+    auto& fun = forwardKernel_.value();
+
+    std::vector<char> paramBytes(4096);
+    if (hasParameters()) {
+        if (parametersForward.has_value()) setParameter(parametersForward.value(), Tensor::INFERENCE);
+        int n = fillParameterMemory(paramBytes.data(), static_cast<int>(paramBytes.size()));
+        (void)n;
+    }
+
+    const int block = 256;
+    const int grid = static_cast<int>(std::min<long long>(divUp<long long>(numel, block), fun.fullGridSize(block, 0)));
+    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+    auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
+    std::vector<void*> args = {&numel, &inputAcc, &outputAcc};
+    if (hasParameters()) args.push_back(paramBytes.data());
+    fun.launch(grid, block, 0, stream, args.data());
+
+    if (hasParameters() && parametersForward.has_value()) setParameter({}, Tensor::INFERENCE);
+}
+
+void IEncoding::adjoint(const Tensor& input, const Tensor& adjOutput, Tensor& adjInput, stream_t stream,
+                        const std::optional<const Tensor>& parametersForward,
+                        const std::optional<const Tensor>& parametersGradients, int adjointMode)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(adjOutput, 2);
+    CHECK_DIM(adjInput, 2);
+    CHECK_DTYPE(input, Tensor::FLOAT);
+    CHECK_DTYPE(adjOutput, Tensor::FLOAT);
+    CHECK_DTYPE(adjInput, Tensor::FLOAT);
+    CHECK_SIZE(adjOutput, 0, input.size(0));
+    CHECK_SIZE(adjInput, 0, input.size(0));
+    CHECK_ERROR(input.size(1) > maxInputChannel());
+    CHECK_ERROR(adjOutput.size(1) >= numOutputChannels());
+    CHECK_ERROR(adjInput.size(1) == input.size(1));
+    CHECK_ERROR(adjointMode >= 1 && adjointMode <= ALL_GRADIENTS, "Illegal adjoint mode");
+    long long numel = input.size(0);
+    if (numel == 0) return;
+
+    if (!adjointKernel_[adjointMode].has_value()) {
+        const bool hasInputGradients = adjointMode & INPUT_GRADIENTS;
+        const bool hasParamGradients = (adjointMode & PARAM_GRADIENTS) && hasParameters();
+        std::stringstream call;
+        call << qualifiedName() << "::template adjoint<" << (hasInputGradients ? "true" : "false") << ", "
+             << (hasParamGradients ? "true" : "false") << ">(encodingInput, encodingAdjOutput, encodingAdjInput";
+        if (hasParameters()) call << ", cEncoding";
+        call << ");\n";
+        std::string source = standaloneSource(*this, "", call.str());
+        adjointKernel_[adjointMode] = QuickMLP::Instance().kernelLoader()->getKernel(
+            "qmlp::kernel::EncodingAdjointKernel", source, QuickMLP::Instance().getCompileFlags()).value();
+    }
+    auto& fun = adjointKernel_[adjointMode].value();
+
+    std::vector<char> paramBytes(4096);
+    if (hasParameters()) {
+        if (parametersForward.has_value()) setParameter(parametersForward.value(), Tensor::INFERENCE);
+        if (parametersGradients.has_value()) setParameter(parametersGradients.value(), Tensor::GRADIENTS);
+        int n = fillParameterMemory(paramBytes.data(), static_cast<int>(paramBytes.size()));
+        (void)n;
+    }
+
+    const int block = 256;
+    const int grid = static_cast<int>(std::min<long long>(divUp<long long>(numel, block), fun.fullGridSize(block, 0)));
+    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+    auto adjOutputAcc = adjOutput.accessor<kernel::Tensor2Read<float>>();
+    auto adjInputAcc = adjInput.accessor<kernel::Tensor2RW<float>>();
+    std::vector<void*> args = {&numel, &inputAcc, &adjOutputAcc, &adjInputAcc};
+    if (hasParameters()) args.push_back(paramBytes.data());
+    fun.launch(grid, block, 0, stream, args.data());
+
+    if (hasParameters() && parametersForward.has_value()) setParameter({}, Tensor::INFERENCE);
+    if (hasParameters() && parametersGradients.has_value()) setParameter({}, Tensor::GRADIENTS);
+}
+
+void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* weights, stream_t stream)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DTYPE(input, Tensor::FLOAT);
+    CHECK_ERROR(input.size(1) > maxInputChannel());
+    long long numel = input.size(0);
+    if (numel == 0) return;
+    if (!cornersKernel_.has_value()) {
+        std::string call = qualifiedName() + "::corners(encodingInput, cEncoding, cornerIndices, cornerWeights);\n";
+        std::string source = standaloneSource(*this, "", "", call);
+        cornersKernel_ = QuickMLP::Instance().kernelLoader()->getKernel(
+            "qmlp::kernel::EncodingCornersKernel", source, QuickMLP::Instance().getCompileFlags()).value();
+    }
+    auto& fun = cornersKernel_.value();
+    std::vector<char> paramBytes(4096);
+    int n = fillParameterMemory(paramBytes.data(), static_cast<int>(paramBytes.size()));
+    (void)n;
+    const int block = 256;
+    const int grid = static_cast<int>(std::min<long long>(divUp<long long>(numel, block), fun.fullGridSize(block, 0)));
+    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+    int perPoint = numLevels() * (1 << ndim());
+    void* args[] = {&numel, &inputAcc, &indices, &weights, &perPoint, paramBytes.data()};
+    fun.launch(grid, block, 0, stream, args);
+}
+
+EncodingFactory::EncodingFactory()
+{
+    encodings_[EncodingIdentity::ID()] = [](const json& cfg) { return std::make_shared<EncodingIdentity>(cfg); };
+    encodings_[EncodingHashGrid::ID()] = [](const json& cfg) { return std::make_shared<EncodingHashGrid>(cfg); };
+}
+
+EncodingFactory& EncodingFactory::Instance()
+{
+    static EncodingFactory INSTANCE;
+    return INSTANCE;
+}
+
+IEncoding_ptr EncodingFactory::create(const json& cfg)
+{
+    const std::string id = cfg.at("id").get<std::string>();
+    auto it = encodings_.find(id);
+    if (it == encodings_.end()) throw configuration_error("No encoding with id '%s' found", id.c_str());
+    return it->second(cfg);
+}
+
+QUICKMLP_NAMESPACE_END
