@@ -1,0 +1,236 @@
+"""CPU-only tests of the host side: the C ABI library loads and exports what the headers
+declare, the specification layer follows the reference's rules (validated against the
+oracle's restatement and the golden level table), and the code generator's output compiles
+for gfx950 through hipRTC without a GPU."""
+import ctypes
+import json
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import qmlp
+import qmlp_oracle as qo
+from qmlp import baseline_configs as bc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qmlp_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.mark.parametrize("header", ["qmlp_hip.h", "qmlp_capi.h"])
+def test_library_exports_every_declared_symbol(header):
+    lib = ctypes.CDLL(qmlp._lib.LIB_PATH)
+    names = _declared_functions(header)
+    assert len(names) > 20
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_static_queries_without_gpu():
+    assert qmlp.Network.MatrixSize() == 16
+    assert qmlp.Network.WarpSize() == 64
+    assert qmlp.Network.MaxSharedMemoryBytes() >= 64 * 1024
+    assert qmlp.QuickMLP.is_compile_debug_mode() is False
+
+
+@pytest.mark.parametrize("cfg_id", [1, 2, 3, 4, 5])
+def test_parameter_layout_matches_the_oracle(cfg_id):
+    cfg = bc.CONFIGS[cfg_id]["cfg"]
+    net = qmlp.Network(json.dumps(cfg))
+    onet = qo.Network(cfg, bc.ORACLE_ACTIVATIONS)
+    assert net.num_network_parameters() == onet.num_parameters
+    assert net.channels_in() == cfg["num_inputs"] and net.channels_out() == cfg["num_outputs"]
+    assert net.num_layers() == len(cfg["network"])
+    layers, n = bc.padded_layout(cfg)
+    assert n == onet.num_parameters
+    import torch
+    flat = torch.zeros(n, dtype=torch.float16)
+    for i, l in enumerate(onet.layers):
+        w = net.parameter_view(i, False, flat)
+        assert tuple(w.shape) == (l["cout"], l["cin"]) and w.stride() == (l["cin"], 1)
+        assert (w.data_ptr() - flat.data_ptr()) // 2 == l["w_start"]
+        b = net.parameter_view(i, True, flat)
+        if l["bias"]:
+            assert tuple(b.shape) == (l["cout"],)
+            assert (b.data_ptr() - flat.data_ptr()) // 2 == l["b_start"]
+        else:
+            assert b is None
+    assert {1: 512, 2: 7168, 3: 7168, 4: 14336, 5: 3184}[cfg_id] == n
+
+
+def test_level_table_matches_golden_and_oracle():
+    gold = json.load(open(os.path.join(GOLDEN, "cfg2_level_table.json")))
+    enc = qmlp.Encoding(json.dumps(gold["spec"]))
+    got = [[r, int(h), off] for (r, h, off, _) in enc.hashgrid_levels()]
+    assert got == gold["levels"]
+    assert enc.num_parameters() == gold["total_parameters"]
+    for spec in [bc.densegrid4d("float"),
+                 dict(bc.hashgrid3d("float"), n_in=2, bounding_box_min=[0, 0], bounding_box_size=[1, 1],
+                      n_levels=5, n_features_per_level=4, log2_hashmap_size=-1, max_resolution=2048),
+                 dict(bc.hashgrid3d("float"), n_levels=7, log2_hashmap_size=12, min_resolution=3, max_resolution=300)]:
+        e = qmlp.Encoding(json.dumps(spec))
+        g = qo.HashGrid(spec)
+        assert e.hashgrid_levels() == g.level_table()
+        assert e.num_parameters() == g.n_params
+        assert e.num_output_channels() == g.num_outputs
+
+
+def test_encoding_json_round_trip_and_defaults():
+    spec = {"id": "HashGrid", "start_in": 1, "n_in": 2, "n_levels": 2, "n_features_per_level": 4,
+            "log2_hashmap_size": 8, "min_resolution": 4, "max_resolution": 64, "combination_mode": "add"}
+    e = qmlp.Encoding(json.dumps(spec))
+    j = json.loads(e.to_json())
+    assert j["bounding_box_min"] == [-0.5, -0.5] and j["bounding_box_size"] == [1.0, 1.0]
+    assert j["combination_mode"] == "add" and j["parameter_precision"] == "float"
+    assert e.max_input_channel() == 2 and e.num_output_channels() == 4 and e.has_parameters()
+    e2 = qmlp.Encoding(e.to_json())
+    assert json.loads(e2.to_json()) == j
+    cat = qmlp.Encoding(json.dumps(dict(spec, combination_mode="cat")))
+    assert cat.num_output_channels() == 8
+    ident = qmlp.Encoding('{"id": "Identity", "start_in": 2, "n_in": 3}')
+    assert ident.max_input_channel() == 4 and ident.num_output_channels() == 3 and not ident.has_parameters()
+
+
+BASE = bc.CONFIGS[1]["cfg"]
+
+
+@pytest.mark.parametrize("mutate,code,message", [
+    (lambda c: c.update(num_outputs=2), 1, "does not match the number of outputs"),
+    (lambda c: c.update(network=[]), 1, "Empty network"),
+    (lambda c: c["encodings"][0].update(id="identity"), 1, "No encoding with id 'identity'"),
+    (lambda c: c["encodings"][0].update(n_in=4), 1, "out of bounds"),
+    (lambda c: c["network"][0].update(activation="gelu"), 1, "No activation with id 'gelu'"),
+    (lambda c: c["network"][0].update(activation=["relu"] * 3), 1, "must match the number of output channels"),
+    (lambda c: c.pop("num_inputs"), 1, "num_inputs"),
+    (lambda c: c.update(activation_specification=["does-not-exist.json"]), 1, "could not be resolved"),
+    (lambda c: c.update(activation_specification=[{"id": "1bad", "forward": "z=x", "adjoint": "adjx=adjz"}]), 1,
+     "not a valid C.. identifier"),
+])
+def test_specification_errors(mutate, code, message):
+    cfg = json.loads(json.dumps(BASE))
+    mutate(cfg)
+    with pytest.raises(qmlp.QmlpError, match=message) as ei:
+        qmlp.Network(json.dumps(cfg))
+    assert ei.value.code == code
+
+
+def test_malformed_json_and_grid_errors():
+    with pytest.raises(qmlp.QmlpError, match="JSON parse error"):
+        qmlp.Network('{"num_inputs": 3,')
+    bad = dict(bc.hashgrid3d("float"), n_in=7, bounding_box_min=[0] * 7, bounding_box_size=[1] * 7)
+    with pytest.raises(qmlp.QmlpError, match=r"to be in \[1,6\]"):
+        qmlp.Encoding(json.dumps(bad))
+    with pytest.raises(qmlp.QmlpError, match="combination_mode"):
+        qmlp.Encoding(json.dumps(dict(bc.hashgrid3d("float"), combination_mode="multiply")))
+    with pytest.raises(qmlp.QmlpError, match="Unknown log level"):
+        qmlp.set_log_level("chatty")
+
+
+def test_temporary_memory_sizes():
+    net = qmlp.Network(json.dumps(bc.CONFIGS[3]["cfg"]))
+    per_fwd = 2 * (32 + 64 + 64 + 16)
+    per_adj = 2 * (64 + 64 + 16)
+    for n, padded in ((1, 64), (64, 64), (65, 128), (1 << 18, 1 << 18)):
+        assert net.forward_memory(n, 7) == per_fwd * padded
+        assert net.adjoint_memory(n, 7) == per_adj * padded
+        assert net.adjoint_memory(n, 1) == 0
+    with pytest.raises(qmlp.QmlpError, match="At least one derivative"):
+        net.adjoint_memory(10, 0)
+
+
+def test_generated_source_is_specialised():
+    net = qmlp.Network(json.dumps(bc.CONFIGS[2]["cfg"]))
+    src = net.generated_source("forward")
+    assert "Layer<32, 64, false, activations::relu>" in src
+    assert "Layer<64, 16, false, activations::identity>" in src
+    assert "static constexpr int resolution[16] = {16, 23, 33, 48, 70, 101, 147, 212, 307, 445, 645, 933, 1351, 1955, 2830, 4095};" in src
+    assert "typedef f16 table_t;" in src and not re.search(r"\$\$[A-Z_]+\$\$", src)
+    bsrc = net.generated_source("backward", 7)
+    assert "stageAdjoint" in bsrc and not re.search(r"\$\$[A-Z_]+\$\$", bsrc)
+    wsrc = net.generated_source("weight_update")
+    assert "WeightUpdateKernel" in wsrc and not re.search(r"\$\$[A-Z_]+\$\$", wsrc)
+
+
+def test_kernels_compile_for_gfx950_without_a_gpu_and_are_cached(tmp_path):
+    """hipRTC needs no device: generate + compile every kernel of a small fused network, then
+    a second network object finds all of them in the disk cache."""
+    cache = str(tmp_path / "cache")
+    qmlp.set_kernel_cache_dir(cache)
+    try:
+        grid = dict(bc.hashgrid3d("half"), n_levels=3, log2_hashmap_size=8, max_resolution=64)
+        cfg = {"num_inputs": 4, "num_outputs": 3, "activation_specification": [bc.BUILTIN, bc.SINE30],
+               "encodings": [grid, {"id": "Identity", "start_in": 3, "n_in": 1}],
+               "network": [{"n_out": 48, "bias": True, "activation": "sine30"},
+                           {"n_out": 3, "bias": False, "activation": "celu"}]}
+        c0, h0 = qmlp._lib.kernel_cache_stats()
+        qmlp.Network(json.dumps(cfg)).precompile(7)
+        c1, h1 = qmlp._lib.kernel_cache_stats()
+        assert c1 - c0 == 5 and h1 == h0          # inference, forward, backward, 2 weight updates
+        files = os.listdir(cache)
+        assert len(files) == 5 and all(f.endswith(".co") for f in files)
+        qmlp.Network(json.dumps(cfg)).precompile(7)
+        c2, h2 = qmlp._lib.kernel_cache_stats()
+        assert c2 == c1                            # nothing recompiled (memory or disk cache)
+    finally:
+        qmlp.set_kernel_cache_dir(os.environ.get("QMLP_CACHE_DIR", qmlp._lib.DEFAULT_CACHE_DIR))
+
+
+def test_compile_errors_carry_the_compiler_log(tmp_path):
+    qmlp.set_kernel_cache_dir("")
+    try:
+        cfg = json.loads(json.dumps(BASE))
+        cfg["activation_specification"] = [bc.BUILTIN, {"id": "broken", "forward": "z = not_a_function(x)", "adjoint": "adjx = adjz"}]
+        cfg["network"][0]["activation"] = "broken"
+        net = qmlp.Network(json.dumps(cfg))
+        qmlp.set_log_level("off")
+        with pytest.raises(qmlp.QmlpError, match="not_a_function") as ei:
+            net.precompile(0)
+        assert ei.value.code == 3
+    finally:
+        qmlp.set_log_level("warn")
+        qmlp.set_kernel_cache_dir(os.environ.get("QMLP_CACHE_DIR", qmlp._lib.DEFAULT_CACHE_DIR))
+
+
+def test_network_too_large_for_lds_is_rejected():
+    cfg = json.loads(json.dumps(BASE))
+    cfg["network"] = [{"n_out": 256, "bias": False, "activation": "relu"}] * 3 + [{"n_out": 1, "bias": False, "activation": "relu"}]
+    cfg["num_outputs"] = 1
+    net = qmlp.Network(json.dumps(cfg))
+    with pytest.raises(qmlp.QmlpError, match="too large for the fused kernels"):
+        net.precompile(0)
+
+
+def test_simulated_network_and_weight_copy_shapes():
+    import torch
+    cfg = json.dumps({"num_inputs": 5, "num_outputs": 3, "activation_specification": [bc.BUILTIN],
+                      "encodings": [{"id": "Identity", "start_in": 0, "n_in": 5}],
+                      "network": [{"n_out": 20, "bias": True, "activation": "celu"},
+                                  {"n_out": 3, "bias": False, "activation": "identity"}]})
+    sim = qmlp.SimulatedNetwork(cfg, weight_dtype=torch.float32)
+    y = sim(torch.rand(7, 5))
+    assert y.shape == (7, 3) and sim.num_layers() == 2 and sim.has_bias(0) and not sim.has_bias(1)
+    with pytest.raises(ValueError):
+        qmlp.SimulatedNetwork(json.dumps(bc.CONFIGS[2]["cfg"]))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_activation_objects():
+    a = qmlp.Activation("relu")
+    assert json.loads(a.to_json())["id"] == "relu"
+    b = qmlp.Activation(json.dumps(bc.SINE30))
+    assert json.loads(b.to_json())["forward"] == bc.SINE30["forward"]
+    with pytest.raises(qmlp.QmlpError, match="No activation with id"):
+        qmlp.Activation("swish")
