@@ -45,6 +45,10 @@ public:
         int overwriteBlocksizeBackward = -1;
         int overwriteBlocksizeWeightUpdate = -1;
 
+        //Tiles of 64 points that one wavefront of the inference / forward kernel encodes
+        //together (level by level for grid encodings). If <=0, the library chooses.
+        int pointsPerLane = -1;
+
         // Accepted for compatibility; the LDS layouts of this implementation are
         // bank-conflict free for 64 lanes by construction and need no skew.
         bool skewSharedMemory = false;
@@ -86,6 +90,7 @@ private:
     {
         KernelFunction fun;
         int blockSize = 0;
+        int pointsPerLane = 1;
         int sharedMemorySize = 0;
         int fullGrid = 0;
     };
@@ -113,6 +118,7 @@ private:
     {
         CompiledKernel adjoint;
         std::vector<WeightUpdateKernel> layers;
+        CompiledKernel reduce;
         int perEntryAdjointMemoryBytes = 0;
     };
     std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS];
@@ -226,12 +232,15 @@ private:
     void compileForwardKernel(bool compileOnly = false);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 
-    std::string forwardSource(int blockSize) const;
+    std::string forwardSource(int blockSize, int pointsPerLane) const;
     std::string backwardSource(int flags, int blockSize) const;
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks) const;
     void fillEncodingsAndActivations(std::string& codeTemplate) const;
-    int forwardBlockSize(int overwrite, bool adjoint) const;
+    int forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane = nullptr) const;
+    int weightUpdateBlockSize() const;
+    // number of batch slices whose partial weight gradients are kept in the adjoint memory
+    int weightUpdateSlices(int numTiles) const;
     int ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const;
     int ldsParamHalves(bool adjoint) const;
     int stageBytesPerWave() const;

@@ -77,6 +77,24 @@ __device__ __forceinline__ void loadFeatures(const T* __restrict__ p, float (&v)
     }
 }
 
+/** Loads two consecutive table entries (2*F values) with one wide load; the address is
+ *  only guaranteed to be aligned to one entry. */
+template <int F, typename T>
+__device__ __forceinline__ void loadPair(const T* __restrict__ p, float (&a)[F], float (&b)[F])
+{
+    constexpr int ENTRY_BYTES = F * static_cast<int>(sizeof(T));
+    constexpr int ALIGN = ENTRY_BYTES >= 16 ? 16 : ENTRY_BYTES >= 8 ? 8 : ENTRY_BYTES >= 4 ? 4 : static_cast<int>(sizeof(T));
+    typedef T pair_t __attribute__((ext_vector_type(2 * F), aligned(ALIGN)));
+    const pair_t t = *reinterpret_cast<const pair_t*>(p);
+#pragma unroll
+    for (int i = 0; i < F; ++i) {
+        a[i] = static_cast<float>(t[i]);
+        b[i] = static_cast<float>(t[F + i]);
+    }
+}
+
+__device__ __forceinline__ constexpr bool isPow2(unsigned v) { return v != 0u && (v & (v - 1u)) == 0u; }
+
 } // namespace detail
 
 /**
@@ -159,6 +177,138 @@ struct EncodingHashGrid
 #pragma unroll
         for (int d = D - 1; d >= 0; --d) a = a * (((c >> d) & 1) ? s.f[d] : (1.f - s.f[d]));
         return a;
+    }
+
+    /**
+     * Interpolated features of one level at one point. The 2^D corners are fetched as
+     * 2^(D-1) pairs: per lane-load the memory pipeline handles one address regardless of the
+     * width, so one wider load per pair of neighbouring entries halves the number of loads.
+     *  - dense level: neighbours along the last (fastest) coordinate are adjacent entries;
+     *  - hashed level with a power-of-two table: the multiplier of coordinate 0 is 1, so its
+     *    two corners are entries idx and idx^1 of one aligned pair whenever the lower
+     *    coordinate is even (or clamped); only otherwise a second, lane-masked load is needed.
+     * Values and weights are the same as in the corner-by-corner evaluation, only the order
+     * of the fp32 additions differs.
+     */
+    __device__ __forceinline__ static void gatherLevel(int l, const float (&pos)[D],
+                                                       const table_t* __restrict__ table, float (&feat)[F])
+    {
+        const LevelSetup s = setupLevel(l, pos);
+        const int R = Cfg::resolution[l];
+        const bool hashed = Cfg::hashed[l];
+        const unsigned base = static_cast<unsigned>(Cfg::memoryOffset[l]);
+#pragma unroll
+        for (int i = 0; i < F; ++i) feat[i] = 0.f;
+
+        if (!hashed && R >= 2) {
+            // pairs along dimension D-1: entries (zb, zb+1) with zb = min(iL, R-2)
+            constexpr int PD = D - 1;
+            const unsigned zL = s.termL[PD], zH = s.termH[PD];   // multiplier of the last dim is 1
+            const unsigned zb = min(zL, static_cast<unsigned>(R - 2));
+            const bool lSecond = zL != zb, hSecond = zH != zb;
+            const float wzL = 1.f - s.f[PD], wzH = s.f[PD];
+#pragma unroll
+            for (int c = 0; c < NC / 2; ++c) {
+                unsigned idx = zb;
+                float w = 1.f;
+#pragma unroll
+                for (int d = PD - 1; d >= 0; --d) {
+                    const bool hi = (c >> d) & 1;
+                    idx += hi ? s.termH[d] : s.termL[d];
+                    w = w * (hi ? s.f[d] : (1.f - s.f[d]));
+                }
+                float e0[F], e1[F];
+                detail::loadPair<F>(table + (base + idx * static_cast<unsigned>(F)), e0, e1);
+#pragma unroll
+                for (int i = 0; i < F; ++i) {
+                    const float vL = lSecond ? e1[i] : e0[i];
+                    const float vH = hSecond ? e1[i] : e0[i];
+                    feat[i] += w * (wzL * vL + wzH * vH);
+                }
+            }
+        } else if (hashed && detail::isPow2(Cfg::hashGridSize[l]) && Cfg::hashGridSize[l] >= 2u) {
+            const unsigned mask = Cfg::hashGridSize[l] - 1u;
+            const float wxL = 1.f - s.f[0], wxH = s.f[0];
+#pragma unroll
+            for (int c = 0; c < NC / 2; ++c) {
+                unsigned rest = 0u;
+                float w = 1.f;
+#pragma unroll
+                for (int d = D - 1; d >= 1; --d) {
+                    const bool hi = (c >> (d - 1)) & 1;
+                    rest ^= hi ? s.termH[d] : s.termL[d];
+                    w = w * (hi ? s.f[d] : (1.f - s.f[d]));
+                }
+                const unsigned idxL = (s.termL[0] ^ rest) & mask;
+                const unsigned idxH = (s.termH[0] ^ rest) & mask;
+                float e0[F], e1[F];
+                detail::loadPair<F>(table + (base + (idxL & ~1u) * static_cast<unsigned>(F)), e0, e1);
+                float vH[F];
+                const bool samePair = ((idxL ^ idxH) & ~1u) == 0u;
+                if (!samePair) {
+                    detail::loadFeatures<F>(table + (base + idxH * static_cast<unsigned>(F)), vH);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < F; ++i) vH[i] = (idxH & 1u) ? e1[i] : e0[i];
+                }
+#pragma unroll
+                for (int i = 0; i < F; ++i) {
+                    const float vL = (idxL & 1u) ? e1[i] : e0[i];
+                    feat[i] += w * (wxL * vL + wxH * vH[i]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const float w = cornerWeight(s, c);
+                float v[F];
+                detail::loadFeatures<F>(table + cornerOffset(l, s, c), v);
+#pragma unroll
+                for (int i = 0; i < F; ++i) feat[i] += w * v[i];
+            }
+        }
+    }
+
+    /**
+     * Level-major evaluation of PPL points of one lane: all points finish level l before
+     * any starts level l+1, so that the workgroups of the device sweep through the level
+     * tables together and a level's table stays in L2 while it is in use.
+     */
+    template <int PPL, typename I, typename O>
+    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], O (&outputs)[PPL],
+                                                        const param_t& params)
+    {
+        typedef typename O::ValueType O_t;
+        float pos[PPL][D];
+#pragma unroll
+        for (int q = 0; q < PPL; ++q) unitPosition(inputs[q], params, pos[q]);
+        float sum[PPL][F];
+#pragma unroll
+        for (int q = 0; q < PPL; ++q)
+#pragma unroll
+            for (int i = 0; i < F; ++i) sum[q][i] = 0.f;
+#pragma unroll
+        for (int l = 0; l < L; ++l) {
+            float feat[PPL][F];
+#pragma unroll
+            for (int q = 0; q < PPL; ++q) gatherLevel(l, pos[q], params.parametersForward, feat[q]);
+#pragma unroll
+            for (int q = 0; q < PPL; ++q) {
+                if constexpr (Cfg::Concat) {
+#pragma unroll
+                    for (int i = 0; i < F; ++i) outputs[q][l * F + i] = fcast<O_t>(feat[q][i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < F; ++i) sum[q][i] += feat[q][i];
+                }
+            }
+        }
+        if constexpr (!Cfg::Concat) {
+#pragma unroll
+            for (int q = 0; q < PPL; ++q)
+#pragma unroll
+                for (int i = 0; i < F; ++i) outputs[q][i] = fcast<O_t>(sum[q][i]);
+        }
     }
 
     /**
@@ -261,6 +411,112 @@ struct EncodingHashGrid
 #pragma unroll
             for (int d = 0; d < D; ++d)
                 adjInput[d + Cfg::Start] += adjPos[d] * params.boundingBoxInvSize[d];
+        }
+    }
+
+    /** True if the gradient scatter of a whole tile (scatterTile) is available. */
+    static constexpr bool HasTileScatter = detail::isPow2(static_cast<unsigned>(F)) && 2 * F <= WAVE_SIZE;
+
+    /**
+     * Parameter gradients of the 64 points of one wavefront tile. The atomic units handle
+     * one request per group of lanes of an instruction that address contiguous memory, and
+     * their rate is bound by requests, not by lanes. Therefore 2*F neighbouring lanes share
+     * one point and add the 2*F contiguous values of a pair of neighbouring entries (the
+     * same pairs as in gatherLevel) in one request; the wavefront covers its 64 points in
+     * 2*F rounds of 64/(2F) points. Every lane recomputes the level setup of its point; the
+     * arithmetic is free next to the atomics.
+     *
+     * \param index0 index of the first point of the tile
+     * \param adjRows the wave's staging rows with the adjoint of the encoded input; the row of
+     *    point p of the tile is adjRows + stageRow(p) * rowStride, this encoding's channels
+     *    start at channelOffset
+     */
+    __device__ __forceinline__ static void scatterTile(int lane, int index0, int numel,
+                                                       const Tensor2Read<float>& inputs, const f16* adjRows,
+                                                       int rowStride, int channelOffset, const param_t& params)
+    {
+        constexpr int G = 2 * F;            // lanes per point
+        constexpr int PPR = WAVE_SIZE / G;  // points per round
+        const int sub = lane % G;
+        const int k = sub / F;              // position within the pair of entries
+        const int i = sub % F;              // feature
+        float* __restrict__ grad = params.parametersBackward;
+#pragma unroll 1
+        for (int round = 0; round < G; ++round) {
+            const int pt = round * PPR + lane / G;
+            const int index = index0 + pt;
+            if (index >= numel) continue;
+            float in[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                in[d] = inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
+                                     + static_cast<long long>(d + Cfg::Start) * inputs.strides_[1]];
+            float pos[D];
+            {
+#pragma clang fp contract(off)
+#pragma unroll
+                for (int d = 0; d < D; ++d) pos[d] = (in[d] - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
+            }
+            const f16* adjRow = adjRows + stageRow(pt) * rowStride + channelOffset;
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                const LevelSetup s = setupLevel(l, pos);
+                const int R = Cfg::resolution[l];
+                const bool hashed = Cfg::hashed[l];
+                const unsigned base = static_cast<unsigned>(Cfg::memoryOffset[l]);
+                const float adj = static_cast<float>(adjRow[(Cfg::Concat ? l * F : 0) + i]);
+                if (!hashed && R >= 2) {
+                    constexpr int PD = D - 1;
+                    const unsigned zL = s.termL[PD], zH = s.termH[PD];
+                    const unsigned zb = min(zL, static_cast<unsigned>(R - 2));
+                    const unsigned zk = zb + static_cast<unsigned>(k);
+                    const float wz = (zL == zk ? 1.f - s.f[PD] : 0.f) + (zH == zk ? s.f[PD] : 0.f);
+#pragma unroll
+                    for (int c = 0; c < NC / 2; ++c) {
+                        unsigned idx = zb;
+                        float w = 1.f;
+#pragma unroll
+                        for (int d = PD - 1; d >= 0; --d) {
+                            const bool hi = (c >> d) & 1;
+                            idx += hi ? s.termH[d] : s.termL[d];
+                            w = w * (hi ? s.f[d] : (1.f - s.f[d]));
+                        }
+                        unsafeAtomicAdd(grad + (base + idx * static_cast<unsigned>(F) + static_cast<unsigned>(sub)),
+                                        (w * wz) * adj);
+                    }
+                } else if (hashed && detail::isPow2(Cfg::hashGridSize[l]) && Cfg::hashGridSize[l] >= 2u) {
+                    const unsigned mask = Cfg::hashGridSize[l] - 1u;
+                    const float wxL = 1.f - s.f[0], wxH = s.f[0];
+#pragma unroll
+                    for (int c = 0; c < NC / 2; ++c) {
+                        unsigned rest = 0u;
+                        float w = 1.f;
+#pragma unroll
+                        for (int d = D - 1; d >= 1; --d) {
+                            const bool hi = (c >> (d - 1)) & 1;
+                            rest ^= hi ? s.termH[d] : s.termL[d];
+                            w = w * (hi ? s.f[d] : (1.f - s.f[d]));
+                        }
+                        const unsigned idxL = (s.termL[0] ^ rest) & mask;
+                        const unsigned idxH = (s.termH[0] ^ rest) & mask;
+                        const bool samePair = ((idxL ^ idxH) & ~1u) == 0u;
+                        const unsigned uk = static_cast<unsigned>(k);
+                        const float wx = ((idxL & 1u) == uk ? wxL : 0.f) + ((samePair && (idxH & 1u) == uk) ? wxH : 0.f);
+                        unsafeAtomicAdd(grad + (base + (idxL & ~1u) * static_cast<unsigned>(F) + static_cast<unsigned>(sub)),
+                                        (w * wx) * adj);
+                        if (!samePair && (idxH & 1u) == uk)
+                            unsafeAtomicAdd(grad + (base + idxH * static_cast<unsigned>(F) + static_cast<unsigned>(i)),
+                                            (w * wxH) * adj);
+                    }
+                } else {
+                    // corner by corner; the lanes of the lower half of the group add the F features
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) {
+                        if (k == 0)
+                            unsafeAtomicAdd(grad + (cornerOffset(l, s, c) + static_cast<unsigned>(i)), cornerWeight(s, c) * adj);
+                    }
+                }
+            }
         }
     }
 

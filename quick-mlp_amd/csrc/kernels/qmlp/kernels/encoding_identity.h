@@ -20,6 +20,13 @@ struct EncodingIdentity
         for (int i = 0; i < NumChannels; ++i) output[i] = fcast<O_t>(input[i + StartChannel]);
     }
 
+    template <int PPL, typename I, typename O>
+    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], O (&outputs)[PPL])
+    {
+#pragma unroll
+        for (int q = 0; q < PPL; ++q) forward(inputs[q], outputs[q]);
+    }
+
     template <bool EvaluateInputGradients, bool EvaluateParameterGradients, typename I, typename O, typename AdjI>
     __device__ __forceinline__ static void adjoint(const I& input, const O& adjOutput, AdjI& adjInput)
     {

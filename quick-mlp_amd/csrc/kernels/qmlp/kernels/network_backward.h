@@ -128,6 +128,9 @@ $$CALL_ENCODINGS$$
                                         + static_cast<long long>(i) * adjInputs.strides_[1]] += adjEncodingInput[i];
                 }
             }
+
+            // parameter gradients of the grid encodings, scattered by the whole wavefront
+$$CALL_ENCODING_SCATTER$$
             waveLdsSync();
         }
     }

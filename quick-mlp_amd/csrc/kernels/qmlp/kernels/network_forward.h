@@ -1,10 +1,12 @@
 // Template of the fused forward / inference kernel. The host code generator replaces
 // everything in $$..$$ before the source is handed to the runtime compiler.
 //
-// One wavefront owns a tile of 64 points: each lane first evaluates all input
-// encodings of one point into a row of the wave's LDS staging area (fp16), then the
-// wave reads the rows back as matrix-core B operands and runs every layer with the
-// activations kept in registers. Weights (and biases) are staged into LDS once per
+// One wavefront owns groups of PPL tiles of 64 points: each lane first evaluates all
+// input encodings of one point of every tile into rows of the wave's LDS staging area
+// (fp16; the grid encodings go level by level over the PPL points, which keeps many
+// gathers in flight and lets all waves of the device sweep the level tables together),
+// then the wave reads the rows of one tile after the other back as matrix-core B
+// operands and runs every layer with the activations kept in registers. Weights (and biases) are staged into LDS once per
 // workgroup, already permuted into operand order.
 //
 // Replaces NetworkKernelInferenceAndForward of the reference
@@ -46,6 +48,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     constexpr int STAGE_STRIDE = CHANNELS_IN + 8;         // halves; odd multiple of 16 bytes
     constexpr int LDS_PARAM_HALVES = $$LDS_PARAM_HALVES$$;
     constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
+    constexpr int PPL = $$POINTS_PER_LANE$$;              // tiles a wave encodes together
 
     const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
     f16* __restrict__ forwardTmpMemory = reinterpret_cast<f16*>(forwardTmpMemoryH);
@@ -55,7 +58,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     const int wave = threadIdx.x / WAVE_SIZE;
     const int lane = threadIdx.x % WAVE_SIZE;
     const int g = lane >> 4, r = lane & 15;
-    f16* sStage = sParams + LDS_PARAM_HALVES + wave * (TILE_POINTS * STAGE_STRIDE);
+    f16* sStage = sParams + LDS_PARAM_HALVES + wave * (PPL * TILE_POINTS * STAGE_STRIDE);
 
     // stage the weights in operand order, then the biases
 $$STAGE_PARAMETERS$$
@@ -64,31 +67,45 @@ $$STAGE_PARAMETERS$$
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
     (void)numel64;
-    for (int tile = blockIdx.x * WAVES + wave; tile < numTiles; tile += gridDim.x * WAVES)
+    for (int tile0 = (blockIdx.x * WAVES + wave) * PPL; tile0 < numTiles; tile0 += gridDim.x * WAVES * PPL)
     {
-        const int index = tile * TILE_POINTS + lane;
-        const bool valid = index < numel;
-
-        // encodings: one point per lane into its staging row
+        // encodings: PPL points per lane (one of each tile), each into its staging row.
+        // Rows outside the batch are evaluated at the origin and zeroed afterwards so that
+        // no NaN enters the matrix cores.
         {
-            f16* rowPtr = sStage + stageRow(lane) * STAGE_STRIDE;
-            WrappedArray<f16> encodingOutput{rowPtr};
-            if (valid) {
-                StaticArray<float, NUM_INPUTS> encodingInput;
+            StaticArray<float, NUM_INPUTS> encodingInput[PPL];
+            WrappedArray<f16> encodingOutput[PPL];
+            bool valid[PPL];
+#pragma unroll
+            for (int q = 0; q < PPL; ++q) {
+                const int index = (tile0 + q) * TILE_POINTS + lane;
+                valid[q] = index < numel;
+                encodingOutput[q].data_ = sStage + (q * TILE_POINTS + stageRow(lane)) * STAGE_STRIDE;
 #pragma unroll
                 for (int i = 0; i < NUM_INPUTS; ++i)
-                    encodingInput[i] = inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
-                                                    + static_cast<long long>(i) * inputs.strides_[1]];
+                    encodingInput[q][i] = valid[q] ? inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
+                                                                  + static_cast<long long>(i) * inputs.strides_[1]]
+                                                   : 0.f;
+            }
 $$CALL_ENCODINGS$$
 #pragma unroll
-                for (int c = ENCODED_CHANNELS; c < CHANNELS_IN; ++c) rowPtr[c] = static_cast<f16>(0);
-            } else {
-                // rows outside the batch are zero so that no NaN enters the matrix cores
+            for (int q = 0; q < PPL; ++q) {
 #pragma unroll
-                for (int c = 0; c < CHANNELS_IN; ++c) rowPtr[c] = static_cast<f16>(0);
+                for (int c = ENCODED_CHANNELS; c < CHANNELS_IN; ++c) encodingOutput[q][c] = static_cast<f16>(0);
+                if (!valid[q]) {
+#pragma unroll
+                    for (int c = 0; c < ENCODED_CHANNELS; ++c) encodingOutput[q][c] = static_cast<f16>(0);
+                }
             }
         }
         waveLdsSync();
+
+#pragma unroll 1
+        for (int q = 0; q < PPL; ++q)
+        {
+        const int tile = tile0 + q;
+        if (tile >= numTiles) break;
+        const f16* sTile = sStage + q * (TILE_POINTS * STAGE_STRIDE);
 
         // B operands of the first layer
         f16x4 x0[NT][KT0];
@@ -96,8 +113,7 @@ $$CALL_ENCODINGS$$
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int t = 0; t < KT0; ++t)
-                x0[nt][t] = *reinterpret_cast<const f16x4*>(sStage + (16 * nt + r) * STAGE_STRIDE + 16 * t + 4 * g);
-        waveLdsSync();   // the staging rows may be overwritten by the next tile
+                x0[nt][t] = *reinterpret_cast<const f16x4*>(sTile + (16 * nt + r) * STAGE_STRIDE + 16 * t + 4 * g);
 
         if constexpr (STORE) {
             // encoded input, channel-major per tile, for the weight update of layer 0
@@ -132,6 +148,8 @@ $$CALL_NETWORK_LAYERS$$
                     }
                 }
             }
+        }
+        waveLdsSync();   // the staging rows are overwritten by the next group of tiles
     }
 }
 

@@ -8,8 +8,11 @@
 // channel per lane = one 16-byte load in operand layout); in_l is the activation of
 // the previous layer re-applied on the fly, or the stored encoded input for layer 0.
 // Many workgroups reduce disjoint slices of the batch; each wave accumulates in fp32
-// registers, waves of a workgroup are combined through LDS, workgroups through
-// hardware fp32 atomics.
+// registers, the waves of a workgroup are combined through LDS and the workgroup stores
+// its partial sums (slice-major) without atomics: thousands of atomic additions onto the
+// same few cache lines serialise in the memory system and took ten times longer than
+// the reduction itself. WeightUpdateReduceKernel then adds the partial sums of all slices
+// to the gradient tensor, in a fixed order, so the result is reproducible bit by bit.
 //
 // Replaces WeightUpdateSingleBlockKernel of the reference
 // (src_cpp/include/qmlp/kernels/network_weight_update_block.cuh:356-494), which runs
@@ -40,8 +43,9 @@ $$DEFINE_ACTIVATIONS$$
 template <int CIN, int COUT, bool BIAS, typename InputActivation, int MO_CHUNK>
 __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
     int numTiles,                     // 64-point tiles in the batch
-    float* __restrict__ gradWeights,  // (COUT, CIN) row-major, accumulated
-    float* __restrict__ gradBias,     // (COUT) or nullptr
+    float* __restrict__ partialWeights,  // slice 0 of this layer's (COUT, CIN) row-major partial sums
+    float* __restrict__ partialBias,     // slice 0 of this layer's (COUT) partial sums, or nullptr
+    int sliceStride,                     // distance between the slices in floats
     const half* __restrict__ adjPreH, // dpre tiles of this layer: (numTiles, COUT, 64)
     const half* __restrict__ inputH)  // input tiles of this layer: (numTiles, CIN, 64)
 {
@@ -94,7 +98,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
         }
     }
 
-    // combine the waves of the workgroup through LDS, then one atomic per entry
+    // combine the waves of the workgroup through LDS, then store the slice's partial sums
     extern __shared__ __align__(16) unsigned char sMemory[];
     float* sAcc = reinterpret_cast<float*>(sMemory);   // (MO_CHUNK*KT + MO_CHUNK) tiles of 256 floats
     constexpr int TILES = MO_CHUNK * KT + (BIAS ? MO_CHUNK : 0);
@@ -120,13 +124,47 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
         const int t = e >> 8, within = e & 255;
         const int mo = t / KT, mi = t - mo * KT;
         const int row = 16 * (mo0 + mo) + (within >> 4), col = 16 * mi + (within & 15);
-        unsafeAtomicAdd(gradWeights + row * CIN + col, sAcc[e]);
+        partialWeights[static_cast<long long>(slice) * sliceStride + row * CIN + col] = sAcc[e];
     }
     if constexpr (BIAS) {
         for (int e = threadIdx.x; e < MO_CHUNK * 16; e += blockDim.x) {
             const int mo = e >> 4;
-            unsafeAtomicAdd(gradBias + 16 * (mo0 + mo) + (e & 15), sAcc[(MO_CHUNK * KT + mo) * 256 + (e & 15)]);
+            partialBias[static_cast<long long>(slice) * sliceStride + 16 * (mo0 + mo) + (e & 15)]
+                = sAcc[(MO_CHUNK * KT + mo) * 256 + (e & 15)];
         }
+    }
+}
+
+/**
+ * gradients[i] += sum over the slices of partial[slice * count + i]. One workgroup of
+ * 1024 threads per 64 parameters: 16 wavefronts each sum every 16th slice, LDS combines them.
+ */
+__global__ void __launch_bounds__(1024) WeightUpdateReduceKernel(
+    int count, int numSlices, const float* __restrict__ partial, float* __restrict__ gradients)
+{
+    __shared__ float sSum[16][WAVE_SIZE];
+    const int lane = threadIdx.x % WAVE_SIZE;
+    const int group = threadIdx.x / WAVE_SIZE;
+    const int i = blockIdx.x * WAVE_SIZE + lane;
+    float sum = 0.f;
+    if (i < count) {
+        int s = group;
+        for (; s + 7 * 16 < numSlices; s += 8 * 16) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[static_cast<long long>(s + 16 * u) * count + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += v[u];
+        }
+        for (; s < numSlices; s += 16) sum += partial[static_cast<long long>(s) * count + i];
+    }
+    sSum[group][lane] = sum;
+    __syncthreads();
+    if (group == 0 && i < count) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) total += sSum[w][lane];
+        gradients[i] += total;
     }
 }
 

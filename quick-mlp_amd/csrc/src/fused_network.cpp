@@ -16,6 +16,7 @@ QUICKMLP_NAMESPACE_BEGIN
 namespace {
 constexpr int TILE_POINTS = 64;          // points per wavefront tile
 constexpr int DEFAULT_BLOCK_SIZE = 256;  // 4 wavefronts
+constexpr int MAX_WEIGHT_UPDATE_SLICES = 512;  // batch slices with partial weight gradients
 constexpr int STAGE_PAD = 8;             // halves of padding per staging row
 
 int gfx950LdsBytes() { return 160 * 1024; }
@@ -66,6 +67,9 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
             options.value("overwrite_blocksize_backward", compileOptions_.overwriteBlocksizeBackward);
         compileOptions_.overwriteBlocksizeWeightUpdate =
             options.value("overwrite_blocksize_weight_update", compileOptions_.overwriteBlocksizeWeightUpdate);
+        compileOptions_.pointsPerLane = options.value("points_per_lane", compileOptions_.pointsPerLane);
+        if (compileOptions_.pointsPerLane > 8)
+            throw configuration_error("points_per_lane must be at most 8, but is %d", compileOptions_.pointsPerLane);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
             options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
@@ -364,7 +368,7 @@ int FusedNetwork::stageBytesPerWave() const
     return TILE_POINTS * (layers_[0].channelsIn + STAGE_PAD) * static_cast<int>(sizeof(half));
 }
 
-int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint) const
+int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane) const
 {
     int blockSize = DEFAULT_BLOCK_SIZE;
     if (overwrite > 0) {
@@ -380,7 +384,34 @@ int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint) const
                                   "tile need %d bytes of LDS, the device offers %d",
                                   numParameters_, paramBytes + stageBytesPerWave(), maxLds);
     while (paramBytes + (blockSize / WARP_SIZE) * stageBytesPerWave() > maxLds) blockSize -= WARP_SIZE;
+    if (pointsPerLane) {
+        // Grid encodings gather level by level over several points per lane; two workgroups
+        // should still fit on a compute unit.
+        bool gathers = false;
+        for (const auto& e : encodings_) gathers = gathers || e->hasParameters();
+        int ppl = compileOptions_.pointsPerLane > 0 ? compileOptions_.pointsPerLane : (gathers ? 2 : 1);
+        const int budget = compileOptions_.pointsPerLane > 0 ? maxLds : maxLds / 2;
+        while (ppl > 1 && paramBytes + (blockSize / WARP_SIZE) * ppl * stageBytesPerWave() > budget) --ppl;
+        *pointsPerLane = ppl;
+    }
     return blockSize;
+}
+
+int FusedNetwork::weightUpdateBlockSize() const
+{
+    int blockSize = DEFAULT_BLOCK_SIZE;
+    if (compileOptions_.overwriteBlocksizeWeightUpdate > 0) {
+        blockSize = compileOptions_.overwriteBlocksizeWeightUpdate;
+        if (blockSize % WARP_SIZE != 0 || blockSize > 1024)
+            throw configuration_error("The block size must be a multiple of %d and at most 1024, but is %d", WARP_SIZE, blockSize);
+    }
+    return blockSize;
+}
+
+int FusedNetwork::weightUpdateSlices(int numTiles) const
+{
+    const int waves = weightUpdateBlockSize() / WARP_SIZE;
+    return std::max(1, std::min(divUp(numTiles, waves), MAX_WEIGHT_UPDATE_SLICES));
 }
 
 static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
@@ -390,12 +421,13 @@ static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
     return ss.str();
 }
 
-std::string FusedNetwork::forwardSource(int blockSize) const
+std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string code = kl->findFile("qmlp/kernels/network_forward.h").value();
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
+    replaceAll(code, "$$POINTS_PER_LANE$$", std::to_string(pointsPerLane));
     std::vector<int> ldsW, ldsB;
     replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(false, ldsW, ldsB)));
 
@@ -422,10 +454,12 @@ std::string FusedNetwork::forwardSource(int blockSize) const
     int encodingOffset = 0;
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
-        callEncodings << "                {\n                    auto encodingOutputK = encodingOutput + " << encodingOffset
-                      << ";\n                    " << e->qualifiedName() << "::forward(encodingInput, encodingOutputK";
+        callEncodings << "            {\n                WrappedArray<f16> encodingOutputK[PPL];\n"
+                      << "#pragma unroll\n                for (int q = 0; q < PPL; ++q) encodingOutputK[q] = encodingOutput[q] + "
+                      << encodingOffset << ";\n                " << e->qualifiedName()
+                      << "::template forwardBatch<PPL>(encodingInput, encodingOutputK";
         if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
-        callEncodings << ");\n                }\n";
+        callEncodings << ");\n            }\n";
         encodingOffset += e->numOutputChannels();
     }
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
@@ -500,20 +534,29 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     callLayers << "        auto& dxIn = dx0;\n        (void)dxIn;\n";
     replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
 
-    std::stringstream callEncodings;
+    std::stringstream callEncodings, callScatter;
     int encodingOffset = 0;
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
+        const bool parameterGradients = hasEncodingGradients && e->hasParameters();
+        const std::string name = e->qualifiedName();
+        // encodings with a tile-wide scatter take their parameter gradients out of the per-point call
+        const std::string perPointParameterGradients =
+            parameterGradients ? "!" + name + "::HasTileScatter" : std::string("false");
         callEncodings << "                {\n                    auto adjEncodingOutputK = adjEncodingOutput + "
-                      << encodingOffset << ";\n                    " << e->qualifiedName() << "::template adjoint<"
-                      << (hasInputGradients ? "true" : "false") << ", "
-                      << ((hasEncodingGradients && e->hasParameters()) ? "true" : "false")
+                      << encodingOffset << ";\n                    " << name << "::template adjoint<"
+                      << (hasInputGradients ? "true" : "false") << ", " << perPointParameterGradients
                       << ">(encodingInput, adjEncodingOutputK, adjEncodingInput";
         if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
         callEncodings << ");\n                }\n";
+        if (parameterGradients)
+            callScatter << "            if constexpr (" << name << "::HasTileScatter)\n                " << name
+                        << "::scatterTile(lane, tile * TILE_POINTS, numel, inputs, sStage, STAGE_STRIDE, "
+                        << encodingOffset << ", cEncoding" << encodingIdx << ");\n";
         encodingOffset += e->numOutputChannels();
     }
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
+    replaceAll(code, "$$CALL_ENCODING_SCATTER$$", callScatter.str());
     return code;
 }
 
@@ -552,7 +595,11 @@ std::string FusedNetwork::weightUpdateKernelName(int layer, int& numChunks) cons
 
 std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFlags)
 {
-    if (kind == "inference" || kind == "forward") return forwardSource(forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false));
+    if (kind == "inference" || kind == "forward") {
+        int ppl = 1;
+        const int blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false, &ppl);
+        return forwardSource(blockSize, ppl);
+    }
     if (kind == "backward") return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true));
     if (kind == "weight_update") return weightUpdateSource(DEFAULT_BLOCK_SIZE);
     throw std::runtime_error("unknown kernel kind '" + kind + "'");
@@ -572,9 +619,10 @@ void FusedNetwork::compileInferenceKernel(bool compileOnly)
     if (inferenceKernel_.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
-    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeInference, false);
-    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half)) + (ck.blockSize / WARP_SIZE) * stageBytesPerWave();
-    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<false>", forwardSource(ck.blockSize),
+    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeInference, false, &ck.pointsPerLane);
+    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
+        + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave();
+    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<false>", forwardSource(ck.blockSize, ck.pointsPerLane),
                            loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
@@ -588,9 +636,10 @@ void FusedNetwork::compileForwardKernel(bool compileOnly)
     if (forwardKernel_.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
-    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false);
-    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half)) + (ck.blockSize / WARP_SIZE) * stageBytesPerWave();
-    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<true>", forwardSource(ck.blockSize),
+    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false, &ck.pointsPerLane);
+    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
+        + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave();
+    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<true>", forwardSource(ck.blockSize, ck.pointsPerLane),
                            loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
@@ -624,13 +673,10 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
     ak.perEntryAdjointMemoryBytes = hasNetworkGradients ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
 
     if (hasNetworkGradients) {
-        int blockSize = DEFAULT_BLOCK_SIZE;
-        if (compileOptions_.overwriteBlocksizeWeightUpdate > 0) {
-            blockSize = compileOptions_.overwriteBlocksizeWeightUpdate;
-            if (blockSize % WARP_SIZE != 0 || blockSize > 1024)
-                throw configuration_error("The block size must be a multiple of %d and at most 1024, but is %d", WARP_SIZE, blockSize);
-        }
+        const int blockSize = weightUpdateBlockSize();
         const std::string source = weightUpdateSource(blockSize);
+        ak.reduce.blockSize = 1024;
+        ak.reduce.fun = kl->getKernel("qmlp::kernel::WeightUpdateReduceKernel", source, loaderFlags(compileOnly)).value();
         ak.layers.resize(layers_.size());
         for (size_t layer = 0; layer < layers_.size(); ++layer) {
             auto& wk = ak.layers[layer];
@@ -695,7 +741,7 @@ void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t strea
 
     const int waves = ck.blockSize / WARP_SIZE;
     const int numTiles = divUp(numel, TILE_POINTS);
-    const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+    const int grid = std::min(divUp(numTiles, waves * ck.pointsPerLane), ck.fullGrid);
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
     const half* networkParams = parametersInference_.dataPtr<half>();
@@ -740,7 +786,7 @@ void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory,
 
     const int waves = ck.blockSize / WARP_SIZE;
     const int numTiles = divUp(numel, TILE_POINTS);
-    const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+    const int grid = std::min(divUp(numTiles, waves * ck.pointsPerLane), ck.fullGrid);
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
     const half* networkParams = parametersInference_.dataPtr<half>();
@@ -765,7 +811,11 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
     for (const auto& l : layers_) adjointChannels += l.channelsOut;
     const int perEntry = (adjointFlags & GRADIENTS_NETWORK_WEIGHTS) ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
     numElements = roundUp(numElements, WARP_SIZE);
-    return static_cast<size_t>(perEntry) * static_cast<size_t>(numElements);
+    size_t bytes = static_cast<size_t>(perEntry) * static_cast<size_t>(numElements);
+    // behind the adjoint pre-activations: the partial weight gradients of the batch slices
+    if (adjointFlags & GRADIENTS_NETWORK_WEIGHTS)
+        bytes += static_cast<size_t>(weightUpdateSlices(numElements / TILE_POINTS)) * numParameters_ * sizeof(float);
+    return bytes;
 }
 
 size_t FusedNetwork::adjointMemory(const Tensor& input, AdjointModeFlags adjointFlags)
@@ -843,14 +893,17 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         ensureStreams();
         QMLP_HIP_CALL(qmlp_hip_event_record(adjointEvent_, stream));
     }
+    const int slices = weightUpdateSlices(numTiles);
+    float* partial = reinterpret_cast<float*>(static_cast<char*>(tmpMemoryAdjoint)
+                                              + static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64));
     for (size_t layer = 0; layer < layers_.size(); ++layer) {
         const auto& ls = layers_[layer];
         const auto& ali = backwardInfo_[layer];
         const auto& wk = ak.layers[layer];
 
-        float* gradBase = parametersGradients_.dataPtr<float>();
-        float* outAdjWeights = gradBase + ls.weightsStart;
-        float* outAdjBias = ls.useBias ? gradBase + ls.biasStart : nullptr;
+        float* outAdjWeights = partial + ls.weightsStart;
+        float* outAdjBias = ls.useBias ? partial + ls.biasStart : nullptr;
+        int sliceStride = numParameters_;
         const half* aIn = static_cast<const half*>(tmpMemoryAdjoint) + static_cast<ptrdiff_t>(ali.offsetAdjOut) * numel64;
         const half* bIn = static_cast<const half*>(tmpMemoryForward) + static_cast<ptrdiff_t>(ali.offsetIn) * numel64;
 
@@ -859,15 +912,20 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
             layerStream = ali.stream;
             QMLP_HIP_CALL(qmlp_hip_stream_wait_event(ali.stream, adjointEvent_));
         }
-        const int waves = wk.kernel.blockSize / WARP_SIZE;
-        const int slices = std::max(1, std::min(divUp(numTiles, waves), std::max(1, wk.kernel.fullGrid / wk.numChunks)));
         int numTilesArg = numTiles;
-        void* args[] = {&numTilesArg, &outAdjWeights, &outAdjBias, &aIn, &bIn};
+        void* args[] = {&numTilesArg, &outAdjWeights, &outAdjBias, &sliceStride, &aIn, &bIn};
         wk.kernel.fun.launch(slices * wk.numChunks, wk.kernel.blockSize, wk.kernel.sharedMemorySize, layerStream, args);
         if (parallel) {
             QMLP_HIP_CALL(qmlp_hip_event_record(ali.event, ali.stream));
             QMLP_HIP_CALL(qmlp_hip_stream_wait_event(stream, ali.event));
         }
+    }
+    {
+        int count = numParameters_, numSlices = slices;
+        const float* partialArg = partial;
+        float* gradBase = parametersGradients_.dataPtr<float>();
+        void* args[] = {&count, &numSlices, &partialArg, &gradBase};
+        ak.reduce.fun.launch(divUp(numParameters_, WARP_SIZE), ak.reduce.blockSize, 0, stream, args);
     }
 }
 

@@ -139,10 +139,15 @@ def test_temporary_memory_sizes():
     net = qmlp.Network(json.dumps(bc.CONFIGS[3]["cfg"]))
     per_fwd = 2 * (32 + 64 + 64 + 16)
     per_adj = 2 * (64 + 64 + 16)
-    for n, padded in ((1, 64), (64, 64), (65, 128), (1 << 18, 1 << 18)):
+    # behind the adjoint pre-activations: fp32 partial weight gradients of up to 512 batch
+    # slices (one workgroup of 4 wavefronts = 4 tiles each)
+    n_params = net.num_network_parameters()
+    for n, padded, slices in ((1, 64, 1), (64, 64, 1), (65, 128, 1), (1000, 1024, 4), (1 << 18, 1 << 18, 512)):
         assert net.forward_memory(n, 7) == per_fwd * padded
-        assert net.adjoint_memory(n, 7) == per_adj * padded
+        assert net.adjoint_memory(n, 7) == per_adj * padded + slices * n_params * 4
+        assert net.adjoint_memory(n, 2) == per_adj * padded + slices * n_params * 4
         assert net.adjoint_memory(n, 1) == 0
+        assert net.adjoint_memory(n, 5) == 0
     with pytest.raises(qmlp.QmlpError, match="At least one derivative"):
         net.adjoint_memory(10, 0)
 
@@ -174,9 +179,9 @@ def test_kernels_compile_for_gfx950_without_a_gpu_and_are_cached(tmp_path):
         c0, h0 = qmlp._lib.kernel_cache_stats()
         qmlp.Network(json.dumps(cfg)).precompile(7)
         c1, h1 = qmlp._lib.kernel_cache_stats()
-        assert c1 - c0 == 5 and h1 == h0          # inference, forward, backward, 2 weight updates
+        assert c1 - c0 == 6 and h1 == h0          # inference, forward, backward, 2 weight updates + reduce
         files = os.listdir(cache)
-        assert len(files) == 5 and all(f.endswith(".co") for f in files)
+        assert len(files) == 6 and all(f.endswith(".co") for f in files)
         qmlp.Network(json.dumps(cfg)).precompile(7)
         c2, h2 = qmlp._lib.kernel_cache_stats()
         assert c2 == c1                            # nothing recompiled (memory or disk cache)
