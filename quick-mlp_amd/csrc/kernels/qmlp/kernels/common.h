@@ -33,6 +33,50 @@ __device__ __forceinline__ half2 h2ZERO() { return __half2{hZERO(), hZERO()}; }
 __device__ __forceinline__ half toHalf(f16 v) { return __half_raw{v}; }
 __device__ __forceinline__ f16 fromHalf(half v) { return static_cast<__half_raw>(v).data; }
 
+/**
+ * Transcendental functions of the half-precision intrinsics vocabulary that activation
+ * snippets use (hsin, hcos, hexp), evaluated with the hardware's fp32 units on the
+ * fp16 argument: convert, one multiply, one quarter-rate instruction, convert back.
+ * The library versions of the HIP headers run a software argument reduction of some
+ * forty instructions per value, which made sine networks ALU-bound at a small fraction
+ * of the matrix-core rate. The results differ from the correctly rounded ones by at
+ * most one fp16 ulp.
+ *
+ * They are function objects on purpose: a snippet inside this namespace that calls
+ * hsin(x) finds the object by ordinary lookup, and because that is not a function, the
+ * argument-dependent lookup that would also bring in ::hsin(__half) does not take place.
+ */
+namespace fastmath
+{
+struct Sin
+{
+    __device__ __forceinline__ half operator()(half x) const
+    {
+        // v_sin_f32 takes revolutions and is defined on [-256, 256]
+        const float rev = __half2float(x) * 0.15915494309189535f;
+        return __float2half(__builtin_amdgcn_sinf(__builtin_amdgcn_fractf(rev)));
+    }
+};
+struct Cos
+{
+    __device__ __forceinline__ half operator()(half x) const
+    {
+        const float rev = __half2float(x) * 0.15915494309189535f;
+        return __float2half(__builtin_amdgcn_cosf(__builtin_amdgcn_fractf(rev)));
+    }
+};
+struct Exp
+{
+    __device__ __forceinline__ half operator()(half x) const
+    {
+        return __float2half(__builtin_amdgcn_exp2f(__half2float(x) * 1.4426950408889634f));
+    }
+};
+}
+static constexpr fastmath::Sin hsin{};
+static constexpr fastmath::Cos hcos{};
+static constexpr fastmath::Exp hexp{};
+
 /** Templated casting between float and half datatypes */
 template <typename Dst, typename Src> __device__ __forceinline__ Dst fcast(const Src& src);
 template <> __device__ __forceinline__ float fcast<float, half>(const half& src) { return __half2float(src); }

@@ -419,11 +419,11 @@ struct EncodingHashGrid
 
     /**
      * Parameter gradients of the 64 points of one wavefront tile. The atomic units handle
-     * one request per group of lanes of an instruction that address contiguous memory, and
-     * their rate is bound by requests, not by lanes. Therefore 2*F neighbouring lanes share
-     * one point and add the 2*F contiguous values of a pair of neighbouring entries (the
-     * same pairs as in gatherLevel) in one request; the wavefront covers its 64 points in
-     * 2*F rounds of 64/(2F) points. Every lane recomputes the level setup of its point; the
+     * one request per aligned 64-byte block that neighbouring lanes of an instruction
+     * address, and their rate is bound by requests (about 21e9 per second on the whole
+     * device, wherever the data lives), not by lanes. Therefore 2*F neighbouring lanes share
+     * one point and add the F features of two corners that are neighbours in memory; the
+     * wavefront covers its 64 points in 2*F rounds of 64/(2F) points. Every lane recomputes the level setup of its point; the
      * arithmetic is free next to the atomics.
      *
      * \param index0 index of the first point of the tile
@@ -461,60 +461,31 @@ struct EncodingHashGrid
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 const LevelSetup s = setupLevel(l, pos);
-                const int R = Cfg::resolution[l];
                 const bool hashed = Cfg::hashed[l];
                 const unsigned base = static_cast<unsigned>(Cfg::memoryOffset[l]);
                 const float adj = static_cast<float>(adjRow[(Cfg::Concat ? l * F : 0) + i]);
-                if (!hashed && R >= 2) {
-                    constexpr int PD = D - 1;
-                    const unsigned zL = s.termL[PD], zH = s.termH[PD];
-                    const unsigned zb = min(zL, static_cast<unsigned>(R - 2));
-                    const unsigned zk = zb + static_cast<unsigned>(k);
-                    const float wz = (zL == zk ? 1.f - s.f[PD] : 0.f) + (zH == zk ? s.f[PD] : 0.f);
+                // The lanes k = 0 | 1 of a group take the lower | upper corner along the dimension whose
+                // neighbours are close in memory: the last one in a dense level (adjacent entries), the
+                // first one in a hashed level (multiplier 1: the same 64-byte block 7 times out of 8).
+                const int PD = hashed ? 0 : D - 1;
+                const float wk = k ? s.f[PD] : 1.f - s.f[PD];
+                const unsigned tk = k ? s.termH[PD] : s.termL[PD];
 #pragma unroll
-                    for (int c = 0; c < NC / 2; ++c) {
-                        unsigned idx = zb;
-                        float w = 1.f;
+                for (int c = 0; c < NC / 2; ++c) {
+                    unsigned idx = tk;
+                    float w = 1.f;
+                    int bit = 0;
 #pragma unroll
-                        for (int d = PD - 1; d >= 0; --d) {
-                            const bool hi = (c >> d) & 1;
-                            idx += hi ? s.termH[d] : s.termL[d];
-                            w = w * (hi ? s.f[d] : (1.f - s.f[d]));
-                        }
-                        unsafeAtomicAdd(grad + (base + idx * static_cast<unsigned>(F) + static_cast<unsigned>(sub)),
-                                        (w * wz) * adj);
+                    for (int d = D - 1; d >= 0; --d) {
+                        if (d == PD) continue;
+                        const bool hi = (c >> bit) & 1;
+                        ++bit;
+                        const unsigned t = hi ? s.termH[d] : s.termL[d];
+                        idx = hashed ? (idx ^ t) : (idx + t);
+                        w = w * (hi ? s.f[d] : (1.f - s.f[d]));
                     }
-                } else if (hashed && detail::isPow2(Cfg::hashGridSize[l]) && Cfg::hashGridSize[l] >= 2u) {
-                    const unsigned mask = Cfg::hashGridSize[l] - 1u;
-                    const float wxL = 1.f - s.f[0], wxH = s.f[0];
-#pragma unroll
-                    for (int c = 0; c < NC / 2; ++c) {
-                        unsigned rest = 0u;
-                        float w = 1.f;
-#pragma unroll
-                        for (int d = D - 1; d >= 1; --d) {
-                            const bool hi = (c >> (d - 1)) & 1;
-                            rest ^= hi ? s.termH[d] : s.termL[d];
-                            w = w * (hi ? s.f[d] : (1.f - s.f[d]));
-                        }
-                        const unsigned idxL = (s.termL[0] ^ rest) & mask;
-                        const unsigned idxH = (s.termH[0] ^ rest) & mask;
-                        const bool samePair = ((idxL ^ idxH) & ~1u) == 0u;
-                        const unsigned uk = static_cast<unsigned>(k);
-                        const float wx = ((idxL & 1u) == uk ? wxL : 0.f) + ((samePair && (idxH & 1u) == uk) ? wxH : 0.f);
-                        unsafeAtomicAdd(grad + (base + (idxL & ~1u) * static_cast<unsigned>(F) + static_cast<unsigned>(sub)),
-                                        (w * wx) * adj);
-                        if (!samePair && (idxH & 1u) == uk)
-                            unsafeAtomicAdd(grad + (base + idxH * static_cast<unsigned>(F) + static_cast<unsigned>(i)),
-                                            (w * wxH) * adj);
-                    }
-                } else {
-                    // corner by corner; the lanes of the lower half of the group add the F features
-#pragma unroll
-                    for (int c = 0; c < NC; ++c) {
-                        if (k == 0)
-                            unsafeAtomicAdd(grad + (cornerOffset(l, s, c) + static_cast<unsigned>(i)), cornerWeight(s, c) * adj);
-                    }
+                    if (hashed) idx %= Cfg::hashGridSize[l];
+                    unsafeAtomicAdd(grad + (base + idx * static_cast<unsigned>(F) + static_cast<unsigned>(i)), (w * wk) * adj);
                 }
             }
         }
