@@ -26,6 +26,14 @@ for p in (os.path.join(ROOT, "quick-mlp_amd"), os.path.join(ROOT, "oracle")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 
+# HBM bytes one launch moves, from hardware counters (two profiler runs of this script:
+# FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for the
+# 256 MiB device copy of --copy-calibration: x2.000 and x1.000 on MI355X). The summary
+# with the commands is kept under profiles/. Workloads without a counter run report null.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg2-inference": {"points": 1 << 20, "fetch": 660933.1 * 1024 * 2.0, "write": 4110.1 * 1024 * 1.0},
+}
+
 WORKLOADS = {
     "cfg1-inference": (1, False),
     "cfg2-inference": (2, False),
@@ -203,6 +211,11 @@ def main():
     bytes_per_point = c["gather_bytes_per_point"] + c["io_bytes_per_point"]
     achieved_gbs = bytes_per_point * n / (launch_ms * 1e-3) / 1e9
     flops = c["flop_per_point"] * n / (launch_ms * 1e-3)
+    traffic = None
+    m = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    if m is not None and m["points"] == n:
+        # same form as "achieved": bytes of one launch over the launch duration measured now
+        traffic = (m["fetch"] + m["write"]) / (launch_ms * 1e-3) / 1e9
     result = {
         "metric": "points/sec fused hashgrid+MLP inference & train step; % MFMA/HBM roofline",
         "value": value, "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -212,7 +225,9 @@ def main():
                    "network": "x".join(str(l["n_out"]) for l in c["cfg"]["network"]),
                    "encodings": [e["id"] for e in c["cfg"]["encodings"]]},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_bytes_per_launch": None if traffic is None else m["fetch"] + m["write"],
+                     "algorithmic_bytes_per_launch": bytes_per_point * n,
                      "kernel": "NetworkKernelInferenceAndForward" if not train else "train step (4-5 kernels)",
                      "launch_ms": launch_ms, "algorithmic_bytes_per_point": bytes_per_point},
         "mfma": {"achieved_tflops": flops / 1e12, "peak_tflops": MFMA_FP16_PEAK_TFLOPS,
