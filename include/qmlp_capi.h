@@ -134,6 +134,10 @@ int qmlp_encoding_forward(qmlp_encoding_t encoding, const qmlp_tensor* input, co
 int qmlp_encoding_adjoint(qmlp_encoding_t encoding, const qmlp_tensor* input, const qmlp_tensor* adj_output,
                           const qmlp_tensor* adj_input, void* stream, const qmlp_tensor* parameters_forward,
                           const qmlp_tensor* parameters_gradients, int adjoint_mode);
+/* Compiles the standalone kernels (forward, and the adjoint of adjoint_mode if > 0) into the
+ * kernel cache without a GPU. No counterpart in the reference, which compiles lazily inside
+ * forward()/adjoint() (src_cpp/src/iencoding.cpp:30-43,98-112). */
+int qmlp_encoding_precompile(qmlp_encoding_t encoding, int adjoint_mode);
 /* HashGrid only: level table as the reference computes it in
  * src_cpp/src/encoding_hashgrid.cpp:63-96. Arrays hold `capacity` entries. */
 int qmlp_encoding_hashgrid_levels(qmlp_encoding_t encoding, int capacity, int* num_levels, int* memory_offset,

@@ -302,6 +302,93 @@ void qo_hashgrid_adjoint(const qo_hashgrid* g, const float* table, const float* 
                                res_factor, 1);
 }
 
+/* ------------------------------------------------------------------ line integration */
+
+/* Slab test of encoding_line_integration.cuh:33-49: fp32, IEEE division (a zero direction
+ * component gives +-inf or NaN, which fminf/fmaxf drop). */
+static void line_intersect(const qo_line* line, const float* start, const float* dir,
+                           float* tmin, float* tmax)
+{
+    float lo[3], hi[3];
+    for (int d = 0; d < 3; ++d) {
+        const float inv = 1.0f / dir[d];
+        const float ta = (line->bb_min[d] - start[d]) * inv;
+        const float tb = (line->bb_min[d] + line->bb_size[d] - start[d]) * inv;
+        lo[d] = fminf(ta, tb);
+        hi[d] = fmaxf(ta, tb);
+    }
+    *tmin = fmaxf(fmaxf(lo[0], lo[1]), lo[2]);
+    *tmax = fminf(fminf(hi[0], hi[1]), hi[2]);
+}
+
+static void line_forward_point(const qo_line* line, const qo_hashgrid* child, const float* table,
+                               const float* x, float* out)
+{
+    const int C = qo_hashgrid_num_outputs(child);
+    const float* start = x + line->start_in;
+    const float* dir = start + 3;
+    float tmin, tmax, contribution[QO_MAX_LEVELS * 16], pos[3];
+    line_intersect(line, start, dir, &tmin, &tmax);
+    const int steps = (int)floorf((tmax - tmin) / line->stepsize);
+    for (int i = 0; i < C; ++i) out[i] = 0.f;
+    for (float t = tmin; t < tmax; t += line->stepsize) {
+        for (int d = 0; d < 3; ++d) pos[d] = fmaf(t, dir[d], start[d]);
+        hashgrid_forward_point(child, table, pos, contribution);
+        for (int i = 0; i < C; ++i) out[i] += contribution[i];
+    }
+    if (line->blending == QO_BLEND_AVERAGE && steps > 0) {
+        const float scale = 1.0f / (float)steps;
+        for (int i = 0; i < C; ++i) out[i] *= scale;
+    }
+}
+
+/* tmin / tmax are constants of the adjoint (encoding_line_integration.cuh:138-152). */
+static void line_adjoint_point(const qo_line* line, const qo_hashgrid* child, const float* table,
+                               const float* x, const float* adj_out, float* adj_x, float* grad_table,
+                               int res_factor, int atomic)
+{
+    const int C = qo_hashgrid_num_outputs(child);
+    const float* start = x + line->start_in;
+    const float* dir = start + 3;
+    float tmin, tmax, adj_accu[QO_MAX_LEVELS * 16], pos[3], adj_pos[3];
+    float adj_start[3] = {0.f, 0.f, 0.f}, adj_dir[3] = {0.f, 0.f, 0.f};
+    line_intersect(line, start, dir, &tmin, &tmax);
+    const int steps = (int)floorf((tmax - tmin) / line->stepsize);
+    float scale = 1.0f;
+    if (line->blending == QO_BLEND_AVERAGE) scale = steps > 0 ? 1.0f / (float)steps : 1.0f;
+    for (int i = 0; i < C; ++i) adj_accu[i] = scale * adj_out[i];
+    for (float t = tmin; t < tmax; t += line->stepsize) {
+        for (int d = 0; d < 3; ++d) { pos[d] = fmaf(t, dir[d], start[d]); adj_pos[d] = 0.f; }
+        hashgrid_adjoint_point(child, table, pos, adj_accu, adj_x ? adj_pos : NULL, grad_table,
+                               res_factor, atomic);
+        if (adj_x)
+            for (int d = 0; d < 3; ++d) { adj_start[d] += adj_pos[d]; adj_dir[d] += adj_pos[d] * t; }
+    }
+    if (adj_x)
+        for (int d = 0; d < 3; ++d) {
+            adj_x[line->start_in + d] += adj_start[d];
+            adj_x[line->start_in + 3 + d] += adj_dir[d];
+        }
+}
+
+void qo_line_forward(const qo_line* line, const qo_hashgrid* child, const float* table, const float* x,
+                     long N, long x_stride, float* out, long out_stride)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (long n = 0; n < N; ++n)
+        line_forward_point(line, child, table, x + n * x_stride, out + n * out_stride);
+}
+
+void qo_line_adjoint(const qo_line* line, const qo_hashgrid* child, const float* table, const float* x,
+                     long N, long x_stride, const float* adj_out, long adj_out_stride,
+                     float* adj_x, long adj_x_stride, float* grad_table, int res_factor)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (long n = 0; n < N; ++n)
+        line_adjoint_point(line, child, table, x + n * x_stride, adj_out + n * adj_out_stride,
+                           adj_x ? adj_x + n * adj_x_stride : NULL, grad_table, res_factor, 1);
+}
+
 /* ------------------------------------------------------------------ activations */
 
 float qo_act_forward(int act, float param, float x)
@@ -333,7 +420,7 @@ int qo_network_encoded_channels(const qo_network* net)
     int c = 0;
     for (int e = 0; e < net->n_enc; ++e)
         c += net->enc_kind[e] == QO_ENC_IDENTITY ? net->enc_nin[e]
-                                                 : qo_hashgrid_num_outputs(net->enc_grid[e]);
+                                                 : qo_hashgrid_num_outputs(net->enc_grid[e]);  /* grid, or a line's child */
     return c;
 }
 
@@ -351,6 +438,9 @@ static void encode_point(const qo_network* net, const float* x, float* row)
         if (net->enc_kind[e] == QO_ENC_IDENTITY) {
             for (int i = 0; i < net->enc_nin[e]; ++i) row[off + i] = x[net->enc_start[e] + i];
             off += net->enc_nin[e];
+        } else if (net->enc_kind[e] == QO_ENC_LINE) {
+            line_forward_point(net->enc_line[e], net->enc_grid[e], net->enc_table[e], x, row + off);
+            off += qo_hashgrid_num_outputs(net->enc_grid[e]);
         } else {
             hashgrid_forward_point(net->enc_grid[e], net->enc_table[e], x, row + off);
             off += qo_hashgrid_num_outputs(net->enc_grid[e]);
@@ -499,7 +589,10 @@ void qo_network_backward(const qo_network* net, const float* X, long N, long x_s
                         off += net->enc_nin[e];
                     } else {
                         float* gt = (flags & QO_GRAD_ENCODINGS) ? net->enc_grad[e] : NULL;
-                        if (ax || gt)
+                        if ((ax || gt) && net->enc_kind[e] == QO_ENC_LINE)
+                            line_adjoint_point(net->enc_line[e], net->enc_grid[e], net->enc_table[e], x,
+                                               cur + off, ax, gt, net->res_factor, 1);
+                        else if (ax || gt)
                             hashgrid_adjoint_point(net->enc_grid[e], net->enc_table[e], x,
                                                    cur + off, ax, gt, net->res_factor, 1);
                         off += qo_hashgrid_num_outputs(net->enc_grid[e]);

@@ -13,6 +13,8 @@
  *   qo_hashgrid_corners   encoding_hashgrid.cuh:72-85,174-215,267-285 (corner set + weights)
  *   qo_hashgrid_forward   encoding_hashgrid.cuh:92-115,267-336
  *   qo_hashgrid_adjoint   encoding_hashgrid.cuh:117-166,187-241,345-422
+ *   qo_line_forward/adjoint  src_cpp/include/qmlp/kernels/encoding_line_integration.cuh:26-166
+ *                         (slab test :26-49, march + blending :62-100, adjoint :103-163)
  *   identity encoding     src_cpp/include/qmlp/kernels/encoding_identity.cuh:12-39
  *   activations           src_cpp/include/qmlp/builtin-activations.json:1-21,
  *                         tests_cpp/test_against_eigen.h:31-87
@@ -55,7 +57,8 @@ extern "C" {
 enum { QO_ACT_RELU = 0, QO_ACT_CELU = 1, QO_ACT_SINE = 2, QO_ACT_IDENTITY = 3,
        QO_ACT_SINE_FREQ = 4 /* z = sin(param*x) */ };
 enum { QO_CONCAT = 0, QO_ADD = 1 };
-enum { QO_ENC_IDENTITY = 0, QO_ENC_HASHGRID = 1 };
+enum { QO_ENC_IDENTITY = 0, QO_ENC_HASHGRID = 1, QO_ENC_LINE = 2 };
+enum { QO_BLEND_ADDITIVE = 0, QO_BLEND_AVERAGE = 1 };
 enum { QO_GRAD_INPUT = 1, QO_GRAD_WEIGHTS = 2, QO_GRAD_ENCODINGS = 4 };
 
 typedef struct {
@@ -69,6 +72,16 @@ typedef struct {
     float bb_inv[QO_MAX_DIM];
 } qo_hashgrid;
 
+/* Fixed-step line integration through a 3-D child grid (whose start_in must be 0): ray
+ * start in columns [start_in, start_in+3), direction in the 3 columns after. */
+typedef struct {
+    int start_in;
+    int blending;
+    float stepsize;
+    float bb_min[3];
+    float bb_size[3];
+} qo_line;
+
 typedef struct {
     int n_in;                              /* columns of the raw input */
     int n_enc;
@@ -78,6 +91,7 @@ typedef struct {
     const qo_hashgrid* enc_grid[QO_MAX_ENCODINGS];
     const float* enc_table[QO_MAX_ENCODINGS];
     float* enc_grad[QO_MAX_ENCODINGS];     /* += ; may be NULL */
+    const qo_line* enc_line[QO_MAX_ENCODINGS]; /* QO_ENC_LINE: the march; enc_grid is its child */
     int n_layers;
     int cin[QO_MAX_LAYERS];                /* padded widths (multiples of 16) */
     int cout[QO_MAX_LAYERS];
@@ -109,6 +123,12 @@ void qo_hashgrid_forward(const qo_hashgrid* g, const float* table, const float* 
 void qo_hashgrid_adjoint(const qo_hashgrid* g, const float* table, const float* x, long N,
                          long x_stride, const float* adj_out, long adj_out_stride,
                          float* adj_x, long adj_x_stride, float* grad_table, int res_factor);
+
+void qo_line_forward(const qo_line* line, const qo_hashgrid* child, const float* table, const float* x,
+                     long N, long x_stride, float* out, long out_stride);
+void qo_line_adjoint(const qo_line* line, const qo_hashgrid* child, const float* table, const float* x,
+                     long N, long x_stride, const float* adj_out, long adj_out_stride,
+                     float* adj_x, long adj_x_stride, float* grad_table, int res_factor);
 
 float qo_act_forward(int act, float param, float x);
 float qo_act_adjoint(int act, float param, float x, float adjz);

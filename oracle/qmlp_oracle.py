@@ -22,7 +22,7 @@ _LIB_PATH = os.path.join(_HERE, "libqmlp_oracle.so")
 MAX_LEVELS, MAX_DIM, MAX_ENC, MAX_LAYERS = 32, 6, 8, 16
 ACT_RELU, ACT_CELU, ACT_SINE, ACT_IDENTITY, ACT_SINE_FREQ = 0, 1, 2, 3, 4
 CONCAT, ADD = 0, 1
-ENC_IDENTITY, ENC_HASHGRID = 0, 1
+ENC_IDENTITY, ENC_HASHGRID, ENC_LINE = 0, 1, 2
 GRAD_INPUT, GRAD_WEIGHTS, GRAD_ENCODINGS = 1, 2, 4
 
 BUILTIN_ACTIVATIONS = {
@@ -46,6 +46,13 @@ class HashGridStruct(ctypes.Structure):
     ]
 
 
+class LineStruct(ctypes.Structure):
+    _fields_ = [
+        ("start_in", ctypes.c_int), ("blending", ctypes.c_int), ("stepsize", ctypes.c_float),
+        ("bb_min", ctypes.c_float * 3), ("bb_size", ctypes.c_float * 3),
+    ]
+
+
 class NetworkStruct(ctypes.Structure):
     _fields_ = [
         ("n_in", ctypes.c_int), ("n_enc", ctypes.c_int),
@@ -53,6 +60,7 @@ class NetworkStruct(ctypes.Structure):
         ("enc_nin", ctypes.c_int * MAX_ENC),
         ("enc_grid", ctypes.POINTER(HashGridStruct) * MAX_ENC),
         ("enc_table", _fp * MAX_ENC), ("enc_grad", _fp * MAX_ENC),
+        ("enc_line", ctypes.POINTER(LineStruct) * MAX_ENC),
         ("n_layers", ctypes.c_int),
         ("cin", ctypes.c_int * MAX_LAYERS), ("cout", ctypes.c_int * MAX_LAYERS),
         ("act", ctypes.c_int * MAX_LAYERS), ("act_param", ctypes.c_float * MAX_LAYERS),
@@ -96,6 +104,11 @@ def lib():
         L.qo_hashgrid_adjoint.argtypes = [ctypes.POINTER(HashGridStruct), _fp, _fp, ctypes.c_long,
                                           ctypes.c_long, _fp, ctypes.c_long, _fp, ctypes.c_long,
                                           _fp, ctypes.c_int]
+        L.qo_line_forward.argtypes = [ctypes.POINTER(LineStruct), ctypes.POINTER(HashGridStruct), _fp, _fp,
+                                      ctypes.c_long, ctypes.c_long, _fp, ctypes.c_long]
+        L.qo_line_adjoint.argtypes = [ctypes.POINTER(LineStruct), ctypes.POINTER(HashGridStruct), _fp, _fp,
+                                      ctypes.c_long, ctypes.c_long, _fp, ctypes.c_long, _fp, ctypes.c_long,
+                                      _fp, ctypes.c_int]
         L.qo_act_forward.restype = ctypes.c_float
         L.qo_act_forward.argtypes = [ctypes.c_int, ctypes.c_float, ctypes.c_float]
         L.qo_act_adjoint.restype = ctypes.c_float
@@ -198,6 +211,47 @@ class HashGrid:
         return adj_x, grad
 
 
+class LineIntegration:
+    """Fixed-step ray march through a child HashGrid (encoding_line_integration.cpp:43-51 keys:
+    start_in, n_in, volume, stepsize, blending)."""
+
+    def __init__(self, cfg):
+        if int(cfg["n_in"]) != 3:
+            raise ValueError("LineIntegration is only defined for 3D volumes")
+        child = dict(cfg["volume"], start_in=0, n_in=3)
+        self.child = HashGrid(child)
+        self.start_in = int(cfg["start_in"])
+        self.stepsize = float(cfg["stepsize"])
+        if not self.stepsize > 0:
+            raise ValueError("Stepsize must be positive")
+        self.blending = {"additive": 0, "average": 1}[cfg["blending"]]
+        self.num_outputs = self.child.num_outputs
+        self.n_params = self.child.n_params
+        self.s = LineStruct()
+        self.s.start_in, self.s.blending, self.s.stepsize = self.start_in, self.blending, self.stepsize
+        bb_min = child.get("bounding_box_min") or [-0.5] * 3
+        bb_size = child.get("bounding_box_size") or [1.0] * 3
+        for d in range(3):
+            self.s.bb_min[d], self.s.bb_size[d] = bb_min[d], bb_size[d]
+
+    def forward(self, table, x):
+        x, table = _f32(x), _f32(table)
+        out = np.zeros((x.shape[0], self.num_outputs), np.float32)
+        lib().qo_line_forward(ctypes.byref(self.s), ctypes.byref(self.child.s), _ptr(table), _ptr(x),
+                              x.shape[0], x.shape[1], _ptr(out), out.shape[1])
+        return out
+
+    def adjoint(self, table, x, adj_out, input_grads=True, param_grads=True, res_factor=1):
+        x, table, adj_out = _f32(x), _f32(table), _f32(adj_out)
+        adj_x = np.zeros_like(x) if input_grads else None
+        grad = np.zeros_like(table) if param_grads else None
+        lib().qo_line_adjoint(ctypes.byref(self.s), ctypes.byref(self.child.s), _ptr(table), _ptr(x),
+                              x.shape[0], x.shape[1], _ptr(adj_out), adj_out.shape[1],
+                              _ptr(adj_x) if input_grads else None, x.shape[1],
+                              _ptr(grad) if param_grads else None, int(res_factor))
+        return adj_x, grad
+
+
 class Network:
     """The fused network of a JSON spec, evaluated on the CPU in fp32."""
 
@@ -221,6 +275,11 @@ class Network:
                 enc = ("hashgrid", g)
                 encoded += g.num_outputs
                 top = g.start_in + g.dim - 1
+            elif e["id"] == "LineIntegration":
+                li = LineIntegration(e)
+                enc = ("line", li)
+                encoded += li.num_outputs
+                top = li.start_in + 5
             else:
                 raise ValueError("No encoding with id '%s' found" % e["id"])
             if top >= self.n_in:
@@ -293,8 +352,13 @@ class Network:
                 s.enc_kind[i] = ENC_IDENTITY
                 s.enc_start[i], s.enc_nin[i] = e[1], e[2]
             else:
-                s.enc_kind[i] = ENC_HASHGRID
-                s.enc_grid[i] = ctypes.pointer(e[1].s)
+                if e[0] == "line":
+                    s.enc_kind[i] = ENC_LINE
+                    s.enc_line[i] = ctypes.pointer(e[1].s)
+                    s.enc_grid[i] = ctypes.pointer(e[1].child.s)
+                else:
+                    s.enc_kind[i] = ENC_HASHGRID
+                    s.enc_grid[i] = ctypes.pointer(e[1].s)
                 assert self.tables[i] is not None, "encoding table not set"
                 s.enc_table[i] = _ptr(self.tables[i])
                 if table_grads is not None and table_grads[i] is not None:

@@ -94,8 +94,9 @@ private:
         int sharedMemorySize = 0;
         int fullGrid = 0;
     };
-    std::optional<CompiledKernel> inferenceKernel_;
-    std::optional<CompiledKernel> forwardKernel_;
+    // [store intermediates][0: the preferred number of tiles per wave, 1: one tile per wave,
+    // for batches too small to fill the device with the former]
+    std::optional<CompiledKernel> forwardKernels_[2][2];
 
     struct AdjointLayerInfo
     {
@@ -228,8 +229,8 @@ public:
     std::string generatedSource(const std::string& kind, int adjointFlags = 0);
 
 private:
-    void compileInferenceKernel(bool compileOnly = false);
-    void compileForwardKernel(bool compileOnly = false);
+    void compileForwardKernel(bool store, bool narrow, bool compileOnly = false);
+    const CompiledKernel& forwardKernelFor(bool store, int numTiles);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane) const;

@@ -102,7 +102,15 @@ public:
                          const std::optional<const Tensor>& parametersGradients,
                          int adjointMode = AdjointMode::ALL_GRADIENTS);
 
+    /**
+     * Compiles the standalone forward kernel and, for adjointMode > 0, the adjoint kernel of
+     * that mode into the kernel cache without loading them; needs no GPU.
+     */
+    void precompile(int adjointMode = AdjointMode::ALL_GRADIENTS);
+
 private:
+    std::string forwardKernelSource() const;
+    std::string adjointKernelSource(int adjointMode) const;
     std::optional<KernelFunction> forwardKernel_;
     std::optional<KernelFunction> adjointKernel_[AdjointMode::ALL_GRADIENTS + 1];
 };

@@ -326,18 +326,8 @@ struct EncodingHashGrid
         for (int i = 0; i < F; ++i) sum[i] = 0.f;
 #pragma unroll
         for (int l = 0; l < L; ++l) {
-            const LevelSetup s = setupLevel(l, pos);
             float feat[F];
-#pragma unroll
-            for (int i = 0; i < F; ++i) feat[i] = 0.f;
-#pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                const float w = cornerWeight(s, c);
-                float v[F];
-                detail::loadFeatures<F>(params.parametersForward + cornerOffset(l, s, c), v);
-#pragma unroll
-                for (int i = 0; i < F; ++i) feat[i] += w * v[i];
-            }
+            gatherLevel(l, pos, params.parametersForward, feat);
             if constexpr (Cfg::Concat) {
 #pragma unroll
                 for (int i = 0; i < F; ++i) output[l * F + i] = fcast<O_t>(feat[i]);
@@ -427,13 +417,13 @@ struct EncodingHashGrid
      * arithmetic is free next to the atomics.
      *
      * \param index0 index of the first point of the tile
-     * \param adjRows the wave's staging rows with the adjoint of the encoded input; the row of
-     *    point p of the tile is adjRows + stageRow(p) * rowStride, this encoding's channels
-     *    start at channelOffset
+     * \param adjOutput callable (point of the tile 0..63, output channel of this encoding) ->
+     *    adjoint of that output as float
      */
-    __device__ __forceinline__ static void scatterTile(int lane, int index0, int numel,
-                                                       const Tensor2Read<float>& inputs, const f16* adjRows,
-                                                       int rowStride, int channelOffset, const param_t& params)
+    template <typename AdjFn>
+    __device__ __forceinline__ static void scatterTile(int lane, long long index0, long long numel,
+                                                       const Tensor2Read<float>& inputs, const AdjFn& adjOutput,
+                                                       const param_t& params)
     {
         constexpr int G = 2 * F;            // lanes per point
         constexpr int PPR = WAVE_SIZE / G;  // points per round
@@ -444,12 +434,12 @@ struct EncodingHashGrid
 #pragma unroll 1
         for (int round = 0; round < G; ++round) {
             const int pt = round * PPR + lane / G;
-            const int index = index0 + pt;
+            const long long index = index0 + pt;
             if (index >= numel) continue;
             float in[D];
 #pragma unroll
             for (int d = 0; d < D; ++d)
-                in[d] = inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
+                in[d] = inputs.data_[index * inputs.strides_[0]
                                      + static_cast<long long>(d + Cfg::Start) * inputs.strides_[1]];
             float pos[D];
             {
@@ -457,13 +447,12 @@ struct EncodingHashGrid
 #pragma unroll
                 for (int d = 0; d < D; ++d) pos[d] = (in[d] - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
             }
-            const f16* adjRow = adjRows + stageRow(pt) * rowStride + channelOffset;
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 const LevelSetup s = setupLevel(l, pos);
                 const bool hashed = Cfg::hashed[l];
                 const unsigned base = static_cast<unsigned>(Cfg::memoryOffset[l]);
-                const float adj = static_cast<float>(adjRow[(Cfg::Concat ? l * F : 0) + i]);
+                const float adj = adjOutput(pt, (Cfg::Concat ? l * F : 0) + i);
                 // The lanes k = 0 | 1 of a group take the lower | upper corner along the dimension whose
                 // neighbours are close in memory: the last one in a dense level (adjacent entries), the
                 // first one in a hashed level (multiplier 1: the same 64-byte block 7 times out of 8).

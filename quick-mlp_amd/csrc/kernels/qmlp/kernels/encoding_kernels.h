@@ -24,20 +24,30 @@ __global__ void EncodingForwardKernel(
     }
 }
 
-__global__ void EncodingAdjointKernel(
+// One wavefront takes 64 consecutive points at a time: one lane per point for the input
+// gradients, then all lanes together for the parameter gradients of grid encodings (groups
+// of lanes add neighbouring table entries in one atomic request).
+__global__ void __launch_bounds__(256) EncodingAdjointKernel(
     long long numel,
     const Tensor2Read<float> inputs,      //shape (numel, Cin)
     const Tensor2Read<float> adjOutputs,  //shape (numel, Cout)
     Tensor2RW<float> adjInputs            //shape (numel, Cin), accumulated
     $$ENCODING_PARAMETERS$$)
 {
-    for (long long index = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; index < numel;
-         index += static_cast<long long>(blockDim.x) * gridDim.x)
+    const int lane = threadIdx.x % WAVE_SIZE;
+    const long long wavesPerBlock = blockDim.x / WAVE_SIZE;
+    const long long stride = wavesPerBlock * gridDim.x * TILE_POINTS;
+    for (long long tileBase = (blockIdx.x * wavesPerBlock + threadIdx.x / WAVE_SIZE) * TILE_POINTS; tileBase < numel;
+         tileBase += stride)
     {
-        const StridedArray<const float> encodingInput{inputs.data_ + index * inputs.strides_[0], inputs.strides_[1]};
-        const StridedArray<const float> encodingAdjOutput{adjOutputs.data_ + index * adjOutputs.strides_[0], adjOutputs.strides_[1]};
-        StridedArray<float> encodingAdjInput{adjInputs.data_ + index * adjInputs.strides_[0], adjInputs.strides_[1]};
-        $$CALL_ENCODINGS_ADJOINT$$
+        const long long index = tileBase + lane;
+        if (index < numel) {
+            const StridedArray<const float> encodingInput{inputs.data_ + index * inputs.strides_[0], inputs.strides_[1]};
+            const StridedArray<const float> encodingAdjOutput{adjOutputs.data_ + index * adjOutputs.strides_[0], adjOutputs.strides_[1]};
+            StridedArray<float> encodingAdjInput{adjInputs.data_ + index * adjInputs.strides_[0], adjInputs.strides_[1]};
+            $$CALL_ENCODINGS_ADJOINT$$
+        }
+        $$CALL_ENCODINGS_SCATTER$$
     }
 }
 

@@ -451,6 +451,13 @@ int qmlp_encoding_hashgrid_levels(qmlp_encoding_t encoding, int capacity, int* n
     QMLP_API_END
 }
 
+int qmlp_encoding_precompile(qmlp_encoding_t encoding, int adjoint_mode)
+{
+    QMLP_API_BEGIN
+    encoding->encoding->precompile(adjoint_mode);
+    QMLP_API_END
+}
+
 int qmlp_encoding_hashgrid_corners(qmlp_encoding_t encoding, const qmlp_tensor* input, uint32_t* indices,
                                    float* weights, void* stream)
 {

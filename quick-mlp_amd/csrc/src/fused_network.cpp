@@ -551,8 +551,9 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
         callEncodings << ");\n                }\n";
         if (parameterGradients)
             callScatter << "            if constexpr (" << name << "::HasTileScatter)\n                " << name
-                        << "::scatterTile(lane, tile * TILE_POINTS, numel, inputs, sStage, STAGE_STRIDE, "
-                        << encodingOffset << ", cEncoding" << encodingIdx << ");\n";
+                        << "::scatterTile(lane, static_cast<long long>(tile) * TILE_POINTS, numel, inputs,\n"
+                        << "                    [&](int pt, int c) { return static_cast<float>(sStage[stageRow(pt) * STAGE_STRIDE + "
+                        << encodingOffset << " + c]); },\n                    cEncoding" << encodingIdx << ");\n";
         encodingOffset += e->numOutputChannels();
     }
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
@@ -614,38 +615,39 @@ static int loaderFlags(bool compileOnly)
     return flags;
 }
 
-void FusedNetwork::compileInferenceKernel(bool compileOnly)
+void FusedNetwork::compileForwardKernel(bool store, bool narrow, bool compileOnly)
 {
-    if (inferenceKernel_.has_value() && !compileOnly) return;
+    auto& slot = forwardKernels_[store ? 1 : 0][narrow ? 1 : 0];
+    if (slot.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
-    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeInference, false, &ck.pointsPerLane);
+    ck.blockSize = forwardBlockSize(store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference,
+                                    false, &ck.pointsPerLane);
+    if (narrow) ck.pointsPerLane = 1;
     ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
         + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave();
-    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<false>", forwardSource(ck.blockSize, ck.pointsPerLane),
-                           loaderFlags(compileOnly)).value();
+    ck.fun = kl->getKernel(store ? "qmlp::kernel::NetworkKernelInferenceAndForward<true>"
+                                 : "qmlp::kernel::NetworkKernelInferenceAndForward<false>",
+                           forwardSource(ck.blockSize, ck.pointsPerLane), loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
-    QuickMLP::Instance().getLogger()->debug("inference kernel: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
-                                            ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(), ck.fun.scratchBytes(), ck.fullGrid);
-    inferenceKernel_ = std::move(ck);
+    QuickMLP::Instance().getLogger()->debug(
+        "%s kernel, %d tile(s) per wave: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
+        store ? "forward" : "inference", ck.pointsPerLane, ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(),
+        ck.fun.scratchBytes(), ck.fullGrid);
+    slot = std::move(ck);
 }
 
-void FusedNetwork::compileForwardKernel(bool compileOnly)
+const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles)
 {
-    if (forwardKernel_.has_value() && !compileOnly) return;
-    auto kl = QuickMLP::Instance().kernelLoader();
-    CompiledKernel ck;
-    ck.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false, &ck.pointsPerLane);
-    ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
-        + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave();
-    ck.fun = kl->getKernel("qmlp::kernel::NetworkKernelInferenceAndForward<true>", forwardSource(ck.blockSize, ck.pointsPerLane),
-                           loaderFlags(compileOnly)).value();
-    if (compileOnly) return;
-    ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
-    QuickMLP::Instance().getLogger()->debug("forward kernel: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
-                                            ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(), ck.fun.scratchBytes(), ck.fullGrid);
-    forwardKernel_ = std::move(ck);
+    compileForwardKernel(store, false);
+    const auto& wide = forwardKernels_[store ? 1 : 0][0].value();
+    if (wide.pointsPerLane == 1) return wide;
+    // several tiles per wave only pay off once they still fill every compute unit
+    const int waves = wide.blockSize / WARP_SIZE;
+    if (divUp(numTiles, waves * wide.pointsPerLane) >= wide.fullGrid) return wide;
+    compileForwardKernel(store, true);
+    return forwardKernels_[store ? 1 : 0][1].value();
 }
 
 void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
@@ -702,8 +704,12 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
 
 void FusedNetwork::precompile(int adjointFlags)
 {
-    compileInferenceKernel(true);
-    compileForwardKernel(true);
+    for (int store = 0; store < 2; ++store) {
+        compileForwardKernel(store, false, true);
+        int ppl = 1;
+        forwardBlockSize(-1, false, &ppl);
+        if (ppl > 1) compileForwardKernel(store, true, true);
+    }
     if (adjointFlags > 0) compileBackwardKernel(adjointFlags, true);
 }
 
@@ -736,11 +742,9 @@ void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t strea
     CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
     if (numel == 0) return;
 
-    compileInferenceKernel();
-    const auto& ck = inferenceKernel_.value();
-
-    const int waves = ck.blockSize / WARP_SIZE;
     const int numTiles = divUp(numel, TILE_POINTS);
+    const auto& ck = forwardKernelFor(false, numTiles);
+    const int waves = ck.blockSize / WARP_SIZE;
     const int grid = std::min(divUp(numTiles, waves * ck.pointsPerLane), ck.fullGrid);
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
@@ -781,11 +785,9 @@ void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory,
     CHECK_ERROR(tmpMemory != nullptr, "forward() needs temporary memory of forwardMemory() bytes");
     CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemory) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
 
-    compileForwardKernel();
-    const auto& ck = forwardKernel_.value();
-
-    const int waves = ck.blockSize / WARP_SIZE;
     const int numTiles = divUp(numel, TILE_POINTS);
+    const auto& ck = forwardKernelFor(true, numTiles);
+    const int waves = ck.blockSize / WARP_SIZE;
     const int grid = std::min(divUp(numTiles, waves * ck.pointsPerLane), ck.fullGrid);
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
@@ -931,8 +933,8 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
 
 void FusedNetwork::clearCachedKernels()
 {
-    inferenceKernel_ = {};
-    forwardKernel_ = {};
+    for (auto& perStore : forwardKernels_)
+        for (auto& k : perStore) k = {};
     for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i) backwardKernel_[i] = {};
 }
 

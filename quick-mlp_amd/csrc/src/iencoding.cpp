@@ -1,6 +1,7 @@
 #include <qmlp/iencoding.h>
 
 #include <qmlp/encoding_hashgrid.h>
+#include <qmlp/encoding_line_integration.h>
 #include <qmlp/encoding_identity.h>
 #include <qmlp/qmlp.h>
 
@@ -18,7 +19,7 @@ struct ArgPack
 };
 
 std::string standaloneSource(const IEncoding& e, const std::string& callForward, const std::string& callAdjoint,
-                             const std::string& callCorners = "")
+                             const std::string& callCorners = "", const std::string& callScatter = "")
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string codeTemplate = kl->findFile("qmlp/kernels/encoding_kernels.h").value();
@@ -31,10 +32,49 @@ std::string standaloneSource(const IEncoding& e, const std::string& callForward,
     replaceAll(codeTemplate, "$$CALL_ENCODINGS_FORWARD$$", callForward);
     replaceAll(codeTemplate, "$$CALL_ENCODINGS_ADJOINT$$", callAdjoint);
     replaceAll(codeTemplate, "$$CALL_ENCODINGS_CORNERS$$", callCorners);
+    replaceAll(codeTemplate, "$$CALL_ENCODINGS_SCATTER$$", callScatter);
     return codeTemplate;
 }
 
 } // namespace
+
+std::string IEncoding::forwardKernelSource() const
+{
+    std::stringstream call;
+    call << qualifiedName() << "::forward(encodingInput, encodingOutput";
+    if (hasParameters()) call << ", cEncoding";
+    call << ");\n";
+    return standaloneSource(*this, call.str(), "");
+}
+
+std::string IEncoding::adjointKernelSource(int adjointMode) const
+{
+    const bool hasInputGradients = adjointMode & INPUT_GRADIENTS;
+    const bool hasParamGradients = (adjointMode & PARAM_GRADIENTS) && hasParameters();
+    // encodings with a tile-wide scatter take their parameter gradients out of the per-point call
+    std::stringstream call, scatter;
+    call << qualifiedName() << "::template adjoint<" << (hasInputGradients ? "true" : "false") << ", "
+         << (hasParamGradients ? "!" + qualifiedName() + "::HasTileScatter" : std::string("false"))
+         << ">(encodingInput, encodingAdjOutput, encodingAdjInput";
+    if (hasParameters()) call << ", cEncoding";
+    call << ");\n";
+    if (hasParamGradients)
+        scatter << "if constexpr (" << qualifiedName() << "::HasTileScatter)\n            " << qualifiedName()
+                << "::scatterTile(lane, tileBase, numel, inputs, [&](int pt, int c) { return adjOutputs.data_[(tileBase + pt)"
+                   " * adjOutputs.strides_[0] + static_cast<long long>(c) * adjOutputs.strides_[1]]; }, cEncoding);\n";
+    return standaloneSource(*this, "", call.str(), "", scatter.str());
+}
+
+void IEncoding::precompile(int adjointMode)
+{
+    auto kl = QuickMLP::Instance().kernelLoader();
+    const int flags = QuickMLP::Instance().getCompileFlags() | KernelLoader::CompileOnly;
+    kl->getKernel("qmlp::kernel::EncodingForwardKernel", forwardKernelSource(), flags);
+    if (adjointMode > 0) {
+        CHECK_ERROR(adjointMode <= ALL_GRADIENTS, "Illegal adjoint mode");
+        kl->getKernel("qmlp::kernel::EncodingAdjointKernel", adjointKernelSource(adjointMode), flags);
+    }
+}
 
 void IEncoding::forward(const Tensor& input, Tensor& output, stream_t stream,
                         const std::optional<const Tensor>& parametersForward)
@@ -50,15 +90,9 @@ void IEncoding::forward(const Tensor& input, Tensor& output, stream_t stream,
     long long numel = input.size(0);
     if (numel == 0) return;
 
-    if (!forwardKernel_.has_value()) {
-        std::stringstream call;
-        call << qualifiedName() << "::forward(encodingInput, encodingOutput";
-        if (hasParameters()) call << ", cEncoding";
-        call << ");\n";
-        std::string source = standaloneSource(*this, call.str(), "");
+    if (!forwardKernel_.has_value())
         forwardKernel_ = QuickMLP::Instance().kernelLoader()->getKernel(
-            "qmlp::kernel::EncodingForwardKernel", source, QuickMLP::Instance().getCompileFlags()).value();
-    }
+            "qmlp::kernel::EncodingForwardKernel", forwardKernelSource(), QuickMLP::Instance().getCompileFlags()).value();
     auto& fun = forwardKernel_.value();
 
     std::vector<char> paramBytes(4096);
@@ -98,18 +132,10 @@ void IEncoding::adjoint(const Tensor& input, const Tensor& adjOutput, Tensor& ad
     long long numel = input.size(0);
     if (numel == 0) return;
 
-    if (!adjointKernel_[adjointMode].has_value()) {
-        const bool hasInputGradients = adjointMode & INPUT_GRADIENTS;
-        const bool hasParamGradients = (adjointMode & PARAM_GRADIENTS) && hasParameters();
-        std::stringstream call;
-        call << qualifiedName() << "::template adjoint<" << (hasInputGradients ? "true" : "false") << ", "
-             << (hasParamGradients ? "true" : "false") << ">(encodingInput, encodingAdjOutput, encodingAdjInput";
-        if (hasParameters()) call << ", cEncoding";
-        call << ");\n";
-        std::string source = standaloneSource(*this, "", call.str());
+    if (!adjointKernel_[adjointMode].has_value())
         adjointKernel_[adjointMode] = QuickMLP::Instance().kernelLoader()->getKernel(
-            "qmlp::kernel::EncodingAdjointKernel", source, QuickMLP::Instance().getCompileFlags()).value();
-    }
+            "qmlp::kernel::EncodingAdjointKernel", adjointKernelSource(adjointMode),
+            QuickMLP::Instance().getCompileFlags()).value();
     auto& fun = adjointKernel_[adjointMode].value();
 
     std::vector<char> paramBytes(4096);
@@ -162,6 +188,7 @@ EncodingFactory::EncodingFactory()
 {
     encodings_[EncodingIdentity::ID()] = [](const json& cfg) { return std::make_shared<EncodingIdentity>(cfg); };
     encodings_[EncodingHashGrid::ID()] = [](const json& cfg) { return std::make_shared<EncodingHashGrid>(cfg); };
+    encodings_[EncodingLineIntegration::ID()] = [](const json& cfg) { return std::make_shared<EncodingLineIntegration>(cfg); };
 }
 
 EncodingFactory& EncodingFactory::Instance()

@@ -195,6 +195,10 @@ class Encoding:
         check(lib.qmlp_encoding_set_parameter(self._handle, desc(tensor),
                                               QMLP_GRADIENTS if gradients else QMLP_INFERENCE))
 
+    def precompile(self, adjoint_mode=3):
+        """Compiles the standalone kernels into the kernel cache (needs no GPU)."""
+        check(lib.qmlp_encoding_precompile(self._handle, int(adjoint_mode)))
+
     def hashgrid_levels(self):
         """[(resolution, hashed, memory_offset, hash_grid_size)] of a HashGrid encoding."""
         n = ctypes.c_int()

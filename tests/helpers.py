@@ -15,8 +15,17 @@ REL, ABS = 1e-2, 1e-3          # tolerance of the fp16 path against the fp32 ora
 FLAG_INPUT, FLAG_WEIGHTS, FLAG_ENC = 1, 2, 4
 
 
-def require_gpu():
-    """For tests that do not go through Case: nothing to do in a CPU cache-warming pass."""
+def require_gpu(encoding_cfg=None, adjoint_modes=(3,)):
+    """For tests that do not go through Case. In a CPU cache-warming pass the standalone
+    kernels of encoding_cfg are compiled into the in-tree kernel cache, then the test stops."""
+    if os.environ.get("QMLP_WARM_CACHE") and encoding_cfg is not None:
+        import json
+        import qmlp
+        enc = qmlp.Encoding(json.dumps(encoding_cfg))
+        enc.precompile(0)
+        for m in adjoint_modes:
+            enc.precompile(m)
+        pytest.skip("kernel cache warmed")
     if not torch.cuda.is_available():
         pytest.skip("no GPU in this environment")
 

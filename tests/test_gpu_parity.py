@@ -193,10 +193,10 @@ def test_grid_indices_are_bit_exact(spec):
 @pytest.mark.parametrize("spec", GRID_SPECS)
 @pytest.mark.parametrize("precision", ["float", "half"])
 def test_standalone_grid_encoding(spec, precision):
-    require_gpu()
     import json
     import qmlp
     cfg = _grid_cfg(spec, precision, start=1)
+    require_gpu(cfg)
     enc = qmlp.Encoding(json.dumps(cfg))
     g = qo.HashGrid(cfg)
     rng = np.random.default_rng(3)
@@ -223,13 +223,13 @@ def test_standalone_grid_encoding(spec, precision):
 def test_dense_grid_against_grid_sample(dim):
     """The reference's encoding tests (tests_py/qmlp_tests/test_encoding.py:123-188): a dense
     grid of resolution 2 with 4 features on [-1,1]^D equals torch grid_sample."""
-    require_gpu()
     import json
     import qmlp
     R, C = 2, 4
     cfg = {"id": "HashGrid", "start_in": 0, "n_in": dim, "n_levels": 1, "n_features_per_level": C,
            "log2_hashmap_size": -1, "min_resolution": R, "max_resolution": 16, "combination_mode": "add",
            "bounding_box_min": [-1] * dim, "bounding_box_size": [2] * dim}
+    require_gpu(cfg)
     enc = qmlp.FusedEncoding(json.dumps(cfg))
     torch.manual_seed(0)
     params = enc.create_parameter_tensor().requires_grad_(True)
@@ -282,6 +282,78 @@ def test_fused_grid_network_against_oracle(precision):
     got_e = case.gpu_train(X, adj, FLAG_ENC)
     check_gradients(case, X, adj, FLAG_ENC, got_e, what="alone: ")
     assert got_e["adj_x"] is None and got_e["grads"] is None
+
+
+# ---------------------------------------------------------------------------- line integration
+def _line_cfg(blending, precision="float", start=0):
+    child = {"id": "HashGrid", "start_in": 0, "n_in": 3, "n_levels": 4, "n_features_per_level": 2,
+             "log2_hashmap_size": 10, "min_resolution": 4, "max_resolution": 40, "combination_mode": "concat",
+             "bounding_box_min": [-1.0, -1.0, -0.5], "bounding_box_size": [2.0, 2.0, 1.0],
+             "parameter_precision": precision}
+    return {"id": "LineIntegration", "start_in": start, "n_in": 3, "volume": child, "stepsize": 0.13,
+            "blending": blending}
+
+
+def _rays(rng, N, lead=0):
+    start = rng.uniform(-2.5, 2.5, (N, 3))
+    target = rng.uniform(-0.9, 0.9, (N, 3)) * np.array([1.0, 1.0, 0.5])
+    d = target - start
+    d /= np.linalg.norm(d, axis=1, keepdims=True)
+    X = np.concatenate([rng.uniform(-1, 1, (N, lead)), start, d], 1).astype(np.float32)
+    X[0, lead:] = [0.2, -3.0, 0.1, 0.0, 1.0, 0.0]          # zero direction components
+    X[1, lead:] = [5.0, 5.0, 5.0, 1.0, 0.0, 0.0]           # misses the box
+    X[2, lead:] = [0.1, 0.2, 0.0, 0.6, 0.0, 0.8]           # starts inside
+    return X
+
+
+@pytest.mark.parametrize("blending", ["additive", "average"])
+def test_standalone_line_integration(blending):
+    """Ray marching through a child grid (tests_cpp/test_hashgrid.cpp:68-150 of the reference only
+    prints its results; here the device is compared with the oracle's march)."""
+    import json
+    import qmlp
+    cfg = _line_cfg(blending, start=1)
+    require_gpu(cfg)
+    enc = qmlp.Encoding(json.dumps(cfg))
+    li = qo.LineIntegration(cfg)
+    assert enc.num_output_channels() == li.num_outputs == 8 and enc.max_input_channel() == 6
+    assert enc.num_parameters() == li.n_params
+    rng = np.random.default_rng(21)
+    N = 2000
+    X = _rays(rng, N, lead=1)
+    table = rng.standard_normal(li.n_params).astype(np.float32)
+    x, t = torch.from_numpy(X).cuda(), torch.from_numpy(table).cuda()
+    out = enc.inference_with_parameter(x, t).cpu().numpy()
+    want = li.forward(table, X)
+    assert np.all(out[1] == 0) and np.abs(want).max() > 1
+    assert_close(out, want, "line integration forward", rel=1e-4, abs_=1e-4)
+    adj = rng.standard_normal((N, li.num_outputs)).astype(np.float32)
+    ax, gp = enc.adjoint_with_parameter(x, t, torch.from_numpy(adj).cuda())
+    ref_ax, ref_gp = li.adjoint(table, X, adj, res_factor=1)
+    s = float(np.abs(ref_ax).max())
+    assert_close(ax.cpu().numpy() / s, ref_ax / s, "line integration input gradients", rel=1e-3, abs_=1e-4)
+    s = float(np.abs(ref_gp).max())
+    assert_close(gp.cpu().numpy() / s, ref_gp / s, "line integration table gradients", rel=1e-3, abs_=1e-4)
+
+
+def test_fused_network_with_line_integration():
+    line = _line_cfg("average", "half", start=0)
+    cfg = {"num_inputs": 6, "num_outputs": 2, "activation_specification": ["qmlp/builtin-activations.json"],
+           "encodings": [line],
+           "network": [{"n_out": 32, "bias": True, "activation": "celu"},
+                       {"n_out": 2, "bias": False, "activation": "identity"}]}
+    case = Case(cfg)
+    rng = np.random.default_rng(23)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    case.set_table(0, rng.uniform(-1, 1, case.oracle.encodings[0][1].n_params))
+    N = 3000
+    X = _rays(rng, N)
+    adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+    assert_close(case.gpu_inference(X), case.oracle.forward(X), "inference")
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    got = case.gpu_train(X, adj, flags)
+    assert_close(got["out"], case.oracle.forward(X), "forward")
+    check_gradients(case, X, adj, flags, got)
 
 
 # ---------------------------------------------------------------------------- BASELINE configurations

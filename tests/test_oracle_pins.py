@@ -508,3 +508,180 @@ def test_round_mode_one_stays_close_to_fp32():
     frac, worst = qo.compare(b, a, 1e-2, 1e-3)
     assert frac == 0.0
     assert not np.array_equal(a, b)
+
+
+# ------------------------------------------------------------------ line integration
+def line_spec(child, stepsize=0.25, blending="additive", start=0):
+    return {"id": "LineIntegration", "start_in": start, "n_in": 3, "volume": child, "stepsize": stepsize,
+            "blending": blending}
+
+
+def slab_interval(start, direction, bmin, bsize):
+    """Independent float64 slab test (zero direction components: the slab does not bound t)."""
+    lo, hi = -np.inf, np.inf
+    for d in range(3):
+        if direction[d] == 0:
+            assert bmin[d] <= start[d] <= bmin[d] + bsize[d]
+            continue
+        ta = (bmin[d] - start[d]) / direction[d]
+        tb = (bmin[d] + bsize[d] - start[d]) / direction[d]
+        lo, hi = max(lo, min(ta, tb)), min(hi, max(ta, tb))
+    return lo, hi
+
+
+def test_line_integration_known_answer_axis_aligned_ray():
+    """Box [-1,1]^3, ray from (-2,0.1,0.2) along +x: inside for t in [1,3); with a step of 0.25
+    the march samples t = 1, 1.25, .., 2.75: 8 samples, floor(2/0.25) = 8 steps. A constant
+    table c (partition of unity) therefore gives 8c when summing and c when averaging."""
+    child = grid_spec(3, levels=2, feat=2, log2=6, rmin=3, rmax=9, bmin=[-1.0] * 3, bsize=[2.0] * 3)
+    x = np.array([[-2.0, 0.1, 0.2, 1.0, 0.0, 0.0]], np.float32)
+    for blending, want in (("additive", 8 * 0.375), ("average", 0.375)):
+        li = qo.LineIntegration(line_spec(child, 0.25, blending))
+        table = np.full(li.n_params, 0.375, np.float32)
+        out = li.forward(table, x)
+        assert out.shape == (1, 4)
+        assert np.allclose(out, want, rtol=1e-6, atol=0)
+
+
+def test_line_integration_misses_and_rays_starting_inside():
+    child = grid_spec(3, levels=1, feat=1, rmin=4, rmax=4, bmin=[-1.0] * 3, bsize=[2.0] * 3)
+    li = qo.LineIntegration(line_spec(child, 0.3, "additive"))
+    table = np.full(li.n_params, 2.0, np.float32)
+    # passes beside the box: no sample
+    miss = np.array([[-2.0, 3.0, 0.0, 1.0, 0.0, 0.0]], np.float32)
+    assert np.all(li.forward(table, miss) == 0)
+    # starts at the centre: the march begins at the (negative) entry parameter, as in the reference
+    inside = np.array([[0.0, 0.0, 0.0, 0.0, 0.0, 1.0]], np.float32)
+    lo, hi = slab_interval(inside[0, :3].astype(np.float64), inside[0, 3:].astype(np.float64), [-1.0] * 3, [2.0] * 3)
+    assert (lo, hi) == (-1.0, 1.0)
+    count = len([k for k in range(100) if lo + k * 0.3 < hi])      # 7 samples: -1, -0.7, .., 0.8
+    assert count == 7
+    assert np.allclose(li.forward(table, inside), 2.0 * count, rtol=1e-6)
+
+
+def test_line_integration_of_a_linear_field_has_a_closed_form():
+    """A dense level whose node values are an affine function of the node position interpolates
+    that function exactly, so the sum over the samples t_k = tmin + k h is
+    n (a.start + b) + (a.dir) sum t_k."""
+    R = 5
+    bmin, bsize = np.array([-1.0, -0.5, 0.0]), np.array([2.0, 1.5, 1.0])
+    child = grid_spec(3, levels=1, feat=1, rmin=R, rmax=R, bmin=list(bmin), bsize=list(bsize))
+    h = 0.07
+    a, b = np.array([0.3, -0.7, 1.1]), 0.25
+    li = qo.LineIntegration(line_spec(child, h, "additive", start=1))
+    nodes = np.stack(np.meshgrid(*[np.arange(R)] * 3, indexing="ij"), -1).reshape(-1, 3)   # last coordinate fastest
+    table = (bmin + bsize * nodes / (R - 1)) @ a + b
+    rng = np.random.default_rng(5)
+    rays = []
+    while len(rays) < 20:
+        start = bmin + bsize * rng.uniform(-0.5, 1.5, 3)
+        target = bmin + bsize * rng.uniform(0.2, 0.8, 3)
+        d = (target - start) / np.linalg.norm(target - start)
+        lo, hi = slab_interval(start, d, bmin, bsize)
+        frac = ((hi - lo) / h) % 1.0
+        if hi > lo and 0.2 < frac < 0.8:        # the number of samples is not a rounding matter
+            rays.append(np.concatenate([[9.0], start, d]))
+    X = np.array(rays, np.float32)
+    out = li.forward(table.astype(np.float32), X)[:, 0]
+    for n, ray in enumerate(X.astype(np.float64)):
+        start, d = ray[1:4], ray[4:7]
+        lo, hi = slab_interval(start, d, bmin, bsize)
+        t = lo + h * np.arange(int(np.ceil((hi - lo) / h)))
+        want = len(t) * (a @ start + b) + (a @ d) * t.sum()
+        assert abs(out[n] - want) < 2e-4 * max(1.0, abs(want)), (n, out[n], want)
+
+
+def _line_samples(li, cfg_child, ray):
+    """The sample parameters and positions of one ray in the fp32 arithmetic of the march
+    (entry parameter by an fp32 slab test, t += h in fp32, fused multiply-add positions)."""
+    f = np.float32
+    start, d = ray[li.start_in:li.start_in + 3].astype(f), ray[li.start_in + 3:li.start_in + 6].astype(f)
+    bmin, bsize = np.array(cfg_child["bounding_box_min"], f), np.array(cfg_child["bounding_box_size"], f)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        inv = f(1) / d
+        ta, tb = (bmin - start) * inv, ((bmin + bsize) - start) * inv
+    tmin, tmax = np.fmax.reduce(np.fmin(ta, tb)), np.fmin.reduce(np.fmax(ta, tb))
+    ts, t = [], tmin
+    while t < tmax:
+        ts.append(t)
+        t = f(t + f(li.stepsize))
+    ts = np.array(ts, f)
+    pos = (ts.astype(np.float64)[:, None] * d.astype(np.float64) + start.astype(np.float64)).astype(f)  # one rounding = fma
+    steps = int(np.floor(f(f(tmax - tmin) / f(li.stepsize)))) if len(ts) else 0
+    return ts, pos, steps
+
+
+@pytest.mark.parametrize("blending", ["additive", "average"])
+def test_line_integration_is_the_sum_of_the_pinned_grid_over_the_samples(blending):
+    """Forward, input gradients (tmin/tmax constant, as in the reference) and table gradients
+    equal the sums over explicitly generated sample positions of the separately pinned grid
+    forward / adjoint."""
+    child = grid_spec(3, levels=3, feat=2, log2=9, rmin=4, rmax=32, bmin=[-1.0, -1.0, -1.0], bsize=[2.0, 2.0, 2.0])
+    li = qo.LineIntegration(line_spec(child, 0.11, blending, start=1))
+    g = qo.HashGrid(child)
+    rng = np.random.default_rng(11)
+    table = rng.standard_normal(g.n_params).astype(np.float32)
+    N = 40
+    start = rng.uniform(-2, 2, (N, 3))
+    target = rng.uniform(-0.8, 0.8, (N, 3))
+    d = target - start
+    d /= np.linalg.norm(d, axis=1, keepdims=True)
+    X = np.concatenate([np.zeros((N, 1)), start, d], 1).astype(np.float32)
+    X[0, 4:7] = [0.0, 1.0, 0.0]; X[0, 1:4] = [0.3, -2.0, 0.1]       # a zero direction component
+    adj = rng.standard_normal((N, g.num_outputs)).astype(np.float32)
+    out = li.forward(table, X)
+    adj_x, grad = li.adjoint(table, X, adj)
+    want_grad = np.zeros(g.n_params, np.float64)
+    for n in range(N):
+        ts, pos, steps = _line_samples(li, child, X[n])
+        scale = 1.0 / steps if (blending == "average" and steps > 0) else 1.0
+        assert len(ts) > 3
+        feats = g.forward(table, pos).astype(np.float64)
+        assert np.allclose(out[n], feats.sum(0) * scale, rtol=2e-5, atol=2e-5)
+        a_rep = np.repeat((adj[n] * np.float32(scale))[None], len(ts), 0)
+        ap, gp = g.adjoint(table, pos, a_rep)
+        assert np.allclose(adj_x[n, 1:4], ap.astype(np.float64).sum(0), rtol=1e-4, atol=1e-3)
+        assert np.allclose(adj_x[n, 4:7], (ap.astype(np.float64) * ts[:, None]).sum(0), rtol=1e-4, atol=1e-3)
+        assert adj_x[n, 0] == 0
+        want_grad += gp
+    assert np.allclose(grad, want_grad, rtol=1e-4, atol=1e-4)
+
+
+def test_line_integration_table_gradient_is_the_transpose_of_forward():
+    child = grid_spec(3, levels=2, feat=2, log2=8, rmin=3, rmax=20, bmin=[0.0] * 3, bsize=[1.0] * 3)
+    li = qo.LineIntegration(line_spec(child, 0.05, "average"))
+    rng = np.random.default_rng(2)
+    N = 64
+    start = rng.uniform(-0.5, 1.5, (N, 3))
+    d = rng.uniform(0.2, 0.8, (N, 3)) - start
+    X = np.concatenate([start, d / np.linalg.norm(d, axis=1, keepdims=True)], 1).astype(np.float32)
+    theta = rng.standard_normal(li.n_params).astype(np.float32)
+    v = rng.standard_normal((N, li.num_outputs)).astype(np.float32)
+    lhs = float((li.forward(theta, X).astype(np.float64) * v).sum())
+    _, grad = li.adjoint(np.zeros_like(theta), X, v, input_grads=False)
+    rhs = float((grad.astype(np.float64) * theta).sum())
+    assert abs(lhs - rhs) < 1e-4 * max(1.0, abs(lhs))
+
+
+def test_fused_network_with_line_integration_is_the_composition():
+    child = grid_spec(3, levels=2, feat=2, log2=8, rmin=3, rmax=20, bmin=[-1.0] * 3, bsize=[2.0] * 3)
+    line = line_spec(child, 0.2, "average")
+    cfg = {"num_inputs": 6, "num_outputs": 2, "activation_specification": [],
+           "encodings": [line],
+           "network": [{"n_out": 16, "bias": True, "activation": "relu"},
+                       {"n_out": 2, "bias": False, "activation": "identity"}]}
+    net = qo.Network(cfg)
+    li = qo.LineIntegration(line)
+    rng = np.random.default_rng(4)
+    table = rng.standard_normal(li.n_params).astype(np.float32)
+    params = (rng.standard_normal(net.num_parameters) * 0.3).astype(np.float32)
+    net.set_parameters(params)
+    net.set_table(0, table)
+    N = 30
+    start = rng.uniform(-2, 2, (N, 3))
+    d = rng.uniform(-0.5, 0.5, (N, 3)) - start
+    X = np.concatenate([start, d / np.linalg.norm(d, axis=1, keepdims=True)], 1).astype(np.float32)
+    enc = li.forward(table, X)
+    W0, b0, W1 = net.weight(0)[:, :4], net.bias(0), net.weight(1)[:2]
+    want = np.maximum(enc @ W0.T + b0, 0) @ W1.T
+    assert np.allclose(net.forward(X), want, rtol=1e-4, atol=1e-5)
