@@ -321,6 +321,17 @@ static void line_intersect(const qo_line* line, const float* start, const float*
     *tmax = fminf(fminf(hi[0], hi[1]), hi[2]);
 }
 
+/* Steps in [tmin, tmax), or -2 (steps + 2 iterations are none) for rays that take no sample. Deliberate difference to the
+ * reference, whose loop (encoding_line_integration.cuh:81) does not end for them: the
+ * interval must be finite and hold fewer than 2^20 steps; the loops below also stop after
+ * steps + 2 iterations. */
+static int line_num_steps(float tmin, float tmax, float stepsize)
+{
+    const float steps = floorf((tmax - tmin) / stepsize);
+    if (!(fabsf(tmin) < INFINITY && fabsf(tmax) < INFINITY) || !(steps < 1048576.f)) return -2;
+    return (int)steps;
+}
+
 static void line_forward_point(const qo_line* line, const qo_hashgrid* child, const float* table,
                                const float* x, float* out)
 {
@@ -329,9 +340,10 @@ static void line_forward_point(const qo_line* line, const qo_hashgrid* child, co
     const float* dir = start + 3;
     float tmin, tmax, contribution[QO_MAX_LEVELS * 16], pos[3];
     line_intersect(line, start, dir, &tmin, &tmax);
-    const int steps = (int)floorf((tmax - tmin) / line->stepsize);
+    const int steps = line_num_steps(tmin, tmax, line->stepsize);
+    int it = 0;
     for (int i = 0; i < C; ++i) out[i] = 0.f;
-    for (float t = tmin; t < tmax; t += line->stepsize) {
+    for (float t = tmin; t < tmax && it < steps + 2; t += line->stepsize, ++it) {
         for (int d = 0; d < 3; ++d) pos[d] = fmaf(t, dir[d], start[d]);
         hashgrid_forward_point(child, table, pos, contribution);
         for (int i = 0; i < C; ++i) out[i] += contribution[i];
@@ -353,11 +365,12 @@ static void line_adjoint_point(const qo_line* line, const qo_hashgrid* child, co
     float tmin, tmax, adj_accu[QO_MAX_LEVELS * 16], pos[3], adj_pos[3];
     float adj_start[3] = {0.f, 0.f, 0.f}, adj_dir[3] = {0.f, 0.f, 0.f};
     line_intersect(line, start, dir, &tmin, &tmax);
-    const int steps = (int)floorf((tmax - tmin) / line->stepsize);
+    const int steps = line_num_steps(tmin, tmax, line->stepsize);
+    int it = 0;
     float scale = 1.0f;
     if (line->blending == QO_BLEND_AVERAGE) scale = steps > 0 ? 1.0f / (float)steps : 1.0f;
     for (int i = 0; i < C; ++i) adj_accu[i] = scale * adj_out[i];
-    for (float t = tmin; t < tmax; t += line->stepsize) {
+    for (float t = tmin; t < tmax && it < steps + 2; t += line->stepsize, ++it) {
         for (int d = 0; d < 3; ++d) { pos[d] = fmaf(t, dir[d], start[d]); adj_pos[d] = 0.f; }
         hashgrid_adjoint_point(child, table, pos, adj_accu, adj_x ? adj_pos : NULL, grad_table,
                                res_factor, atomic);

@@ -38,7 +38,9 @@
  * Deliberate divergence from the reference: the grid input gradient includes
  * the (resolution-1) chain-rule factor the reference omits
  * (encoding_hashgrid.cuh:232,238,414-420); pass res_factor=0 to get the
- * reference's formula.
+ * reference's formula. The line integration takes no sample for rays whose
+ * parameter interval is unbounded or holds 2^20 steps or more, where the
+ * reference's loop would not end.
  */
 #ifndef QMLP_ORACLE_H
 #define QMLP_ORACLE_H

@@ -9,6 +9,12 @@
 // (which is negative if the ray starts inside the box) in steps of `stepsize` while
 // t < tmax; "average" divides by floor((tmax-tmin)/stepsize) if that is positive; the
 // adjoint treats tmin/tmax as constants.
+//
+// Difference to the reference, on purpose: its loop `for (t = tmin; t < tmax; t += h)` never
+// ends when the interval is unbounded (a zero direction vector gives tmin = -inf) or when h
+// is below the spacing of floats at t. Here a ray takes no sample at all unless tmin and
+// tmax are finite and the interval holds fewer than 2^20 steps, and the loop also counts
+// its iterations (at most steps + 2), so every wavefront leaves the march.
 
 #include <qmlp/kernels/common.h>
 #include <qmlp/kernels/arrays.h>
@@ -68,6 +74,18 @@ struct EncodingLineIntegration
         tmax = fminf(fminf(hi[0], hi[1]), hi[2]);
     }
 
+    static constexpr float MaxSteps = 1048576.f;
+
+    /** Number of steps in [tmin, tmax); -2 (so that steps + 2 iterations are none) if the ray
+     *  takes no sample, see the file header. */
+    __device__ __forceinline__ static int numSteps(float tmin, float tmax, float stepsize)
+    {
+        const float steps = floorf((tmax - tmin) / stepsize);
+        const bool bounded = fabsf(tmin) < __builtin_inff() && fabsf(tmax) < __builtin_inff();
+        if (!bounded || !(steps < MaxSteps)) return -2;
+        return static_cast<int>(steps);
+    }
+
     template <typename I>
     __device__ __forceinline__ static void readRay(const I& input, position_t& rayStart, position_t& rayDir)
     {
@@ -86,12 +104,13 @@ struct EncodingLineIntegration
         readRay(input, rayStart, rayDir);
         float tmin, tmax;
         intersect(rayStart, rayDir, params, tmin, tmax);
-        const int steps = static_cast<int>(floorf((tmax - tmin) / params.stepsize));
+        const int steps = numSteps(tmin, tmax, params.stepsize);
 
         feature_t accu;
 #pragma unroll
         for (int i = 0; i < NumOutputs; ++i) accu[i] = 0.f;
-        for (float t = tmin; t < tmax; t += params.stepsize) {
+        int iteration = 0;
+        for (float t = tmin; t < tmax && iteration < steps + 2; t += params.stepsize, ++iteration) {
             position_t position;
 #pragma unroll
             for (int d = 0; d < D; ++d) position[d] = fmaf(t, rayDir[d], rayStart[d]);
@@ -127,7 +146,7 @@ struct EncodingLineIntegration
         readRay(input, rayStart, rayDir);
         float tmin, tmax;
         intersect(rayStart, rayDir, params, tmin, tmax);
-        const int steps = static_cast<int>(floorf((tmax - tmin) / params.stepsize));
+        const int steps = numSteps(tmin, tmax, params.stepsize);
 
         float scale = 1.0f;
         if constexpr (Blending == LineIntegrationBlendingMode::AVERAGE)
@@ -139,7 +158,8 @@ struct EncodingLineIntegration
         position_t adjRayStart, adjRayDir;
 #pragma unroll
         for (int d = 0; d < D; ++d) adjRayStart[d] = adjRayDir[d] = 0.f;
-        for (float t = tmin; t < tmax; t += params.stepsize) {
+        int iteration = 0;
+        for (float t = tmin; t < tmax && iteration < steps + 2; t += params.stepsize, ++iteration) {
             position_t position, adjPosition;
 #pragma unroll
             for (int d = 0; d < D; ++d) {

@@ -5,6 +5,7 @@
 #include <qmlp/encoding_identity.h>
 #include <qmlp/qmlp.h>
 
+#include <cctype>
 #include <cstring>
 
 QUICKMLP_NAMESPACE_BEGIN
@@ -197,10 +198,23 @@ EncodingFactory& EncodingFactory::Instance()
     return INSTANCE;
 }
 
+static std::string lowerCase(std::string s)
+{
+    for (auto& c : s) c = static_cast<char>(std::tolower(static_cast<unsigned char>(c)));
+    return s;
+}
+
 IEncoding_ptr EncodingFactory::create(const json& cfg)
 {
     const std::string id = cfg.at("id").get<std::string>();
     auto it = encodings_.find(id);
+    if (it == encodings_.end()) {
+        // The reference matches the id exactly, but its own sample specifications write
+        // "identity" for "Identity" (network_configs/test1.json:9, README.md:76): match
+        // without regard to case.
+        for (auto jt = encodings_.begin(); jt != encodings_.end(); ++jt)
+            if (lowerCase(jt->first) == lowerCase(id)) it = jt;
+    }
     if (it == encodings_.end()) throw configuration_error("No encoding with id '%s' found", id.c_str());
     return it->second(cfg);
 }

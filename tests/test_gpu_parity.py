@@ -303,6 +303,7 @@ def _rays(rng, N, lead=0):
     X[0, lead:] = [0.2, -3.0, 0.1, 0.0, 1.0, 0.0]          # zero direction components
     X[1, lead:] = [5.0, 5.0, 5.0, 1.0, 0.0, 0.0]           # misses the box
     X[2, lead:] = [0.1, 0.2, 0.0, 0.6, 0.0, 0.8]           # starts inside
+    X[3, lead:] = [0.1, 0.2, 0.0, 0.0, 0.0, 0.0]           # no direction: unbounded interval, no sample
     return X
 
 

@@ -11,6 +11,7 @@ import sys
 
 import numpy as np
 import pytest
+import torch
 
 import qmlp
 import qmlp_oracle as qo
@@ -240,3 +241,40 @@ def test_activation_objects():
     assert json.loads(b.to_json())["forward"] == bc.SINE30["forward"]
     with pytest.raises(qmlp.QmlpError, match="No activation with id"):
         qmlp.Activation("swish")
+
+
+def test_encoding_ids_ignore_case_like_the_reference_samples():
+    """network_configs/test1.json:9 and README.md:76 of the reference write "identity"."""
+    e = qmlp.Encoding(json.dumps({"id": "identity", "start_in": 1, "n_in": 2}))
+    assert json.loads(e.to_json())["id"] == "Identity" and e.max_input_channel() == 2
+    g = qmlp.Encoding(json.dumps(dict(bc.hashgrid3d("float"), id="hashgrid")))
+    assert json.loads(g.to_json())["id"] == "HashGrid"
+    with pytest.raises(qmlp.QmlpError, match="No encoding with id 'Fourier'"):
+        qmlp.Encoding(json.dumps({"id": "Fourier", "start_in": 0, "n_in": 3}))
+
+
+def test_line_integration_host_side():
+    child = dict(bc.hashgrid3d("half"), n_levels=2, log2_hashmap_size=8, max_resolution=32, start_in=5, n_in=3,
+                 bounding_box_min=[-1, -1, -1], bounding_box_size=[2, 2, 2])
+    cfg = {"id": "LineIntegration", "start_in": 2, "n_in": 3, "volume": child, "stepsize": 0.05, "blending": "average"}
+    e = qmlp.Encoding(json.dumps(cfg))
+    back = json.loads(e.to_json())
+    assert back["blending"] == "average" and back["start_in"] == 2 and abs(back["stepsize"] - 0.05) < 1e-7
+    assert back["volume"]["start_in"] == 0 and back["volume"]["n_in"] == 3      # the child reads the sample position
+    assert e.max_input_channel() == 2 + 6 - 1                                   # ray start + direction
+    assert e.num_output_channels() == 4 and e.has_parameters()
+    assert e.num_parameters() == qmlp.Encoding(json.dumps(child)).num_parameters()
+    assert e.parameter_dtype() == torch.float16
+    with pytest.raises(qmlp.QmlpError, match="only defined for 3D"):
+        qmlp.Encoding(json.dumps(dict(cfg, n_in=2, volume=dict(child, bounding_box_min=[0, 0], bounding_box_size=[1, 1]))))
+    with pytest.raises(qmlp.QmlpError, match="Stepsize must be positive"):
+        qmlp.Encoding(json.dumps(dict(cfg, stepsize=0.0)))
+    with pytest.raises(qmlp.QmlpError, match="Unknown blending"):
+        qmlp.Encoding(json.dumps(dict(cfg, blending="max")))
+    with pytest.raises(qmlp.QmlpError, match="volumetric"):
+        qmlp.Encoding(json.dumps(dict(cfg, volume={"id": "Identity", "start_in": 0, "n_in": 3})))
+    # as part of a network: 6 raw inputs, 4 encoded channels padded to 16
+    net = qmlp.Network(json.dumps({"num_inputs": 8, "num_outputs": 1, "activation_specification": [bc.BUILTIN],
+                                   "encodings": [cfg], "network": [{"n_out": 1, "bias": False, "activation": "identity"}]}))
+    assert net.num_network_parameters() == 16 * 16
+    assert "EncodingLineIntegration<2, 3, qmlp::kernel::LineIntegrationBlendingMode::AVERAGE" in net.generated_source("inference")

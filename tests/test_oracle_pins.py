@@ -685,3 +685,20 @@ def test_fused_network_with_line_integration_is_the_composition():
     W0, b0, W1 = net.weight(0)[:, :4], net.bias(0), net.weight(1)[:2]
     want = np.maximum(enc @ W0.T + b0, 0) @ W1.T
     assert np.allclose(net.forward(X), want, rtol=1e-4, atol=1e-5)
+
+
+def test_line_integration_takes_no_sample_on_unbounded_or_endless_rays():
+    """Where the reference's march would never end (zero direction: tmin = -inf; a step far
+    below the float spacing at t) the ray takes no sample; the result is zero, not a hang."""
+    child = grid_spec(3, levels=1, feat=1, rmin=4, rmax=4, bmin=[-1.0] * 3, bsize=[2.0] * 3)
+    table = np.full(64, 2.0, np.float32)
+    X = np.array([[0.0, 0.0, 0.0, 0.0, 0.0, 0.0],          # no direction at all, start inside the box
+                  [0.0, 0.0, 0.0, 1e-30, 0.0, 0.0],        # interval of 2e30 length
+                  [0.0, 0.0, 0.0, 0.0, 0.0, 1.0]], np.float32)
+    li = qo.LineIntegration(line_spec(child, 0.3, "additive"))
+    out = li.forward(table, X)
+    assert out[0, 0] == 0 and out[1, 0] == 0 and out[2, 0] == 14.0
+    ax, gp = li.adjoint(table, X[:2], np.ones((2, 1), np.float32))
+    assert not ax.any() and not gp.any()
+    tiny = qo.LineIntegration(line_spec(child, 1e-9, "additive"))      # 2e9 steps: refused
+    assert tiny.forward(table, X[2:])[0, 0] == 0
