@@ -404,7 +404,7 @@ class Network:
         _, enc_out, pre = self.forward(X, round_mode, store=True)
         grads = np.zeros(self.num_parameters, dtype=np.float32) if flags & GRAD_WEIGHTS else None
         tgrads = [np.zeros(e[1].n_params, dtype=np.float32)
-                  if (e[0] == "hashgrid" and flags & GRAD_ENCODINGS) else None
+                  if (e[0] in ("hashgrid", "line") and flags & GRAD_ENCODINGS) else None
                   for e in self.encodings]
         s, keep = self._struct(round_mode, res_factor, grads, tgrads)
         adj_x = np.zeros((N, self.n_in), dtype=np.float32) if flags & GRAD_INPUT else None

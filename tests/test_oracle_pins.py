@@ -683,8 +683,16 @@ def test_fused_network_with_line_integration_is_the_composition():
     X = np.concatenate([start, d / np.linalg.norm(d, axis=1, keepdims=True)], 1).astype(np.float32)
     enc = li.forward(table, X)
     W0, b0, W1 = net.weight(0)[:, :4], net.bias(0), net.weight(1)[:2]
-    want = np.maximum(enc @ W0.T + b0, 0) @ W1.T
+    pre0 = enc @ W0.T + b0
+    want = np.maximum(pre0, 0) @ W1.T
     assert np.allclose(net.forward(X), want, rtol=1e-4, atol=1e-5)
+    # backward: the adjoint of the encoded input goes through the march's own (pinned) adjoint
+    adj = rng.standard_normal((N, 2)).astype(np.float32)
+    res = net.backward(X, adj, 7)
+    d_enc = ((adj @ W1) * (pre0 > 0)) @ W0
+    want_ax, want_gt = li.adjoint(table, X, d_enc.astype(np.float32))
+    assert np.allclose(res["adj_x"], want_ax, rtol=1e-3, atol=1e-4)
+    assert np.allclose(res["table_grads"][0], want_gt, rtol=1e-3, atol=1e-4)
 
 
 def test_line_integration_takes_no_sample_on_unbounded_or_endless_rays():
