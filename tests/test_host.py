@@ -107,7 +107,7 @@ BASE = bc.CONFIGS[1]["cfg"]
 @pytest.mark.parametrize("mutate,code,message", [
     (lambda c: c.update(num_outputs=2), 1, "does not match the number of outputs"),
     (lambda c: c.update(network=[]), 1, "Empty network"),
-    (lambda c: c["encodings"][0].update(id="identity"), 1, "No encoding with id 'identity'"),
+    (lambda c: c["encodings"][0].update(id="Fourier"), 1, "No encoding with id 'Fourier'"),
     (lambda c: c["encodings"][0].update(n_in=4), 1, "out of bounds"),
     (lambda c: c["network"][0].update(activation="gelu"), 1, "No activation with id 'gelu'"),
     (lambda c: c["network"][0].update(activation=["relu"] * 3), 1, "must match the number of output channels"),
