@@ -120,6 +120,7 @@ private:
         CompiledKernel adjoint;
         std::vector<WeightUpdateKernel> layers;
         CompiledKernel reduce;
+        CompiledKernel transpose;
         int perEntryAdjointMemoryBytes = 0;
     };
     std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS];
@@ -242,7 +243,14 @@ private:
     int weightUpdateBlockSize() const;
     // number of batch slices whose partial weight gradients are kept in the adjoint memory
     int weightUpdateSlices(int numTiles) const;
+    // Layers whose weights stay in LDS for the whole kernel; the others are read from global
+    // memory by every wavefront (networks whose weights exceed the LDS).
+    std::vector<char> ldsResidency(bool adjoint) const;
+    // offsets in halves; -1 for weights that are not resident
     int ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const;
+    // offsets (in halves) of the transposed copies of the weights the adjoint kernel reads from
+    // global memory, -1 for resident layers; returns their total size in halves
+    size_t transposedWeightLayout(int adjointFlags, std::vector<long long>& offsets) const;
     int ldsParamHalves(bool adjoint) const;
     int stageBytesPerWave() const;
     std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);

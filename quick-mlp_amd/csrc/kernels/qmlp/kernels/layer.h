@@ -94,8 +94,49 @@ struct Layer
     }
 
     /**
+     * A operand of the forward pass: rows 16m..16m+15 of W, k-block kb.
+     * \tparam GLOBAL_W false: w is the LDS copy in forward operand order. true: w is the
+     *   row-major (COUT, CIN) matrix in global memory (networks whose weights exceed the LDS):
+     *   the lane gathers its two runs of 4 halves itself.
+     */
+    template <bool GLOBAL_W>
+    __device__ __forceinline__ static f16x8 forwardOperand(const f16* __restrict__ w, int m, int kb, int lane)
+    {
+        if constexpr (!GLOBAL_W) {
+            return *reinterpret_cast<const f16x8*>(w + m * F_MSTRIDE + kb * 512 + lane * 8);
+        } else {
+            const int g = lane >> 4, r = lane & 15;
+            const f16* row = w + (16 * m + r) * CIN + 32 * kb + 4 * g;
+            const f16x4 lo = *reinterpret_cast<const f16x4*>(row);
+            f16x4 hi = {0, 0, 0, 0};
+            if (2 * kb + 1 < KT) hi = *reinterpret_cast<const f16x4*>(row + 16);
+            return concat(lo, hi);
+        }
+    }
+
+    /**
+     * A operand of the adjoint pass: rows 16mi..16mi+15 of W^T, k-block kb.
+     * \tparam GLOBAL_W false: wT is the LDS copy in adjoint operand order. true: wT is the
+     *   transposed matrix, row-major (CIN, COUT), in global memory.
+     */
+    template <bool GLOBAL_W>
+    __device__ __forceinline__ static f16x8 adjointOperand(const f16* __restrict__ wT, int mi, int kb, int lane)
+    {
+        if constexpr (!GLOBAL_W) {
+            return *reinterpret_cast<const f16x8*>(wT + mi * A_MSTRIDE + kb * 512 + lane * 8);
+        } else {
+            const int g = lane >> 4, r = lane & 15;
+            const f16* row = wT + (16 * mi + r) * COUT + 32 * kb + 4 * g;
+            const f16x4 lo = *reinterpret_cast<const f16x4*>(row);
+            f16x4 hi = {0, 0, 0, 0};
+            if (2 * kb + 1 < MT) hi = *reinterpret_cast<const f16x4*>(row + 16);
+            return concat(lo, hi);
+        }
+    }
+
+    /**
      * Forward pass of the layer for one 64-point tile.
-     * \param w LDS weights in forward operand order
+     * \param w weights: LDS copy in forward operand order, or (GLOBAL_W) the row-major matrix
      * \param bias LDS bias vector (COUT halves) or nullptr
      * \param x input activations: x[nt][t] = channels 16t+4g+{0..3} of point 4r+nt
      * \param y output activations in the same layout
@@ -104,7 +145,7 @@ struct Layer
      *        lane) and the weight update (per channel, 8 consecutive points) read it
      *        with wide loads
      */
-    template <bool STORE>
+    template <bool STORE, bool GLOBAL_W = false>
     __device__ __forceinline__ static void forward(const f16* __restrict__ w, const f16* __restrict__ bias,
                                                    const f16x4 (&x)[NT][KT], f16x4 (&y)[NT][MT],
                                                    f16* __restrict__ preTile, int lane)
@@ -126,7 +167,7 @@ struct Layer
             }
 #pragma unroll
             for (int kb = 0; kb < F_KB; ++kb) {
-                const f16x8 a = *reinterpret_cast<const f16x8*>(w + m * F_MSTRIDE + kb * 512 + lane * 8);
+                const f16x8 a = forwardOperand<GLOBAL_W>(w, m, kb, lane);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     const f16x4 hi = (2 * kb + 1 < KT) ? x[nt][(2 * kb + 1 < KT) ? 2 * kb + 1 : 0] : zero4;
@@ -150,7 +191,8 @@ struct Layer
 
     /**
      * Adjoint pass of the layer for one 64-point tile.
-     * \param wT LDS weights in adjoint operand order
+     * \param wT transposed weights: LDS copy in adjoint operand order, or (GLOBAL_W) the
+     *        row-major (CIN, COUT) matrix in global memory
      * \param dy in: adjoint of the layer output (after the activation);
      *           out: adjoint of the pre-activation, zeroed for points outside the batch
      * \param dx adjoint of the layer input (only written if COMPUTE_DX)
@@ -158,7 +200,7 @@ struct Layer
      * \param dpreTile [STORE_DPRE] receives the pre-activation adjoints, same layout
      * \param validMask bit nt set iff point 4r+nt of this lane is inside the batch
      */
-    template <bool STORE_DPRE, bool COMPUTE_DX>
+    template <bool STORE_DPRE, bool COMPUTE_DX, bool GLOBAL_W = false>
     __device__ __forceinline__ static void adjoint(const f16* __restrict__ wT, f16x4 (&dy)[NT][MT],
                                                    f16x4 (&dx)[NT][KT], const f16* __restrict__ preTile,
                                                    f16* __restrict__ dpreTile, int validMask, int lane)
@@ -189,7 +231,7 @@ struct Layer
                 for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kb = 0; kb < A_KB; ++kb) {
-                    const f16x8 a = *reinterpret_cast<const f16x8*>(wT + mi * A_MSTRIDE + kb * 512 + lane * 8);
+                    const f16x8 a = adjointOperand<GLOBAL_W>(wT, mi, kb, lane);
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
                         const f16x4 hi = (2 * kb + 1 < MT) ? dy[nt][(2 * kb + 1 < MT) ? 2 * kb + 1 : 0] : zero4;

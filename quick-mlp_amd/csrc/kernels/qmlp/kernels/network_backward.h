@@ -27,6 +27,26 @@ namespace activations
 $$DEFINE_ACTIVATIONS$$
 }
 
+/**
+ * dst (cin, cout) row-major = transpose of src (cout, cin) row-major. Run before the adjoint
+ * kernel for layers whose weights are too large to stay in LDS: the adjoint kernel then reads
+ * its matrix-core operands (rows of W^T) from global memory with two 8-byte loads per lane.
+ */
+__global__ void __launch_bounds__(256) TransposeWeightsKernel(const half* __restrict__ src, half* __restrict__ dst,
+                                                              int cout, int cin)
+{
+    __shared__ half tile[16][17];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int tilesX = cin / 16;
+    for (int t = blockIdx.x; t < tilesX * (cout / 16); t += gridDim.x) {
+        const int o0 = (t / tilesX) * 16, k0 = (t % tilesX) * 16;
+        tile[ty][tx] = src[(o0 + ty) * cin + k0 + tx];
+        __syncthreads();
+        dst[(k0 + ty) * cout + o0 + tx] = tile[tx][ty];
+        __syncthreads();
+    }
+}
+
 __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
     int numel,
     const Tensor2Read<float> inputs,      //shape (numel, Cin)
@@ -34,7 +54,8 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
     Tensor2RW<float> adjInputs,           //shape (numel, Cin), accumulated; unused without input gradients
     const half* __restrict__ networkParametersH,
     const half* __restrict__ forwardTmpMemoryH,  //written by the forward kernel
-    half* __restrict__ adjointTmpMemoryH         //receives dpre if weight gradients are requested
+    half* __restrict__ adjointTmpMemoryH,        //receives dpre if weight gradients are requested
+    const half* __restrict__ transposedWeightsH  //W^T of the layers whose weights do not stay in LDS, or nullptr
     $$ENCODING_PARAMETERS$$)
 {
     constexpr int NUM_INPUTS = $$NUM_INPUTS$$;
@@ -56,6 +77,8 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
     const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
     const f16* __restrict__ forwardTmpMemory = reinterpret_cast<const f16*>(forwardTmpMemoryH);
     f16* __restrict__ adjointTmpMemory = reinterpret_cast<f16*>(adjointTmpMemoryH);
+    const f16* __restrict__ transposedWeights = reinterpret_cast<const f16*>(transposedWeightsH);
+    (void)transposedWeights;
 
     extern __shared__ __align__(16) unsigned char sMemory[];
     f16* sParams = reinterpret_cast<f16*>(sMemory);

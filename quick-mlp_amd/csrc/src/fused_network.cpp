@@ -335,17 +335,65 @@ void FusedNetwork::fillEncodingsAndActivations(std::string& codeTemplate) const
     replaceAll(codeTemplate, "$$CHANNELS_OUT$$", std::to_string(layers_.rbegin()->channelsOut));
 }
 
+static int ldsWeightHalves(int channelsIn, int channelsOut, bool adjoint)
+{
+    // matrix-core operand order, contraction width padded to 32 channels
+    return adjoint ? channelsIn * roundUp(channelsOut, 32) : channelsOut * roundUp(channelsIn, 32);
+}
+
+std::vector<char> FusedNetwork::ldsResidency(bool adjoint) const
+{
+    const int L = static_cast<int>(layers_.size());
+    std::vector<char> resident(L, 1);
+    std::vector<long long> bytes(L);
+    long long total = 0, biases = 0;
+    for (int i = 0; i < L; ++i) {
+        bytes[i] = static_cast<long long>(ldsWeightHalves(layers_[i].channelsIn, layers_[i].channelsOut, adjoint)) * sizeof(half);
+        total += bytes[i];
+        if (!adjoint && layers_[i].useBias) biases += layers_[i].channelsOut * sizeof(half);
+    }
+    const long long maxLds = MaxSharedMemoryBytes();
+    // everything stays if four wavefronts still find room for their staging tiles
+    if (total + biases + 16 + 4ll * stageBytesPerWave() <= maxLds) return resident;
+    // otherwise keep the subset with the most bytes that leaves room for eight wavefronts
+    const long long budget = maxLds - biases - 16 - 8ll * stageBytesPerWave();
+    long long best = -1;
+    unsigned bestMask = 0;
+    if (L <= 20) {
+        for (unsigned mask = 0; mask < (1u << L); ++mask) {
+            long long sum = 0;
+            for (int i = 0; i < L; ++i)
+                if (mask & (1u << i)) sum += bytes[i];
+            if (sum <= budget && sum > best) {
+                best = sum;
+                bestMask = mask;
+            }
+        }
+    } else {
+        long long sum = 0;
+        for (int i = 0; i < L; ++i)
+            if (sum + bytes[i] <= budget) {
+                sum += bytes[i];
+                bestMask |= 1u << i;
+            }
+    }
+    for (int i = 0; i < L; ++i) resident[i] = (bestMask >> i) & 1;
+    return resident;
+}
+
 int FusedNetwork::ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const
 {
     // Weights sit in LDS in matrix-core operand order, contraction width padded to 32
     // channels (forward: C_in, adjoint: C_out); the biases follow (forward only).
-    weightOffsets.assign(layers_.size(), 0);
+    weightOffsets.assign(layers_.size(), -1);
     biasOffsets.assign(layers_.size(), 0);
+    const auto resident = ldsResidency(adjoint);
     int n = 0;
     for (size_t i = 0; i < layers_.size(); ++i) {
+        if (!resident[i]) continue;
         const auto& l = layers_[i];
         weightOffsets[i] = n;
-        n += adjoint ? l.channelsIn * roundUp(l.channelsOut, 32) : l.channelsOut * roundUp(l.channelsIn, 32);
+        n += ldsWeightHalves(l.channelsIn, l.channelsOut, adjoint);
     }
     if (!adjoint) {
         for (size_t i = 0; i < layers_.size(); ++i) {
@@ -355,6 +403,20 @@ int FusedNetwork::ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::
         }
     }
     return roundUp(n, 8);
+}
+
+size_t FusedNetwork::transposedWeightLayout(int adjointFlags, std::vector<long long>& offsets) const
+{
+    offsets.assign(layers_.size(), -1);
+    const auto resident = ldsResidency(true);
+    const bool needsEncodingAdjoint = adjointFlags & (GRADIENTS_INPUT | GRADIENTS_INPUT_ENCODINGS);
+    size_t n = 0;
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        if (resident[i] || (i == 0 && !needsEncodingAdjoint)) continue;
+        offsets[i] = static_cast<long long>(n);
+        n += static_cast<size_t>(layers_[i].channelsIn) * layers_[i].channelsOut;
+    }
+    return n;
 }
 
 int FusedNetwork::ldsParamHalves(bool adjoint) const
@@ -384,15 +446,26 @@ int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLa
                                   "tile need %d bytes of LDS, the device offers %d",
                                   numParameters_, paramBytes + stageBytesPerWave(), maxLds);
     while (paramBytes + (blockSize / WARP_SIZE) * stageBytesPerWave() > maxLds) blockSize -= WARP_SIZE;
+    int ppl = 1;
     if (pointsPerLane) {
         // Grid encodings gather level by level over several points per lane; two workgroups
         // should still fit on a compute unit.
         bool gathers = false;
         for (const auto& e : encodings_) gathers = gathers || e->hasParameters();
-        int ppl = compileOptions_.pointsPerLane > 0 ? compileOptions_.pointsPerLane : (gathers ? 2 : 1);
+        ppl = compileOptions_.pointsPerLane > 0 ? compileOptions_.pointsPerLane : (gathers ? 2 : 1);
         const int budget = compileOptions_.pointsPerLane > 0 ? maxLds : maxLds / 2;
         while (ppl > 1 && paramBytes + (blockSize / WARP_SIZE) * ppl * stageBytesPerWave() > budget) --ppl;
         *pointsPerLane = ppl;
+    }
+    if (overwrite <= 0) {
+        // The weights in LDS are per workgroup: when they are large, a workgroup of 8 wavefronts
+        // brings more wavefronts onto a compute unit than two of 4 would.
+        auto wavesPerComputeUnit = [&](int block) {
+            const int lds = paramBytes + (block / WARP_SIZE) * ppl * stageBytesPerWave();
+            if (lds > maxLds) return 0;
+            return std::min(16, (maxLds / lds) * (block / WARP_SIZE));
+        };
+        if (wavesPerComputeUnit(2 * DEFAULT_BLOCK_SIZE) > wavesPerComputeUnit(blockSize)) blockSize = 2 * DEFAULT_BLOCK_SIZE;
     }
     return blockSize;
 }
@@ -442,8 +515,9 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     stage << layerTypedefs(layerTypes);
     for (size_t i = 0; i < layers_.size(); ++i) {
         const auto& l = layers_[i];
-        stage << "    Layer" << i << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + "
-              << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
+        if (ldsW[i] >= 0)
+            stage << "    Layer" << i << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + "
+                  << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
         if (l.useBias)
             stage << "    for (int i = threadIdx.x; i < " << l.channelsOut << "; i += blockDim.x) sParams["
                   << ldsB[i] << " + i] = networkParameters[" << l.biasStart << " + i];\n";
@@ -468,7 +542,11 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     for (size_t i = 0; i < layers_.size(); ++i) {
         const auto& l = layers_[i];
         callLayers << "        f16x4 x" << (i + 1) << "[NT][Layer" << i << "::MT];\n";
-        callLayers << "        Layer" << i << "::template forward<STORE>(sParams + " << ldsW[i] << ", ";
+        if (ldsW[i] >= 0)
+            callLayers << "        Layer" << i << "::template forward<STORE>(sParams + " << ldsW[i] << ", ";
+        else
+            callLayers << "        Layer" << i << "::template forward<STORE, true>(networkParameters + " << l.weightsStart
+                       << ", ";
         if (l.useBias)
             callLayers << "sParams + " << ldsB[i];
         else
@@ -510,21 +588,26 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     std::stringstream stage;
     stage << layerTypedefs(layerTypes);
     for (size_t i = 0; i < layers_.size(); ++i) {
-        if (i == 0 && !needsEncodingAdjoint) continue;
+        if ((i == 0 && !needsEncodingAdjoint) || ldsW[i] < 0) continue;
         const auto& l = layers_[i];
         stage << "    Layer" << i << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + "
               << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
     }
     replaceAll(code, "$$STAGE_PARAMETERS$$", stage.str());
 
+    std::vector<long long> transposed;
+    transposedWeightLayout(flags, transposed);
     std::stringstream callLayers;
     const int L = static_cast<int>(layers_.size());
     for (int i = L - 1; i >= 0; --i) {
         const auto& l = layers_[i];
         const std::string dy = (i == L - 1) ? std::string("dyOut") : "dx" + std::to_string(i + 1);
         callLayers << "        f16x4 dx" << i << "[NT][Layer" << i << "::KT];\n";
+        std::string weights = "sParams + " + std::to_string(ldsW[i]);
+        if (ldsW[i] < 0) weights = transposed[i] >= 0 ? "transposedWeights + " + std::to_string(transposed[i]) : "nullptr";
         callLayers << "        Layer" << i << "::template adjoint<HAS_NETWORK_GRADIENTS, "
-                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << ">(sParams + " << ldsW[i] << ", " << dy
+                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (ldsW[i] < 0 ? ", true" : "") << ">(" << weights
+                   << ", " << dy
                    << ", dx" << i << ",\n            forwardTmpMemory + (" << backwardInfo_[i].offsetPre
                    << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut << " * TILE_POINTS)),\n"
                    << "            HAS_NETWORK_GRADIENTS ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut
@@ -662,8 +745,16 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
     ak.adjoint.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
     ak.adjoint.sharedMemorySize =
         ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (ak.adjoint.blockSize / WARP_SIZE) * stageBytesPerWave();
-    ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", backwardSource(flags, ak.adjoint.blockSize),
-                                   loaderFlags(compileOnly)).value();
+    const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize);
+    ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
+    {
+        std::vector<long long> transposed;
+        if (transposedWeightLayout(flags, transposed) > 0) {
+            ak.transpose.blockSize = 256;
+            ak.transpose.fun =
+                kl->getKernel("qmlp::kernel::TransposeWeightsKernel", adjointSource, loaderFlags(compileOnly)).value();
+        }
+    }
     if (!compileOnly) {
         ak.adjoint.fullGrid = ak.adjoint.fun.fullGridSize(ak.adjoint.blockSize, ak.adjoint.sharedMemorySize);
         logger->debug("backward kernel (flags %d): block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d", flags,
@@ -817,6 +908,9 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
     // behind the adjoint pre-activations: the partial weight gradients of the batch slices
     if (adjointFlags & GRADIENTS_NETWORK_WEIGHTS)
         bytes += static_cast<size_t>(weightUpdateSlices(numElements / TILE_POINTS)) * numParameters_ * sizeof(float);
+    // last: transposed copies of the weights the adjoint kernel cannot keep in LDS
+    std::vector<long long> transposed;
+    bytes += roundUp(transposedWeightLayout(adjointFlags, transposed) * sizeof(half), size_t(16));
     return bytes;
 }
 
@@ -858,7 +952,9 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
     if (numel == 0) return;
     CHECK_ERROR(tmpMemoryForward != nullptr, "adjoint() needs the temporary memory written by forward()");
-    if (hasNetworkGradients) {
+    std::vector<long long> transposedOffsets;
+    const size_t transposedHalves = transposedWeightLayout(adjointFlags, transposedOffsets);
+    if (hasNetworkGradients || transposedHalves > 0) {
         CHECK_ERROR(tmpMemoryAdjoint != nullptr, "adjoint() needs temporary memory of adjointMemory() bytes");
         CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemoryAdjoint) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
     }
@@ -869,6 +965,23 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
 
     const int numTiles = divUp(numel, TILE_POINTS);
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
+    const half* transposedWeights = nullptr;
+    if (transposedHalves > 0) {
+        size_t offset = static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64);
+        if (hasNetworkGradients) offset += static_cast<size_t>(weightUpdateSlices(numTiles)) * numParameters_ * sizeof(float);
+        half* dstBase = reinterpret_cast<half*>(static_cast<char*>(tmpMemoryAdjoint) + offset);
+        transposedWeights = dstBase;
+        for (size_t layer = 0; layer < layers_.size(); ++layer) {
+            if (transposedOffsets[layer] < 0) continue;
+            const auto& ls = layers_[layer];
+            const half* src = parametersInference_.dataPtr<half>() + ls.weightsStart;
+            half* dst = dstBase + transposedOffsets[layer];
+            int cout = ls.channelsOut, cin = ls.channelsIn;
+            void* args[] = {&src, &dst, &cout, &cin};
+            const int tiles = (cout / MATRIX_SIZE) * (cin / MATRIX_SIZE);
+            ak.transpose.fun.launch(std::min(tiles, 1024), ak.transpose.blockSize, 0, stream, args);
+        }
+    }
     {
         const auto& ck = ak.adjoint;
         const int waves = ck.blockSize / WARP_SIZE;
@@ -882,7 +995,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         const half* forwardTmpMemory = static_cast<const half*>(tmpMemoryForward);
         half* adjointTmpMemory = static_cast<half*>(tmpMemoryAdjoint);
         std::vector<void*> args = {&numel, &inputAcc, &adjOutputAcc, &adjInputAcc, &networkParams,
-                                   &forwardTmpMemory, &adjointTmpMemory};
+                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights};
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());

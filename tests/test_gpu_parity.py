@@ -58,6 +58,26 @@ def test_two_layers_against_oracle(c0, c1, c2, acts):
     check_gradients(case, X, one, FLAG_INPUT, case.gpu_train(X, one, FLAG_INPUT), kinks, "single entry: ")
 
 
+@pytest.mark.parametrize("widths,act", [([128] * 6 + [16], "celu"), ([256, 256, 256, 3], "sine"), ([512, 208, 16], "identity")])
+def test_networks_whose_weights_exceed_the_lds(widths, act):
+    """More than 160 KB of fp16 weights: some layers stay in LDS, the kernels read the others
+    (forward: W, adjoint: a transposed copy in the adjoint memory) from global memory."""
+    n_in = 19
+    case = Case(identity_cfg(n_in, widths, [act] * len(widths), [True] * len(widths)))
+    assert "forward<STORE, true>" in case.net.generated_source("forward")
+    assert "transposedWeights +" in case.net.generated_source("backward", 7)
+    rng = np.random.default_rng(77)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    N = 1500
+    X = rng.uniform(-1, 1, (N, n_in)).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, widths[-1])) / N).astype(np.float32)
+    assert_close(case.gpu_inference(X), case.oracle.forward(X), "inference")
+    for flags in (FLAG_INPUT | FLAG_WEIGHTS, FLAG_INPUT):
+        got = case.gpu_train(X, adj, flags)
+        assert_close(got["out"], case.oracle.forward(X), "forward")
+        check_gradients(case, X, adj, flags, got, what="flags %d: " % flags)
+
+
 @pytest.mark.parametrize("widths", [[16], [32, 16], [48, 32, 16], [16, 48, 48]])
 @pytest.mark.parametrize("act", ["celu", "identity"])
 @pytest.mark.parametrize("N", [16, 32, 128, 513, 48621])
