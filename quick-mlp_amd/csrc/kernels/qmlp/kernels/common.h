@@ -111,30 +111,42 @@ __device__ __forceinline__ f16x8 concat(f16x4 a, f16x4 b)
 
 __device__ __forceinline__ f16x4 toF16(f32x4 v)
 {
-    f16x4 o;
-    o[0] = static_cast<f16>(v[0]);
-    o[1] = static_cast<f16>(v[1]);
-    o[2] = static_cast<f16>(v[2]);
-    o[3] = static_cast<f16>(v[3]);
-    return o;
+    // as one vector conversion: two packed round-to-nearest conversions instead of four
+    // scalar ones and two packs
+    return __builtin_convertvector(v, f16x4);
 }
+
+/** Detects the optional packed form `static f16x4 forward4(f16x4)` of an activation. */
+template <typename Act, typename = void>
+struct HasPackedForward
+{
+    static constexpr bool value = false;
+};
+template <typename Act>
+struct HasPackedForward<Act, decltype(void(Act::forward4(f16x4{})))>
+{
+    static constexpr bool value = true;
+};
 
 template <typename Act>
 __device__ __forceinline__ f16x4 activationForward(f16x4 v)
 {
-    f16x4 o;
+    if constexpr (HasPackedForward<Act>::value) {
+        return Act::forward4(v);
+    } else {
+        f16x4 o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = fromHalf(Act::forward(toHalf(v[i])));
-    return o;
+        for (int i = 0; i < 4; ++i) o[i] = fromHalf(Act::forward(toHalf(v[i])));
+        return o;
+    }
 }
 
 template <typename Act>
 __device__ __forceinline__ f16x8 activationForward(f16x8 v)
 {
-    f16x8 o;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = fromHalf(Act::forward(toHalf(v[i])));
-    return o;
+    const f16x4 lo = activationForward<Act>(f16x4{v[0], v[1], v[2], v[3]});
+    const f16x4 hi = activationForward<Act>(f16x4{v[4], v[5], v[6], v[7]});
+    return concat(lo, hi);
 }
 
 /** One row of a strided 2-D tensor. */

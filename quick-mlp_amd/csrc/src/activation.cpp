@@ -3,11 +3,34 @@
 #include <qmlp/errors.h>
 #include <qmlp/qmlp.h>
 
+#include <cctype>
 #include <fstream>
 #include <regex>
 #include <sstream>
 
 QUICKMLP_NAMESPACE_BEGIN
+
+static std::string withoutSpaces(const std::string& s)
+{
+    std::string o;
+    for (char c : s)
+        if (!std::isspace(static_cast<unsigned char>(c))) o += c;
+    return o;
+}
+
+/**
+ * Packed form of snippets that are recognised literally (after removing white space): the
+ * kernels apply it to four values at once (two packed instructions) instead of calling the
+ * scalar snippet four times. Unknown snippets have none.
+ */
+static std::string packedForward(const std::string& forward)
+{
+    const std::string f = withoutSpaces(forward);
+    if (f == "z=__hgt(x,hZERO())?x:hZERO()")   // ReLU: v_pk_max_f16 (NaN -> 0 like the comparison)
+        return "        return __builtin_elementwise_max(x, f16x4{0, 0, 0, 0});\n";
+    if (f == "z=x") return "        return x;\n";
+    return "";
+}
 
 static std::string generateCode(const std::string& id, const std::string& forward, const std::string& adjoint)
 {
@@ -24,13 +47,16 @@ struct %s
         %s ;
         return adjx;
     }
-};
+%s};
     )code";
 
     static const std::regex CPP_IDENTIFIER_REGEX("^[a-zA-Z_][a-zA-Z0-9_]*$");
     if (!std::regex_match(id, CPP_IDENTIFIER_REGEX))
         throw configuration_error("id of the activation function is not a valid C++ identifier: %s", id.c_str());
-    return format(TEMPLATE, id.c_str(), forward.c_str(), adjoint.c_str());
+    std::string packed = packedForward(forward);
+    if (!packed.empty())
+        packed = "    static __device__ __forceinline__ f16x4 forward4(f16x4 x) {\n" + packed + "    }\n";
+    return format(TEMPLATE, id.c_str(), forward.c_str(), adjoint.c_str(), packed.c_str());
 }
 
 Activation::Activation(const std::string& id, const std::string& forward, const std::string& adjoint)
