@@ -94,9 +94,8 @@ private:
         int sharedMemorySize = 0;
         int fullGrid = 0;
     };
-    // [store intermediates][0: the preferred number of tiles per wave, 1: one tile per wave,
-    // for batches too small to fill the device with the former]
-    std::optional<CompiledKernel> forwardKernels_[2][2];
+    // [store intermediates][variant], see ForwardVariant
+    std::optional<CompiledKernel> forwardKernels_[2][3];
 
     struct AdjointLayerInfo
     {
@@ -230,7 +229,13 @@ public:
     std::string generatedSource(const std::string& kind, int adjointFlags = 0);
 
 private:
-    void compileForwardKernel(bool store, bool narrow, bool compileOnly = false);
+    // Shapes of the inference / forward kernel. LARGE: 8 wavefronts with 4 tiles each, for grid
+    // encodings on batches that still fill the device that way (fewer sweeps over the level
+    // tables); DEFAULT: 4 wavefronts, 2 tiles each with grid encodings; NARROW: one tile per
+    // wavefront for small batches.
+    enum ForwardVariant { VARIANT_DEFAULT = 0, VARIANT_NARROW = 1, VARIANT_LARGE = 2 };
+    bool hasLargeVariant(bool store) const;
+    void compileForwardKernel(bool store, int variant, bool compileOnly = false);
     const CompiledKernel& forwardKernelFor(bool store, int numTiles);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 
@@ -252,7 +257,7 @@ private:
     // global memory, -1 for resident layers; returns their total size in halves
     size_t transposedWeightLayout(int adjointFlags, std::vector<long long>& offsets) const;
     int ldsParamHalves(bool adjoint) const;
-    int stageBytesPerWave() const;
+    int stageBytesPerWave(bool adjoint) const;
     std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);
     void ensureStreams();
 };

@@ -45,7 +45,8 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     constexpr int CHANNELS_OUT = $$CHANNELS_OUT$$;        // padded width of the last layer
     constexpr int KT0 = CHANNELS_IN / 16;
     constexpr int MTL = CHANNELS_OUT / 16;
-    constexpr int STAGE_STRIDE = CHANNELS_IN + 8;         // halves; odd multiple of 16 bytes
+    typedef StageLayout<CHANNELS_IN> Stage;               // padded or rotated rows, see arrays.h
+    constexpr int STAGE_STRIDE = Stage::Stride;           // halves
     constexpr int LDS_PARAM_HALVES = $$LDS_PARAM_HALVES$$;
     constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
     constexpr int PPL = $$POINTS_PER_LANE$$;              // tiles a wave encodes together
@@ -74,13 +75,15 @@ $$STAGE_PARAMETERS$$
         // no NaN enters the matrix cores.
         {
             StaticArray<float, NUM_INPUTS> encodingInput[PPL];
-            WrappedArray<f16> encodingOutput[PPL];
+            StageRowArray<f16, CHANNELS_IN> encodingOutput[PPL];
             bool valid[PPL];
 #pragma unroll
             for (int q = 0; q < PPL; ++q) {
                 const int index = (tile0 + q) * TILE_POINTS + lane;
                 valid[q] = index < numel;
-                encodingOutput[q].data_ = sStage + (q * TILE_POINTS + stageRow(lane)) * STAGE_STRIDE;
+                encodingOutput[q].row_ = sStage + (q * TILE_POINTS + stageRow(lane)) * STAGE_STRIDE;
+                encodingOutput[q].rotation_ = Stage::rotation(stageRow(lane));
+                encodingOutput[q].offset_ = 0;
 #pragma unroll
                 for (int i = 0; i < NUM_INPUTS; ++i)
                     encodingInput[q][i] = valid[q] ? inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
@@ -113,7 +116,7 @@ $$CALL_ENCODINGS$$
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int t = 0; t < KT0; ++t)
-                x0[nt][t] = *reinterpret_cast<const f16x4*>(sTile + (16 * nt + r) * STAGE_STRIDE + 16 * t + 4 * g);
+                x0[nt][t] = *reinterpret_cast<const f16x4*>(sTile + Stage::chunkOffset(16 * nt + r, 4 * t + g));
 
         if constexpr (STORE) {
             // encoded input, channel-major per tile, for the weight update of layer 0

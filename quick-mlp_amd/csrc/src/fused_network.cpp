@@ -354,9 +354,9 @@ std::vector<char> FusedNetwork::ldsResidency(bool adjoint) const
     }
     const long long maxLds = MaxSharedMemoryBytes();
     // everything stays if four wavefronts still find room for their staging tiles
-    if (total + biases + 16 + 4ll * stageBytesPerWave() <= maxLds) return resident;
+    if (total + biases + 16 + 4ll * stageBytesPerWave(adjoint) <= maxLds) return resident;
     // otherwise keep the subset with the most bytes that leaves room for eight wavefronts
-    const long long budget = maxLds - biases - 16 - 8ll * stageBytesPerWave();
+    const long long budget = maxLds - biases - 16 - 8ll * stageBytesPerWave(adjoint);
     long long best = -1;
     unsigned bestMask = 0;
     if (L <= 20) {
@@ -425,9 +425,12 @@ int FusedNetwork::ldsParamHalves(bool adjoint) const
     return ldsLayout(adjoint, w, b);
 }
 
-int FusedNetwork::stageBytesPerWave() const
+int FusedNetwork::stageBytesPerWave(bool adjoint) const
 {
-    return TILE_POINTS * (layers_[0].channelsIn + STAGE_PAD) * static_cast<int>(sizeof(half));
+    // the forward kernel rotates the chunks of rows of 32, 64 or 128 halves instead of padding them
+    const int c = layers_[0].channelsIn;
+    const bool rotated = !adjoint && (c == 32 || c == 64 || c == 128);
+    return TILE_POINTS * (c + (rotated ? 0 : STAGE_PAD)) * static_cast<int>(sizeof(half));
 }
 
 int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane) const
@@ -441,11 +444,11 @@ int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLa
     }
     const int maxLds = MaxSharedMemoryBytes();
     const int paramBytes = ldsParamHalves(adjoint) * static_cast<int>(sizeof(half));
-    if (paramBytes + stageBytesPerWave() > maxLds)
+    if (paramBytes + stageBytesPerWave(adjoint) > maxLds)
         throw configuration_error("The network is too large for the fused kernels: its %d parameters plus one staging "
                                   "tile need %d bytes of LDS, the device offers %d",
-                                  numParameters_, paramBytes + stageBytesPerWave(), maxLds);
-    while (paramBytes + (blockSize / WARP_SIZE) * stageBytesPerWave() > maxLds) blockSize -= WARP_SIZE;
+                                  numParameters_, paramBytes + stageBytesPerWave(adjoint), maxLds);
+    while (paramBytes + (blockSize / WARP_SIZE) * stageBytesPerWave(adjoint) > maxLds) blockSize -= WARP_SIZE;
     int ppl = 1;
     if (pointsPerLane) {
         // Grid encodings gather level by level over several points per lane; two workgroups
@@ -454,14 +457,14 @@ int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLa
         for (const auto& e : encodings_) gathers = gathers || e->hasParameters();
         ppl = compileOptions_.pointsPerLane > 0 ? compileOptions_.pointsPerLane : (gathers ? 2 : 1);
         const int budget = compileOptions_.pointsPerLane > 0 ? maxLds : maxLds / 2;
-        while (ppl > 1 && paramBytes + (blockSize / WARP_SIZE) * ppl * stageBytesPerWave() > budget) --ppl;
+        while (ppl > 1 && paramBytes + (blockSize / WARP_SIZE) * ppl * stageBytesPerWave(adjoint) > budget) --ppl;
         *pointsPerLane = ppl;
     }
     if (overwrite <= 0) {
         // The weights in LDS are per workgroup: when they are large, a workgroup of 8 wavefronts
         // brings more wavefronts onto a compute unit than two of 4 would.
         auto wavesPerComputeUnit = [&](int block) {
-            const int lds = paramBytes + (block / WARP_SIZE) * ppl * stageBytesPerWave();
+            const int lds = paramBytes + (block / WARP_SIZE) * ppl * stageBytesPerWave(adjoint);
             if (lds > maxLds) return 0;
             return std::min(16, (maxLds / lds) * (block / WARP_SIZE));
         };
@@ -528,7 +531,7 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     int encodingOffset = 0;
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
-        callEncodings << "            {\n                WrappedArray<f16> encodingOutputK[PPL];\n"
+        callEncodings << "            {\n                StageRowArray<f16, CHANNELS_IN> encodingOutputK[PPL];\n"
                       << "#pragma unroll\n                for (int q = 0; q < PPL; ++q) encodingOutputK[q] = encodingOutput[q] + "
                       << encodingOffset << ";\n                " << e->qualifiedName()
                       << "::template forwardBatch<PPL>(encodingInput, encodingOutputK";
@@ -698,17 +701,31 @@ static int loaderFlags(bool compileOnly)
     return flags;
 }
 
-void FusedNetwork::compileForwardKernel(bool store, bool narrow, bool compileOnly)
+bool FusedNetwork::hasLargeVariant(bool store) const
 {
-    auto& slot = forwardKernels_[store ? 1 : 0][narrow ? 1 : 0];
+    const int overwrite = store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference;
+    if (overwrite > 0 || compileOptions_.pointsPerLane > 0) return false;
+    bool gathers = false;
+    for (const auto& e : encodings_) gathers = gathers || e->hasParameters();
+    const int lds = ldsParamHalves(false) * static_cast<int>(sizeof(half)) + 8 * 4 * stageBytesPerWave(false);
+    return gathers && lds <= MaxSharedMemoryBytes();
+}
+
+void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnly)
+{
+    auto& slot = forwardKernels_[store ? 1 : 0][variant];
     if (slot.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
     ck.blockSize = forwardBlockSize(store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference,
                                     false, &ck.pointsPerLane);
-    if (narrow) ck.pointsPerLane = 1;
+    if (variant == VARIANT_NARROW) ck.pointsPerLane = 1;
+    if (variant == VARIANT_LARGE) {
+        ck.blockSize = 2 * DEFAULT_BLOCK_SIZE;
+        ck.pointsPerLane = 4;
+    }
     ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
-        + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave();
+        + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave(false);
     ck.fun = kl->getKernel(store ? "qmlp::kernel::NetworkKernelInferenceAndForward<true>"
                                  : "qmlp::kernel::NetworkKernelInferenceAndForward<false>",
                            forwardSource(ck.blockSize, ck.pointsPerLane), loaderFlags(compileOnly)).value();
@@ -723,14 +740,20 @@ void FusedNetwork::compileForwardKernel(bool store, bool narrow, bool compileOnl
 
 const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles)
 {
-    compileForwardKernel(store, false);
-    const auto& wide = forwardKernels_[store ? 1 : 0][0].value();
+    const int s = store ? 1 : 0;
+    if (hasLargeVariant(store)) {
+        compileForwardKernel(store, VARIANT_LARGE);
+        const auto& large = forwardKernels_[s][VARIANT_LARGE].value();
+        if (divUp(numTiles, (large.blockSize / WARP_SIZE) * large.pointsPerLane) >= large.fullGrid) return large;
+    }
+    compileForwardKernel(store, VARIANT_DEFAULT);
+    const auto& wide = forwardKernels_[s][VARIANT_DEFAULT].value();
     if (wide.pointsPerLane == 1) return wide;
-    // several tiles per wave only pay off once they still fill every compute unit
+    // several tiles per wave only pay off while they still fill most of the compute units
     const int waves = wide.blockSize / WARP_SIZE;
-    if (divUp(numTiles, waves * wide.pointsPerLane) >= wide.fullGrid) return wide;
-    compileForwardKernel(store, true);
-    return forwardKernels_[store ? 1 : 0][1].value();
+    if (2 * divUp(numTiles, waves * wide.pointsPerLane) >= wide.fullGrid) return wide;
+    compileForwardKernel(store, VARIANT_NARROW);
+    return forwardKernels_[s][VARIANT_NARROW].value();
 }
 
 void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
@@ -744,7 +767,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
     AdjointKernel ak;
     ak.adjoint.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
     ak.adjoint.sharedMemorySize =
-        ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (ak.adjoint.blockSize / WARP_SIZE) * stageBytesPerWave();
+        ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (ak.adjoint.blockSize / WARP_SIZE) * stageBytesPerWave(true);
     const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize);
     ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
     {
@@ -796,10 +819,11 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
 void FusedNetwork::precompile(int adjointFlags)
 {
     for (int store = 0; store < 2; ++store) {
-        compileForwardKernel(store, false, true);
+        compileForwardKernel(store, VARIANT_DEFAULT, true);
         int ppl = 1;
         forwardBlockSize(-1, false, &ppl);
-        if (ppl > 1) compileForwardKernel(store, true, true);
+        if (ppl > 1) compileForwardKernel(store, VARIANT_NARROW, true);
+        if (hasLargeVariant(store)) compileForwardKernel(store, VARIANT_LARGE, true);
     }
     if (adjointFlags > 0) compileBackwardKernel(adjointFlags, true);
 }

@@ -180,10 +180,11 @@ def test_kernels_compile_for_gfx950_without_a_gpu_and_are_cached(tmp_path):
         c0, h0 = qmlp._lib.kernel_cache_stats()
         qmlp.Network(json.dumps(cfg)).precompile(7)
         c1, h1 = qmlp._lib.kernel_cache_stats()
-        # inference and forward with two and one tile(s) per wave, backward, 2 weight updates + reduce
-        assert c1 - c0 == 8 and h1 == h0
+        # inference and forward in three shapes (4x2, 4x1 and 8x4 wavefronts x tiles), backward,
+        # 2 weight updates + reduce
+        assert c1 - c0 == 10 and h1 == h0
         files = os.listdir(cache)
-        assert len(files) == 8 and all(f.endswith(".co") for f in files)
+        assert len(files) == 10 and all(f.endswith(".co") for f in files)
         qmlp.Network(json.dumps(cfg)).precompile(7)
         c2, h2 = qmlp._lib.kernel_cache_stats()
         assert c2 == c1                            # nothing recompiled (memory or disk cache)
@@ -207,13 +208,22 @@ def test_compile_errors_carry_the_compiler_log(tmp_path):
         qmlp.set_kernel_cache_dir(os.environ.get("QMLP_CACHE_DIR", qmlp._lib.DEFAULT_CACHE_DIR))
 
 
-def test_network_too_large_for_lds_is_rejected():
+def test_weights_beyond_the_lds_are_read_from_global_memory():
+    """3 x 256x256 fp16 weights are 384 KB: one layer stays in LDS, the others are gathered from
+    global memory (forward) or from a transposed copy in the adjoint memory (adjoint)."""
     cfg = json.loads(json.dumps(BASE))
     cfg["network"] = [{"n_out": 256, "bias": False, "activation": "relu"}] * 3 + [{"n_out": 1, "bias": False, "activation": "relu"}]
     cfg["num_outputs"] = 1
     net = qmlp.Network(json.dumps(cfg))
-    with pytest.raises(qmlp.QmlpError, match="too large for the fused kernels"):
-        net.precompile(0)
+    fwd = net.generated_source("forward")
+    n_global = fwd.count("forward<STORE, true>(networkParameters +")
+    assert n_global >= 1 and n_global + fwd.count("::stageForward(networkParameters") == 4
+    bwd = net.generated_source("backward", 1)
+    n_transposed = bwd.count("true>(transposedWeights +")
+    assert n_transposed >= 1 and n_transposed + bwd.count("::stageAdjoint(networkParameters") == 4
+    small = qmlp.Network(json.dumps(BASE))
+    assert small.adjoint_memory(64, 1) == 0
+    assert net.adjoint_memory(64, 1) >= 256 * 256 * 2                        # the transposed copies
 
 
 def test_simulated_network_and_weight_copy_shapes():
