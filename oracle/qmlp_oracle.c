@@ -437,6 +437,20 @@ int qo_network_encoded_channels(const qo_network* net)
     return c;
 }
 
+static inline float layer_act_forward(const qo_network* net, int l, int channel, float x)
+{
+    if (net->act_channel[l])
+        return qo_act_forward(net->act_channel[l][channel], net->act_param_channel[l][channel], x);
+    return qo_act_forward(net->act[l], net->act_param[l], x);
+}
+
+static inline float layer_act_adjoint(const qo_network* net, int l, int channel, float x, float adjz)
+{
+    if (net->act_channel[l])
+        return qo_act_adjoint(net->act_channel[l][channel], net->act_param_channel[l][channel], x, adjz);
+    return qo_act_adjoint(net->act[l], net->act_param[l], x, adjz);
+}
+
 static inline float maybe_round(const qo_network* net, float v)
 {
     return net->round_mode ? qo_round_half(v) : v;
@@ -525,7 +539,7 @@ void qo_network_forward(const qo_network* net, const float* X, long N, long x_st
                 for (int o = 0; o < co; ++o) {
                     float p = maybe_round(net, nxt[o]);
                     if (pre) pre[l][n * co + o] = p;
-                    nxt[o] = maybe_round(net, qo_act_forward(net->act[l], net->act_param[l], p));
+                    nxt[o] = maybe_round(net, layer_act_forward(net, l, o, p));
                 }
                 float* t = cur; cur = nxt; nxt = t;
             }
@@ -567,8 +581,7 @@ void qo_network_backward(const qo_network* net, const float* X, long N, long x_s
                 woff -= (size_t)ci * co;
                 boff -= (size_t)co;
                 for (int o = 0; o < co; ++o) {
-                    float d = qo_act_adjoint(net->act[l], net->act_param[l],
-                                             pre[l][n * co + o], cur[o]);
+                    float d = layer_act_adjoint(net, l, o, pre[l][n * co + o], cur[o]);
                     d = maybe_round(net, d);
                     cur[o] = d;
                     if (dpre_out) dpre_out[l][n * co + o] = d;
@@ -579,8 +592,7 @@ void qo_network_backward(const qo_network* net, const float* X, long N, long x_s
                     } else {
                         const int cp = net->cout[l - 1];
                         for (int i = 0; i < cp; ++i)
-                            inrow[i] = maybe_round(net, qo_act_forward(net->act[l - 1],
-                                            net->act_param[l - 1], pre[l - 1][n * cp + i]));
+                            inrow[i] = maybe_round(net, layer_act_forward(net, l - 1, i, pre[l - 1][n * cp + i]));
                     }
                     if (net->dW[l]) outer_accumulate(lw + woff, cur, inrow, ci, co);
                     if (net->db[l]) for (int o = 0; o < co; ++o) lb[boff + o] += cur[o];

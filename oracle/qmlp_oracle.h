@@ -99,6 +99,10 @@ typedef struct {
     int cout[QO_MAX_LAYERS];
     int act[QO_MAX_LAYERS];
     float act_param[QO_MAX_LAYERS];
+    /* optional: one activation per (padded) output channel, cout[l] entries; NULL = act[l] for
+     * all channels (the per-channel lists of src_cpp/src/fused_network.cpp:112-125) */
+    const int* act_channel[QO_MAX_LAYERS];
+    const float* act_param_channel[QO_MAX_LAYERS];
     const float* W[QO_MAX_LAYERS];         /* row-major (cout, cin) */
     const float* b[QO_MAX_LAYERS];         /* NULL if no bias */
     float* dW[QO_MAX_LAYERS];              /* += ; may be NULL */

@@ -64,6 +64,7 @@ class NetworkStruct(ctypes.Structure):
         ("n_layers", ctypes.c_int),
         ("cin", ctypes.c_int * MAX_LAYERS), ("cout", ctypes.c_int * MAX_LAYERS),
         ("act", ctypes.c_int * MAX_LAYERS), ("act_param", ctypes.c_float * MAX_LAYERS),
+        ("act_channel", ctypes.POINTER(ctypes.c_int) * MAX_LAYERS), ("act_param_channel", _fp * MAX_LAYERS),
         ("W", _fp * MAX_LAYERS), ("b", _fp * MAX_LAYERS),
         ("dW", _fp * MAX_LAYERS), ("db", _fp * MAX_LAYERS),
         ("round_mode", ctypes.c_int), ("res_factor", ctypes.c_int),
@@ -290,10 +291,16 @@ class Network:
         prev = encoded
         for l in cfg["network"]:
             a = l["activation"]
+            per_channel = None
             if not isinstance(a, str):
-                raise ValueError("per-channel activations are not supported")
+                # one activation per output channel (fused_network.cpp:112-125); channels of
+                # the padding take the last one
+                if len(a) != int(l["n_out"]):
+                    raise ValueError("the number of activations must match the number of output channels")
+                per_channel = [acts[x] for x in a]
+                a = a[-1]
             self.layers.append(dict(cin=prev, cout=int(l["n_out"]), bias=bool(l["bias"]),
-                                    act=acts[a]))
+                                    act=acts[a], act_channels=per_channel))
             prev = int(l["n_out"])
         if prev != self.n_out:
             raise ValueError("last layer width does not match num_outputs")
@@ -367,6 +374,13 @@ class Network:
         for i, l in enumerate(self.layers):
             s.cin[i], s.cout[i] = l["cin"], l["cout"]
             s.act[i], s.act_param[i] = l["act"]
+            if l["act_channels"] is not None:
+                chans = list(l["act_channels"]) + [l["act_channels"][-1]] * (l["cout"] - len(l["act_channels"]))
+                kinds = np.array([c[0] for c in chans], dtype=np.int32)
+                prms = np.array([c[1] for c in chans], dtype=np.float32)
+                keep += [kinds, prms]
+                s.act_channel[i] = kinds.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+                s.act_param_channel[i] = _ptr(prms)
             w = np.ascontiguousarray(self.weight(i))
             keep.append(w)
             s.W[i] = _ptr(w)

@@ -257,6 +257,10 @@ private:
     // global memory, -1 for resident layers; returns their total size in halves
     size_t transposedWeightLayout(int adjointFlags, std::vector<long long>& offsets) const;
     int ldsParamHalves(bool adjoint) const;
+    // definitions of all activations in use, plus one composite per layer with per-channel activations
+    std::string activationDefinitions() const;
+    // name (inside namespace activations) of the activation type of a layer
+    std::string activationTypeName(int layer) const;
     int stageBytesPerWave(bool adjoint) const;
     std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);
     void ensureStreams();

@@ -128,6 +128,33 @@ struct HasPackedForward<Act, decltype(void(Act::forward4(f16x4{})))>
     static constexpr bool value = true;
 };
 
+/** Detects composites with one activation per channel (forwardAt / adjointAt with a channel). */
+template <typename Act, typename = void>
+struct IsPerChannel
+{
+    static constexpr bool value = false;
+};
+template <typename Act>
+struct IsPerChannel<Act, decltype(void(Act::PerChannel))>
+{
+    static constexpr bool value = true;
+};
+
+/** Activation of 4 values that belong to the consecutive channels channel0 .. channel0+3. */
+template <typename Act>
+__device__ __forceinline__ f16x4 activationForwardChannels(f16x4 v, int channel0);
+
+/** Activation of values that all belong to the same channel. */
+template <typename Act>
+__device__ __forceinline__ f16x8 activationForwardChannel(f16x8 v, int channel);
+
+template <typename Act>
+__device__ __forceinline__ half activationAdjointChannel(half x, half adjz, int channel)
+{
+    if constexpr (IsPerChannel<Act>::value) return Act::adjointAt(x, adjz, channel);
+    else return Act::adjoint(x, adjz);
+}
+
 template <typename Act>
 __device__ __forceinline__ f16x4 activationForward(f16x4 v)
 {
@@ -147,6 +174,32 @@ __device__ __forceinline__ f16x8 activationForward(f16x8 v)
     const f16x4 lo = activationForward<Act>(f16x4{v[0], v[1], v[2], v[3]});
     const f16x4 hi = activationForward<Act>(f16x4{v[4], v[5], v[6], v[7]});
     return concat(lo, hi);
+}
+
+template <typename Act>
+__device__ __forceinline__ f16x4 activationForwardChannels(f16x4 v, int channel0)
+{
+    if constexpr (IsPerChannel<Act>::value) {
+        f16x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = fromHalf(Act::forwardAt(toHalf(v[i]), channel0 + i));
+        return o;
+    } else {
+        return activationForward<Act>(v);
+    }
+}
+
+template <typename Act>
+__device__ __forceinline__ f16x8 activationForwardChannel(f16x8 v, int channel)
+{
+    if constexpr (IsPerChannel<Act>::value) {
+        f16x8 o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = fromHalf(Act::forwardAt(toHalf(v[i]), channel));
+        return o;
+    } else {
+        return activationForward<Act>(v);
+    }
 }
 
 /** One row of a strided 2-D tensor. */

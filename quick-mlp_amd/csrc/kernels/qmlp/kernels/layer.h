@@ -34,7 +34,8 @@ __device__ __forceinline__ f32x4 mfma32(f16x8 a, f16x8 b, f32x4 c)
  * \tparam CIN padded input channels (multiple of 16)
  * \tparam COUT padded output channels (multiple of 16)
  * \tparam BIAS layer has a bias vector
- * \tparam Activation struct with static half forward(half), half adjoint(half x, half adjz)
+ * \tparam Activation struct with static half forward(half), half adjoint(half x, half adjz), or a
+ *         per-channel composite with forwardAt(half, channel), adjointAt(half x, half adjz, channel)
  */
 template <int CIN, int COUT, bool BIAS, typename Activation>
 struct Layer
@@ -185,7 +186,7 @@ struct Layer
                 }
             }
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) y[nt][m] = activationForward<Activation>(p[nt]);
+            for (int nt = 0; nt < NT; ++nt) y[nt][m] = activationForwardChannels<Activation>(p[nt], 16 * m + 4 * g);
         }
     }
 
@@ -214,7 +215,7 @@ struct Layer
                 f16x4 d;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const half a = Activation::adjoint(toHalf(pre[nt]), toHalf(dy[nt][m][i]));
+                    const half a = activationAdjointChannel<Activation>(toHalf(pre[nt]), toHalf(dy[nt][m][i]), 16 * m + 4 * g + i);
                     d[nt] = ((validMask >> nt) & 1) ? fromHalf(a) : static_cast<f16>(0);
                     dy[nt][m][i] = d[nt];
                 }

@@ -86,7 +86,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
 #pragma unroll
             for (int mi = 0; mi < KT; ++mi) {
                 const f16x8 raw = *reinterpret_cast<const f16x8*>(bTile + (16 * mi + r) * TILE_POINTS + 32 * kb + 8 * g);
-                b[mi] = activationForward<InputActivation>(raw);
+                b[mi] = activationForwardChannel<InputActivation>(raw, 16 * mi + r);
             }
 #pragma unroll
             for (int mo = 0; mo < MO_CHUNK; ++mo) {

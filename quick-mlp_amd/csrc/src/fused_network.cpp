@@ -322,12 +322,7 @@ void FusedNetwork::fillEncodingsAndActivations(std::string& codeTemplate) const
     replaceAll(codeTemplate, "$$INCLUDES$$", encodingIncludes.str());
     replaceAll(codeTemplate, "$$ENCODING_PARAMETERS$$", encodingParameters.str());
 
-    std::stringstream activationDefinitions;
-    std::unordered_set<std::string> activationIDs;
-    for (const auto& l : layers_)
-        for (const auto& a : l.activations)
-            if (activationIDs.insert(a->id()).second) activationDefinitions << a->code() << "\n";
-    replaceAll(codeTemplate, "$$DEFINE_ACTIVATIONS$$", activationDefinitions.str());
+    replaceAll(codeTemplate, "$$DEFINE_ACTIVATIONS$$", activationDefinitions());
 
     replaceAll(codeTemplate, "$$NUM_INPUTS$$", std::to_string(channelsIn_));
     replaceAll(codeTemplate, "$$ENCODED_CHANNELS$$", std::to_string(encodedChannels_));
@@ -417,6 +412,54 @@ size_t FusedNetwork::transposedWeightLayout(int adjointFlags, std::vector<long l
         n += static_cast<size_t>(layers_[i].channelsIn) * layers_[i].channelsOut;
     }
     return n;
+}
+
+std::string FusedNetwork::activationTypeName(int layer) const
+{
+    const auto& a = layers_[layer].activations;
+    return a.size() == 1 ? a[0]->id() : "mixed_layer" + std::to_string(layer) + "_";
+}
+
+std::string FusedNetwork::activationDefinitions() const
+{
+    std::stringstream ss;
+    std::unordered_set<std::string> ids;
+    for (const auto& l : layers_)
+        for (const auto& a : l.activations)
+            if (ids.insert(a->id()).second) ss << a->code() << "\n";
+    // One activation per output channel (the reference parses such lists and then rejects them,
+    // fused_network.cpp:112-125,447): a composite that dispatches on the channel. Channels of
+    // the padding use the activation of the last listed channel.
+    for (size_t layer = 0; layer < layers_.size(); ++layer) {
+        const auto& l = layers_[layer];
+        if (l.activations.size() == 1) continue;
+        std::vector<std::string> kinds;
+        std::vector<int> kindOfChannel;
+        for (const auto& a : l.activations) {
+            auto it = std::find(kinds.begin(), kinds.end(), a->id());
+            if (it == kinds.end()) {
+                kinds.push_back(a->id());
+                it = kinds.end() - 1;
+            }
+            kindOfChannel.push_back(static_cast<int>(it - kinds.begin()));
+        }
+        while (static_cast<int>(kindOfChannel.size()) < l.channelsOut) kindOfChannel.push_back(kindOfChannel.back());
+        ss << "struct " << activationTypeName(static_cast<int>(layer)) << "\n{\n"
+           << "    static constexpr bool PerChannel = true;\n"
+           << "    static __device__ __forceinline__ int kind(int channel) {\n"
+           << "        constexpr unsigned char kinds[" << kindOfChannel.size() << "] = {";
+        for (size_t i = 0; i < kindOfChannel.size(); ++i) ss << (i ? "," : "") << kindOfChannel[i];
+        ss << "};\n        return kinds[channel];\n    }\n"
+           << "    static __device__ __forceinline__ half forwardAt(half x, int channel) {\n        switch (kind(channel)) {\n";
+        for (size_t k = 0; k + 1 < kinds.size(); ++k)
+            ss << "        case " << k << ": return " << kinds[k] << "::forward(x);\n";
+        ss << "        default: return " << kinds.back() << "::forward(x);\n        }\n    }\n"
+           << "    static __device__ __forceinline__ half adjointAt(half x, half adjz, int channel) {\n        switch (kind(channel)) {\n";
+        for (size_t k = 0; k + 1 < kinds.size(); ++k)
+            ss << "        case " << k << ": return " << kinds[k] << "::adjoint(x, adjz);\n";
+        ss << "        default: return " << kinds.back() << "::adjoint(x, adjz);\n        }\n    }\n};\n";
+    }
+    return ss.str();
 }
 
 int FusedNetwork::ldsParamHalves(bool adjoint) const
@@ -509,9 +552,9 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
 
     std::vector<std::string> layerTypes;
     for (const auto& l : layers_) {
-        if (l.activations.size() > 1) throw std::runtime_error("Individual activations per channel are not implemented yet");
         layerTypes.push_back(format("Layer<%d, %d, %s, activations::%s>", l.channelsIn, l.channelsOut,
-                                    l.useBias ? "true" : "false", l.activations[0]->id().c_str()));
+                                    l.useBias ? "true" : "false",
+                                    activationTypeName(static_cast<int>(&l - layers_.data())).c_str()));
     }
 
     std::stringstream stage;
@@ -581,9 +624,9 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
 
     std::vector<std::string> layerTypes;
     for (const auto& l : layers_) {
-        if (l.activations.size() > 1) throw std::runtime_error("Individual activations per channel are not implemented yet");
         layerTypes.push_back(format("Layer<%d, %d, %s, activations::%s>", l.channelsIn, l.channelsOut,
-                                    l.useBias ? "true" : "false", l.activations[0]->id().c_str()));
+                                    l.useBias ? "true" : "false",
+                                    activationTypeName(static_cast<int>(&l - layers_.data())).c_str()));
     }
 
     // the first layer's transposed weights are only needed when something consumes dX0
@@ -651,12 +694,7 @@ std::string FusedNetwork::weightUpdateSource(int blockSize) const
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string code = kl->findFile("qmlp/kernels/network_weight_update.h").value();
-    std::stringstream activationDefinitions;
-    std::unordered_set<std::string> activationIDs;
-    for (const auto& l : layers_)
-        for (const auto& a : l.activations)
-            if (activationIDs.insert(a->id()).second) activationDefinitions << a->code() << "\n";
-    replaceAll(code, "$$DEFINE_ACTIVATIONS$$", activationDefinitions.str());
+    replaceAll(code, "$$DEFINE_ACTIVATIONS$$", activationDefinitions());
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
     return code;
 }
@@ -672,9 +710,7 @@ std::string FusedNetwork::weightUpdateKernelName(int layer, int& numChunks) cons
     numChunks = mt / moChunk;
     std::string inputActivation = "qmlp::kernel::activations::passthrough_";
     if (layer > 0) {
-        const auto& prev = layers_[layer - 1].activations;
-        if (prev.size() > 1) throw std::runtime_error("Individual activations per channel are not implemented yet");
-        inputActivation = "qmlp::kernel::activations::" + prev[0]->id();
+        inputActivation = "qmlp::kernel::activations::" + activationTypeName(layer - 1);
     }
     return format("qmlp::kernel::WeightUpdateKernel<%d, %d, %s, %s, %d>", l.channelsIn, l.channelsOut,
                   l.useBias ? "true" : "false", inputActivation.c_str(), moChunk);

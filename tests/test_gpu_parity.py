@@ -58,6 +58,31 @@ def test_two_layers_against_oracle(c0, c1, c2, acts):
     check_gradients(case, X, one, FLAG_INPUT, case.gpu_train(X, one, FLAG_INPUT), kinks, "single entry: ")
 
 
+def test_one_activation_per_channel():
+    """Lists of activations, one per output channel (the reference parses them and then throws,
+    src_cpp/src/fused_network.cpp:112-125,447)."""
+    acts0 = ["relu", "sine", "celu", "identity"] * 5
+    acts1 = ["sine", "identity", "celu", "celu", "sine"]
+    case = Case(identity_cfg(16, [20, 5], [acts0, acts1], [True, False]))
+    rng = np.random.default_rng(31)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    N = 700
+    X = rng.uniform(-1, 1, (N, 16)).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 5)) / 8).astype(np.float32)
+    assert_close(case.gpu_inference(X), case.oracle.forward(X), "inference")
+    flags = FLAG_INPUT | FLAG_WEIGHTS
+    got = case.gpu_train(X, adj, flags)
+    assert_close(got["out"], case.oracle.forward(X), "forward")
+    check_gradients(case, X, adj, flags, got, kinks=True)
+    # a uniform list equals the single name
+    same = Case(identity_cfg(16, [20, 5], [["celu"] * 20, "identity"], [True, False]))
+    single = Case(identity_cfg(16, [20, 5], ["celu", "identity"], [True, False]))
+    p = random_parameters(single.oracle, rng)
+    same.set_parameters(p)
+    single.set_parameters(p)
+    assert np.array_equal(same.gpu_inference(X), single.gpu_inference(X))
+
+
 @pytest.mark.parametrize("widths,act", [([128] * 6 + [16], "celu"), ([256, 256, 256, 3], "sine"), ([512, 208, 16], "identity")])
 def test_networks_whose_weights_exceed_the_lds(widths, act):
     """More than 160 KB of fp16 weights: some layers stay in LDS, the kernels read the others

@@ -111,6 +111,7 @@ BASE = bc.CONFIGS[1]["cfg"]
     (lambda c: c["encodings"][0].update(n_in=4), 1, "out of bounds"),
     (lambda c: c["network"][0].update(activation="gelu"), 1, "No activation with id 'gelu'"),
     (lambda c: c["network"][0].update(activation=["relu"] * 3), 1, "must match the number of output channels"),
+    (lambda c: c["network"][0].update(activation=["relu"] * 15 + [3]), 1, "must be specified as a string"),
     (lambda c: c.pop("num_inputs"), 1, "num_inputs"),
     (lambda c: c.update(activation_specification=["does-not-exist.json"]), 1, "could not be resolved"),
     (lambda c: c.update(activation_specification=[{"id": "1bad", "forward": "z=x", "adjoint": "adjx=adjz"}]), 1,

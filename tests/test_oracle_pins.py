@@ -403,7 +403,12 @@ def torch_mlp(net, X, adj, params):
         W = p[l["w_start"]: l["w_start"] + l["cin"] * l["cout"]].reshape(l["cout"], l["cin"])
         b = p[l["b_start"]: l["b_start"] + l["cout"]] if l["bias"] else None
         h = torch.nn.functional.linear(h, W, b)
-        h = TORCH_ACT[net.cfg["network"][i]["activation"]](h)
+        a = net.cfg["network"][i]["activation"]
+        if isinstance(a, str):
+            h = TORCH_ACT[a](h)
+        else:   # one activation per channel; the padding takes the last one
+            a = list(a) + [a[-1]] * (l["cout"] - len(a))
+            h = torch.stack([TORCH_ACT[a[c]](h[:, c]) for c in range(l["cout"])], dim=1)
     out = h[:, :net.n_out]
     (out * torch.from_numpy(adj)).sum().backward()
     return out.detach().numpy(), x.grad.numpy(), p.grad.numpy()
@@ -416,7 +421,8 @@ def torch_mlp(net, X, adj, params):
     (20, [16, 24], ["identity", "identity"], [False, False], 32),
     (3, [16, 1], ["relu", "relu"], [True, True], 513),
     (4, [128, 64, 48, 4], ["sine", "sine", "celu", "identity"], [True, True, True, True], 128),
-    (5, [32, 48, 16], ["celu", "relu", "identity"], [False, True, False], 16)])
+    (5, [32, 48, 16], ["celu", "relu", "identity"], [False, True, False], 16),
+    (7, [20, 5], [["relu", "sine", "celu", "identity"] * 5, ["sine", "identity", "relu", "relu", "celu"]], [True, False], 64)])
 def test_mlp_matches_torch_linear_autograd(n_in, widths, acts, biases, N):
     net = qo.Network(mlp_cfg(n_in, widths, acts, biases))
     rng = np.random.default_rng(42)
