@@ -248,11 +248,17 @@ private:
     int weightUpdateBlockSize() const;
     // number of batch slices whose partial weight gradients are kept in the adjoint memory
     int weightUpdateSlices(int numTiles) const;
-    // Layers whose weights stay in LDS for the whole kernel; the others are read from global
-    // memory by every wavefront (networks whose weights exceed the LDS).
-    std::vector<char> ldsResidency(bool adjoint) const;
-    // offsets in halves; -1 for weights that are not resident
-    int ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const;
+    // Where a kernel finds the weights of a layer. RESIDENT: in LDS for the whole kernel.
+    // STREAMED: staged into a shared LDS buffer by the whole workgroup right before the layer
+    // runs, for every group of tiles (networks whose weights exceed the LDS). GLOBAL: gathered
+    // from global memory by every wavefront (single layers that exceed the LDS on their own).
+    enum WeightPlacement { WEIGHTS_RESIDENT = 0, WEIGHTS_STREAMED = 1, WEIGHTS_GLOBAL = 2 };
+    std::vector<int> weightPlacement(bool adjoint) const;
+    // LDS offsets in halves: resident weights, then biases (forward), then the stream buffer
+    // (streamOffset, -1 if no layer is streamed); weightOffsets is -1 for global layers and
+    // streamOffset for streamed ones. Returns the total size in halves.
+    int ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets,
+                  int* streamOffset = nullptr) const;
     // offsets (in halves) of the transposed copies of the weights the adjoint kernel reads from
     // global memory, -1 for resident layers; returns their total size in halves
     size_t transposedWeightLayout(int adjointFlags, std::vector<long long>& offsets) const;

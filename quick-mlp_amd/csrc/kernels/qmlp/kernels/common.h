@@ -99,6 +99,22 @@ __device__ __forceinline__ void waveLdsSync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+/**
+ * Makes the compiler materialise the activations of a tile at this point of the program.
+ * Used in front of workgroup barriers inside the layer sequence: otherwise the matrix
+ * instructions that produce them are sunk behind the barrier (they touch no memory), while
+ * the LDS reads feeding them have to stay in front of it, and the operands of whole layers
+ * end up spilled to scratch memory in between.
+ */
+template <int A, int B>
+__device__ __forceinline__ void materialize(f16x4 (&x)[A][B])
+{
+#pragma unroll
+    for (int a = 0; a < A; ++a)
+#pragma unroll
+        for (int b = 0; b < B; ++b) asm volatile("" : "+v"(x[a][b]));
+}
+
 /** Row of the per-wave staging area that holds point p (0..63) of the tile. Points
  *  4r+nt (fixed nt) of the 16 lanes r land in 16 consecutive rows, which together with
  *  an odd multiple of 16 bytes as row stride makes the tile reads bank-conflict free. */

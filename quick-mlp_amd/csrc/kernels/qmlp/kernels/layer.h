@@ -53,44 +53,66 @@ struct Layer
     static constexpr int A_LDS_HALVES = KT * A_MSTRIDE;
 
     /**
-     * Copies the row-major (COUT, CIN) weight matrix into LDS in forward operand
-     * order. Called by all threads of the block; 'W' must be 8-byte aligned.
+     * Copies the row-major (COUT, CIN) weight matrix into LDS in forward operand order.
+     * Called by all threads of the block; 'W' must be 16-byte aligned. The matrix is read in
+     * memory order with 16-byte loads, four of them in flight per thread (layers that are
+     * streamed through LDS are staged once per group of tiles, so this is on the critical
+     * path there), and scattered into the operand layout.
      */
     __device__ static void stageForward(const f16* __restrict__ W, f16* __restrict__ dst, int tid, int nthreads)
     {
-        // one unit = 4 consecutive halves of a weight row
-        constexpr int UNITS = F_LDS_HALVES / 4;
-        for (int u = tid; u < UNITS; u += nthreads) {
-            const int m = u / (F_MSTRIDE / 4);
-            int rest = u - m * (F_MSTRIDE / 4);
-            const int kb = rest / 128;
-            rest -= kb * 128;
-            const int lane = rest >> 1;
-            const int tile = 2 * kb + (rest & 1);
-            const int g = lane >> 4, r = lane & 15;
-            f16x4 v = {0, 0, 0, 0};
-            if (tile < KT) v = *reinterpret_cast<const f16x4*>(W + (16 * m + r) * CIN + 16 * tile + 4 * g);
-            *reinterpret_cast<f16x4*>(dst + 4 * u) = v;
+        if constexpr ((KT & 1) != 0) {
+            // the upper half of the last k-block has no channels: zero
+            for (int u = tid; u < MT * 64; u += nthreads)
+                *reinterpret_cast<f16x4*>(dst + (u >> 6) * F_MSTRIDE + (F_KB - 1) * 512 + (u & 63) * 8 + 4) = f16x4{0, 0, 0, 0};
+        }
+        constexpr int NV = COUT * CIN / 8;   // 16-byte pieces
+        constexpr int INFLIGHT = 4;
+        for (int v0 = tid; v0 < NV; v0 += nthreads * INFLIGHT) {
+            f16x8 val[INFLIGHT];
+#pragma unroll
+            for (int j = 0; j < INFLIGHT; ++j) {
+                const int v = v0 + j * nthreads;
+                if (v < NV) val[j] = *reinterpret_cast<const f16x8*>(W + v * 8);
+            }
+#pragma unroll
+            for (int j = 0; j < INFLIGHT; ++j) {
+                const int v = v0 + j * nthreads;
+                if (v >= NV) continue;
+                const int o = (v * 8) / CIN, k = (v * 8) % CIN;
+                const int m = o >> 4, r = o & 15, tile = k >> 4, g = (k & 15) >> 2;   // g is 0 or 2
+                f16* base = dst + m * F_MSTRIDE + (tile >> 1) * 512 + (tile & 1) * 4 + r * 8;
+                *reinterpret_cast<f16x4*>(base + (16 * g) * 8) = f16x4{val[j][0], val[j][1], val[j][2], val[j][3]};
+                *reinterpret_cast<f16x4*>(base + (16 * (g + 1)) * 8) = f16x4{val[j][4], val[j][5], val[j][6], val[j][7]};
+            }
         }
     }
 
     /**
-     * Copies the weight matrix into LDS in adjoint operand order (A = tiles of W^T).
+     * Copies the weight matrix into LDS in adjoint operand order (A = tiles of W^T): a thread
+     * reads 8 consecutive columns of 4 consecutive rows (four 16-byte loads) and writes, per
+     * column, the 4 row values that are neighbours in the operand.
      */
     __device__ static void stageAdjoint(const f16* __restrict__ W, f16* __restrict__ dst, int tid, int nthreads)
     {
-        constexpr int N = A_LDS_HALVES;
-        for (int e = tid; e < N; e += nthreads) {
-            const int mi = e / A_MSTRIDE;
-            int rest = e - mi * A_MSTRIDE;
-            const int kb = rest / 512;
-            rest -= kb * 512;
-            const int lane = rest >> 3;
-            const int slot = rest & 7;
-            const int tile = 2 * kb + (slot >> 2);
-            const int j = slot & 3;
-            const int g = lane >> 4, r = lane & 15;
-            dst[e] = tile < MT ? W[(16 * tile + 4 * g + j) * CIN + 16 * mi + r] : static_cast<f16>(0);
+        if constexpr ((MT & 1) != 0) {
+            for (int u = tid; u < KT * 64; u += nthreads)
+                *reinterpret_cast<f16x4*>(dst + (u >> 6) * A_MSTRIDE + (A_KB - 1) * 512 + (u & 63) * 8 + 4) = f16x4{0, 0, 0, 0};
+        }
+        constexpr int COLS8 = CIN / 8;
+        constexpr int ITEMS = (COUT / 4) * COLS8;
+        for (int item = tid; item < ITEMS; item += nthreads) {
+            const int q = item / COLS8, k0 = (item % COLS8) * 8;
+            const int o0 = 4 * q;                       // rows o0..o0+3: same tile and lane group, j = 0..3
+            f16x8 rows[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) rows[j] = *reinterpret_cast<const f16x8*>(W + (o0 + j) * CIN + k0);
+            const int tile = o0 >> 4, g = (o0 & 15) >> 2;
+            const int mi = k0 >> 4, r0 = k0 & 15;
+            f16* base = dst + mi * A_MSTRIDE + (tile >> 1) * 512 + (tile & 1) * 4 + (16 * g + r0) * 8;
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                *reinterpret_cast<f16x4*>(base + c * 8) = f16x4{rows[0][c], rows[1][c], rows[2][c], rows[3][c]};
         }
     }
 
@@ -141,7 +163,7 @@ struct Layer
      * \param bias LDS bias vector (COUT halves) or nullptr
      * \param x input activations: x[nt][t] = channels 16t+4g+{0..3} of point 4r+nt
      * \param y output activations in the same layout
-     * \param preTile [STORE] where the pre-activations of this tile go: (COUT, 64) halves,
+     * \param preTile [STORE] where the pre-activations of this tile go (nullptr: nowhere): (COUT, 64) halves,
      *        channel-major, so that both the adjoint pass (per channel, 4 points of one
      *        lane) and the weight update (per channel, 8 consecutive points) read it
      *        with wide loads
@@ -178,7 +200,7 @@ struct Layer
             f16x4 p[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) p[nt] = toF16(acc[nt]);
-            if constexpr (STORE) {
+            if (STORE && preTile != nullptr) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const f16x4 v = {p[0][i], p[1][i], p[2][i], p[3][i]};
@@ -219,7 +241,7 @@ struct Layer
                     d[nt] = ((validMask >> nt) & 1) ? fromHalf(a) : static_cast<f16>(0);
                     dy[nt][m][i] = d[nt];
                 }
-                if constexpr (STORE_DPRE)
+                if (STORE_DPRE && dpreTile != nullptr)
                     *reinterpret_cast<f16x4*>(dpreTile + (16 * m + 4 * g + i) * TILE_POINTS + 4 * r) = d;
             }
         }

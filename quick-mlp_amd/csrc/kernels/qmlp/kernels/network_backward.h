@@ -70,6 +70,10 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
     constexpr bool HAS_INPUT_GRADIENTS = $$HAS_INPUT_GRADIENTS$$;
     constexpr bool HAS_NETWORK_GRADIENTS = $$HAS_NETWORK_GRADIENTS$$;
     constexpr bool HAS_ENCODING_GRADIENTS = $$HAS_ENCODING_GRADIENTS$$;
+    // Some layers' weights are staged into a shared LDS buffer right before the layer runs:
+    // the wavefronts of the workgroup then walk the tiles and layers in lockstep (workgroup
+    // barriers inside the loop), wavefronts without a tile work on zeros.
+    constexpr bool HAS_STREAMED_LAYERS = $$HAS_STREAMED_LAYERS$$;
     // the adjoint of the encoded input is only needed if something sits behind it
     constexpr bool NEEDS_ENCODING_ADJOINT = HAS_INPUT_GRADIENTS || HAS_ENCODING_GRADIENTS;
     (void)ENCODED_CHANNELS; (void)NUM_INPUTS; (void)KT0; (void)STAGE_STRIDE;
@@ -95,8 +99,18 @@ $$STAGE_PARAMETERS$$
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
     const int actualChannelsOut = adjOutputs.sizes_[1];
-    for (int tile = blockIdx.x * WAVES + wave; tile < numTiles; tile += gridDim.x * WAVES)
+    for (int tileBase = blockIdx.x * WAVES; tileBase < numTiles; tileBase += gridDim.x * WAVES)
     {
+        const int tile = tileBase + wave;
+        if (!HAS_STREAMED_LAYERS && tile >= numTiles) continue;
+        const bool tileValid = tile < numTiles;
+        const int tileRead = tileValid ? tile : numTiles - 1;   // stored intermediates are read from a valid tile
+        (void)tileRead;
+        // The weights in LDS do not change between the tiles; an offset the compiler cannot see
+        // through keeps it from hoisting their reads out of this loop (it then spills them).
+        int ldsOffset = 0;
+        asm volatile("" : "+s"(ldsOffset));
+        const f16* sWeights = sParams + ldsOffset;
         // dL/dy -> accumulator layout (fp32 -> fp16), zero outside batch / real channels
         f16x4 dyOut[NT][MTL];
         int validMask = 0;

@@ -50,6 +50,10 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     constexpr int LDS_PARAM_HALVES = $$LDS_PARAM_HALVES$$;
     constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
     constexpr int PPL = $$POINTS_PER_LANE$$;              // tiles a wave encodes together
+    // Some layers' weights are staged into a shared LDS buffer right before the layer runs:
+    // the wavefronts of the workgroup then walk the tiles and layers in lockstep (workgroup
+    // barriers inside the loops), wavefronts without a tile compute on zero rows.
+    constexpr bool HAS_STREAMED_LAYERS = $$HAS_STREAMED_LAYERS$$;
 
     const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
     f16* __restrict__ forwardTmpMemory = reinterpret_cast<f16*>(forwardTmpMemoryH);
@@ -68,8 +72,11 @@ $$STAGE_PARAMETERS$$
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
     (void)numel64;
-    for (int tile0 = (blockIdx.x * WAVES + wave) * PPL; tile0 < numTiles; tile0 += gridDim.x * WAVES * PPL)
+    for (int tileBase = blockIdx.x * WAVES * PPL; tileBase < numTiles; tileBase += gridDim.x * WAVES * PPL)
     {
+        const int tile0 = tileBase + wave * PPL;
+        if (!HAS_STREAMED_LAYERS && tile0 >= numTiles) continue;
+
         // encodings: PPL points per lane (one of each tile), each into its staging row.
         // Rows outside the batch are evaluated at the origin and zeroed afterwards so that
         // no NaN enters the matrix cores.
@@ -107,7 +114,13 @@ $$CALL_ENCODINGS$$
         for (int q = 0; q < PPL; ++q)
         {
         const int tile = tile0 + q;
-        if (tile >= numTiles) break;
+        if (!HAS_STREAMED_LAYERS && tile >= numTiles) break;
+        const bool tileValid = tile < numTiles;
+        // The weights in LDS do not change between the tiles; an offset the compiler cannot see
+        // through keeps it from hoisting their reads out of the loops (it then spills them).
+        int ldsOffset = 0;
+        asm volatile("" : "+s"(ldsOffset));
+        const f16* sWeights = sParams + ldsOffset;
         const f16* sTile = sStage + q * (TILE_POINTS * STAGE_STRIDE);
 
         // B operands of the first layer
@@ -118,7 +131,7 @@ $$CALL_ENCODINGS$$
             for (int t = 0; t < KT0; ++t)
                 x0[nt][t] = *reinterpret_cast<const f16x4*>(sTile + Stage::chunkOffset(16 * nt + r, 4 * t + g));
 
-        if constexpr (STORE) {
+        if (STORE && tileValid) {
             // encoded input, channel-major per tile, for the weight update of layer 0
             f16* encTile = forwardTmpMemory + static_cast<long long>(tile) * (CHANNELS_IN * TILE_POINTS);
 #pragma unroll

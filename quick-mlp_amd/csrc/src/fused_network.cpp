@@ -336,10 +336,10 @@ static int ldsWeightHalves(int channelsIn, int channelsOut, bool adjoint)
     return adjoint ? channelsIn * roundUp(channelsOut, 32) : channelsOut * roundUp(channelsIn, 32);
 }
 
-std::vector<char> FusedNetwork::ldsResidency(bool adjoint) const
+std::vector<int> FusedNetwork::weightPlacement(bool adjoint) const
 {
     const int L = static_cast<int>(layers_.size());
-    std::vector<char> resident(L, 1);
+    std::vector<int> placement(L, WEIGHTS_RESIDENT);
     std::vector<long long> bytes(L);
     long long total = 0, biases = 0;
     for (int i = 0; i < L; ++i) {
@@ -349,46 +349,68 @@ std::vector<char> FusedNetwork::ldsResidency(bool adjoint) const
     }
     const long long maxLds = MaxSharedMemoryBytes();
     // everything stays if four wavefronts still find room for their staging tiles
-    if (total + biases + 16 + 4ll * stageBytesPerWave(adjoint) <= maxLds) return resident;
-    // otherwise keep the subset with the most bytes that leaves room for eight wavefronts
-    const long long budget = maxLds - biases - 16 - 8ll * stageBytesPerWave(adjoint);
-    long long best = -1;
-    unsigned bestMask = 0;
-    if (L <= 20) {
-        for (unsigned mask = 0; mask < (1u << L); ++mask) {
-            long long sum = 0;
-            for (int i = 0; i < L; ++i)
-                if (mask & (1u << i)) sum += bytes[i];
-            if (sum <= budget && sum > best) {
-                best = sum;
+    if (total + biases + 16 + 4ll * stageBytesPerWave(adjoint) <= maxLds) return placement;
+
+    // Otherwise the workgroup shares a stream buffer as large as the largest streamed layer; of
+    // the layers that fit into such a buffer, the subset with the most bytes that still fits
+    // beside it stays resident. Room is left for the staging tiles of eight wavefronts, or of
+    // four if that lets a layer be streamed that would otherwise have to be read from global
+    // memory by every wavefront.
+    auto place = [&](int waves, std::vector<int>& out) {
+        out.assign(L, WEIGHTS_RESIDENT);
+        const long long budget = maxLds - biases - 16 - static_cast<long long>(waves) * stageBytesPerWave(adjoint);
+        std::vector<int> candidates;
+        int numGlobal = 0;
+        for (int i = 0; i < L; ++i) {
+            if (bytes[i] > budget) {
+                out[i] = WEIGHTS_GLOBAL;
+                ++numGlobal;
+            } else {
+                candidates.push_back(i);
+            }
+        }
+        const int C = static_cast<int>(candidates.size());
+        long long best = -1;
+        unsigned bestMask = 0;
+        const unsigned numMasks = C <= 16 ? (1u << C) : 1u;   // many layers: stream them all
+        for (unsigned mask = 0; mask < numMasks; ++mask) {
+            long long resident = 0, stream = 0;
+            for (int k = 0; k < C; ++k) {
+                if (mask & (1u << k)) resident += bytes[candidates[k]];
+                else stream = std::max(stream, bytes[candidates[k]]);
+            }
+            if (resident + stream <= budget && resident > best) {
+                best = resident;
                 bestMask = mask;
             }
         }
-    } else {
-        long long sum = 0;
-        for (int i = 0; i < L; ++i)
-            if (sum + bytes[i] <= budget) {
-                sum += bytes[i];
-                bestMask |= 1u << i;
-            }
+        for (int k = 0; k < C; ++k) out[candidates[k]] = (bestMask >> k) & 1 ? WEIGHTS_RESIDENT : WEIGHTS_STREAMED;
+        return numGlobal;
+    };
+    const int globalWithEight = place(8, placement);
+    if (globalWithEight > 0) {
+        std::vector<int> withFour;
+        if (place(4, withFour) < globalWithEight) placement = withFour;
     }
-    for (int i = 0; i < L; ++i) resident[i] = (bestMask >> i) & 1;
-    return resident;
+    return placement;
 }
 
-int FusedNetwork::ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets) const
+int FusedNetwork::ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::vector<int>& biasOffsets,
+                            int* streamOffset) const
 {
     // Weights sit in LDS in matrix-core operand order, contraction width padded to 32
     // channels (forward: C_in, adjoint: C_out); the biases follow (forward only).
     weightOffsets.assign(layers_.size(), -1);
     biasOffsets.assign(layers_.size(), 0);
-    const auto resident = ldsResidency(adjoint);
-    int n = 0;
+    const auto placement = weightPlacement(adjoint);
+    int n = 0, streamHalves = 0;
     for (size_t i = 0; i < layers_.size(); ++i) {
-        if (!resident[i]) continue;
         const auto& l = layers_[i];
+        const int halves = ldsWeightHalves(l.channelsIn, l.channelsOut, adjoint);
+        if (placement[i] == WEIGHTS_STREAMED) streamHalves = std::max(streamHalves, halves);
+        if (placement[i] != WEIGHTS_RESIDENT) continue;
         weightOffsets[i] = n;
-        n += ldsWeightHalves(l.channelsIn, l.channelsOut, adjoint);
+        n += halves;
     }
     if (!adjoint) {
         for (size_t i = 0; i < layers_.size(); ++i) {
@@ -397,17 +419,21 @@ int FusedNetwork::ldsLayout(bool adjoint, std::vector<int>& weightOffsets, std::
             n += layers_[i].channelsOut;
         }
     }
-    return roundUp(n, 8);
+    n = roundUp(n, 8);
+    if (streamOffset) *streamOffset = streamHalves > 0 ? n : -1;
+    for (size_t i = 0; i < layers_.size(); ++i)
+        if (placement[i] == WEIGHTS_STREAMED) weightOffsets[i] = n;
+    return roundUp(n + streamHalves, 8);
 }
 
 size_t FusedNetwork::transposedWeightLayout(int adjointFlags, std::vector<long long>& offsets) const
 {
     offsets.assign(layers_.size(), -1);
-    const auto resident = ldsResidency(true);
+    const auto placement = weightPlacement(true);
     const bool needsEncodingAdjoint = adjointFlags & (GRADIENTS_INPUT | GRADIENTS_INPUT_ENCODINGS);
     size_t n = 0;
     for (size_t i = 0; i < layers_.size(); ++i) {
-        if (resident[i] || (i == 0 && !needsEncodingAdjoint)) continue;
+        if (placement[i] != WEIGHTS_GLOBAL || (i == 0 && !needsEncodingAdjoint)) continue;
         offsets[i] = static_cast<long long>(n);
         n += static_cast<size_t>(layers_[i].channelsIn) * layers_[i].channelsOut;
     }
@@ -511,7 +537,13 @@ int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLa
             if (lds > maxLds) return 0;
             return std::min(16, (maxLds / lds) * (block / WARP_SIZE));
         };
-        if (wavesPerComputeUnit(2 * DEFAULT_BLOCK_SIZE) > wavesPerComputeUnit(blockSize)) blockSize = 2 * DEFAULT_BLOCK_SIZE;
+        // Input and output activations of a layer live in registers: one VGPR per channel each.
+        // Above 128 channels a wave needs more than the 256 registers it gets in a workgroup
+        // of 8 wavefronts.
+        int widest = 0;
+        for (const auto& l : layers_) widest = std::max(widest, std::max(l.channelsIn, l.channelsOut));
+        if (widest <= 128 && wavesPerComputeUnit(2 * DEFAULT_BLOCK_SIZE) > wavesPerComputeUnit(blockSize))
+            blockSize = 2 * DEFAULT_BLOCK_SIZE;
     }
     return blockSize;
 }
@@ -548,7 +580,10 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
     replaceAll(code, "$$POINTS_PER_LANE$$", std::to_string(pointsPerLane));
     std::vector<int> ldsW, ldsB;
-    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(false, ldsW, ldsB)));
+    int streamOffset = -1;
+    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(false, ldsW, ldsB, &streamOffset)));
+    replaceAll(code, "$$HAS_STREAMED_LAYERS$$", streamOffset >= 0 ? "true" : "false");
+    const auto placement = weightPlacement(false);
 
     std::vector<std::string> layerTypes;
     for (const auto& l : layers_) {
@@ -561,7 +596,7 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     stage << layerTypedefs(layerTypes);
     for (size_t i = 0; i < layers_.size(); ++i) {
         const auto& l = layers_[i];
-        if (ldsW[i] >= 0)
+        if (placement[i] == WEIGHTS_RESIDENT)
             stage << "    Layer" << i << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + "
                   << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
         if (l.useBias)
@@ -587,17 +622,24 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     std::stringstream callLayers;
     for (size_t i = 0; i < layers_.size(); ++i) {
         const auto& l = layers_[i];
+        // the instruction scheduler stays within one layer (across several it hoists the LDS reads
+        // of all of them to the front and spills them)
+        callLayers << "        __builtin_amdgcn_sched_barrier(0);\n";
         callLayers << "        f16x4 x" << (i + 1) << "[NT][Layer" << i << "::MT];\n";
-        if (ldsW[i] >= 0)
-            callLayers << "        Layer" << i << "::template forward<STORE>(sParams + " << ldsW[i] << ", ";
+        if (placement[i] == WEIGHTS_STREAMED)
+            callLayers << "        materialize(x" << i << ");\n        __syncthreads();   // the stream buffer is free\n        Layer" << i
+                       << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + " << ldsW[i]
+                       << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
+        if (placement[i] != WEIGHTS_GLOBAL)
+            callLayers << "        Layer" << i << "::template forward<STORE>(sWeights + " << ldsW[i] << ", ";
         else
             callLayers << "        Layer" << i << "::template forward<STORE, true>(networkParameters + " << l.weightsStart
                        << ", ";
         if (l.useBias)
-            callLayers << "sParams + " << ldsB[i];
+            callLayers << "sWeights + " << ldsB[i];
         else
             callLayers << "nullptr";
-        callLayers << ", x" << i << ", x" << (i + 1) << ",\n            STORE ? forwardTmpMemory + ("
+        callLayers << ", x" << i << ", x" << (i + 1) << ",\n            (STORE && tileValid) ? forwardTmpMemory + ("
                    << backwardInfo_[i].offsetPre << "ll * numel64 + static_cast<long long>(tile) * ("
                    << l.channelsOut << " * TILE_POINTS)) : nullptr, lane);\n";
     }
@@ -620,7 +662,9 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
     replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
     std::vector<int> ldsW, ldsB;
-    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(true, ldsW, ldsB)));
+    int streamOffset = -1;
+    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(true, ldsW, ldsB, &streamOffset)));
+    const auto placement = weightPlacement(true);
 
     std::vector<std::string> layerTypes;
     for (const auto& l : layers_) {
@@ -634,7 +678,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     std::stringstream stage;
     stage << layerTypedefs(layerTypes);
     for (size_t i = 0; i < layers_.size(); ++i) {
-        if ((i == 0 && !needsEncodingAdjoint) || ldsW[i] < 0) continue;
+        if ((i == 0 && !needsEncodingAdjoint) || placement[i] != WEIGHTS_RESIDENT) continue;
         const auto& l = layers_[i];
         stage << "    Layer" << i << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + "
               << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
@@ -645,23 +689,34 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     transposedWeightLayout(flags, transposed);
     std::stringstream callLayers;
     const int L = static_cast<int>(layers_.size());
+    bool anyStreamed = false;
     for (int i = L - 1; i >= 0; --i) {
         const auto& l = layers_[i];
         const std::string dy = (i == L - 1) ? std::string("dyOut") : "dx" + std::to_string(i + 1);
+        const bool needsWeights = i > 0 || needsEncodingAdjoint;
+        callLayers << "        __builtin_amdgcn_sched_barrier(0);\n";
         callLayers << "        f16x4 dx" << i << "[NT][Layer" << i << "::KT];\n";
-        std::string weights = "sParams + " + std::to_string(ldsW[i]);
-        if (ldsW[i] < 0) weights = transposed[i] >= 0 ? "transposedWeights + " + std::to_string(transposed[i]) : "nullptr";
+        std::string weights = "sWeights + " + std::to_string(ldsW[i]);
+        if (placement[i] == WEIGHTS_GLOBAL)
+            weights = transposed[i] >= 0 ? "transposedWeights + " + std::to_string(transposed[i]) : "nullptr";
+        if (placement[i] == WEIGHTS_STREAMED && needsWeights) {
+            anyStreamed = true;
+            callLayers << "        materialize(" << dy << ");\n        __syncthreads();   // the stream buffer is free\n        Layer" << i
+                       << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + " << ldsW[i]
+                       << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
+        }
         callLayers << "        Layer" << i << "::template adjoint<HAS_NETWORK_GRADIENTS, "
-                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (ldsW[i] < 0 ? ", true" : "") << ">(" << weights
-                   << ", " << dy
+                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (placement[i] == WEIGHTS_GLOBAL ? ", true" : "")
+                   << ">(" << weights << ", " << dy
                    << ", dx" << i << ",\n            forwardTmpMemory + (" << backwardInfo_[i].offsetPre
-                   << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut << " * TILE_POINTS)),\n"
-                   << "            HAS_NETWORK_GRADIENTS ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut
+                   << "ll * numel64 + static_cast<long long>(tileRead) * (" << l.channelsOut << " * TILE_POINTS)),\n"
+                   << "            (HAS_NETWORK_GRADIENTS && tileValid) ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut
                    << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut
                    << " * TILE_POINTS)) : nullptr,\n            validMask, lane);\n";
     }
     callLayers << "        auto& dxIn = dx0;\n        (void)dxIn;\n";
     replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
+    replaceAll(code, "$$HAS_STREAMED_LAYERS$$", anyStreamed ? "true" : "false");
 
     std::stringstream callEncodings, callScatter;
     int encodingOffset = 0;

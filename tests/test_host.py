@@ -209,22 +209,28 @@ def test_compile_errors_carry_the_compiler_log(tmp_path):
         qmlp.set_kernel_cache_dir(os.environ.get("QMLP_CACHE_DIR", qmlp._lib.DEFAULT_CACHE_DIR))
 
 
-def test_weights_beyond_the_lds_are_read_from_global_memory():
-    """3 x 256x256 fp16 weights are 384 KB: one layer stays in LDS, the others are gathered from
-    global memory (forward) or from a transposed copy in the adjoint memory (adjoint)."""
+def test_weights_beyond_the_lds_are_streamed_or_read_from_global_memory():
+    """3 x 256x256 fp16 weights are 384 KB: the layers are staged one after the other into a
+    shared LDS buffer. A 512x512 layer alone exceeds the LDS: it is gathered from global
+    memory (forward) or from a transposed copy in the adjoint memory (adjoint)."""
     cfg = json.loads(json.dumps(BASE))
     cfg["network"] = [{"n_out": 256, "bias": False, "activation": "relu"}] * 3 + [{"n_out": 1, "bias": False, "activation": "relu"}]
     cfg["num_outputs"] = 1
     net = qmlp.Network(json.dumps(cfg))
-    fwd = net.generated_source("forward")
-    n_global = fwd.count("forward<STORE, true>(networkParameters +")
-    assert n_global >= 1 and n_global + fwd.count("::stageForward(networkParameters") == 4
-    bwd = net.generated_source("backward", 1)
-    n_transposed = bwd.count("true>(transposedWeights +")
-    assert n_transposed >= 1 and n_transposed + bwd.count("::stageAdjoint(networkParameters") == 4
+    fwd, bwd = net.generated_source("forward"), net.generated_source("backward", 1)
+    assert "HAS_STREAMED_LAYERS = true" in fwd and "HAS_STREAMED_LAYERS = true" in bwd
+    n_streamed = fwd.count("the stream buffer is free")
+    assert n_streamed >= 2 and "forward<STORE, true>" not in fwd
+    assert net.adjoint_memory(64, 1) == 0
+    cfg["network"] = [{"n_out": 512, "bias": False, "activation": "relu"}] * 2 + [{"n_out": 1, "bias": False, "activation": "relu"}]
+    big = qmlp.Network(json.dumps(cfg))
+    fwd, bwd = big.generated_source("forward"), big.generated_source("backward", 1)
+    assert fwd.count("forward<STORE, true>(networkParameters +") == 1
+    assert bwd.count("true>(transposedWeights +") == 1
+    assert big.adjoint_memory(64, 1) == 512 * 512 * 2                         # the transposed copy
     small = qmlp.Network(json.dumps(BASE))
+    assert "HAS_STREAMED_LAYERS = false" in small.generated_source("forward")
     assert small.adjoint_memory(64, 1) == 0
-    assert net.adjoint_memory(64, 1) >= 256 * 256 * 2                        # the transposed copies
 
 
 def test_simulated_network_and_weight_copy_shapes():
