@@ -163,12 +163,14 @@ struct Layer
      * \param bias LDS bias vector (COUT halves) or nullptr
      * \param x input activations: x[nt][t] = channels 16t+4g+{0..3} of point 4r+nt
      * \param y output activations in the same layout
-     * \param preTile [STORE] where the pre-activations of this tile go (nullptr: nowhere): (COUT, 64) halves,
+     * \param preTile [STORE] where the pre-activations of this tile go (with GUARDED, nullptr means
+     *        nowhere; the test is compiled in only then, as its branches break up the instruction
+     *        scheduling of the layer): (COUT, 64) halves,
      *        channel-major, so that both the adjoint pass (per channel, 4 points of one
      *        lane) and the weight update (per channel, 8 consecutive points) read it
      *        with wide loads
      */
-    template <bool STORE, bool GLOBAL_W = false>
+    template <bool STORE, bool GLOBAL_W = false, bool GUARDED = false>
     __device__ __forceinline__ static void forward(const f16* __restrict__ w, const f16* __restrict__ bias,
                                                    const f16x4 (&x)[NT][KT], f16x4 (&y)[NT][MT],
                                                    f16* __restrict__ preTile, int lane)
@@ -200,7 +202,7 @@ struct Layer
             f16x4 p[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) p[nt] = toF16(acc[nt]);
-            if (STORE && preTile != nullptr) {
+            if (STORE && (!GUARDED || preTile != nullptr)) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const f16x4 v = {p[0][i], p[1][i], p[2][i], p[3][i]};
@@ -223,7 +225,7 @@ struct Layer
      * \param dpreTile [STORE_DPRE] receives the pre-activation adjoints, same layout
      * \param validMask bit nt set iff point 4r+nt of this lane is inside the batch
      */
-    template <bool STORE_DPRE, bool COMPUTE_DX, bool GLOBAL_W = false>
+    template <bool STORE_DPRE, bool COMPUTE_DX, bool GLOBAL_W = false, bool GUARDED = false>
     __device__ __forceinline__ static void adjoint(const f16* __restrict__ wT, f16x4 (&dy)[NT][MT],
                                                    f16x4 (&dx)[NT][KT], const f16* __restrict__ preTile,
                                                    f16* __restrict__ dpreTile, int validMask, int lane)
@@ -241,7 +243,7 @@ struct Layer
                     d[nt] = ((validMask >> nt) & 1) ? fromHalf(a) : static_cast<f16>(0);
                     dy[nt][m][i] = d[nt];
                 }
-                if (STORE_DPRE && dpreTile != nullptr)
+                if (STORE_DPRE && (!GUARDED || dpreTile != nullptr))
                     *reinterpret_cast<f16x4*>(dpreTile + (16 * m + 4 * g + i) * TILE_POINTS + 4 * r) = d;
             }
         }

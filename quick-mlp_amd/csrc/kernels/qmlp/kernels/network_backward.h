@@ -106,11 +106,6 @@ $$STAGE_PARAMETERS$$
         const bool tileValid = tile < numTiles;
         const int tileRead = tileValid ? tile : numTiles - 1;   // stored intermediates are read from a valid tile
         (void)tileRead;
-        // The weights in LDS do not change between the tiles; an offset the compiler cannot see
-        // through keeps it from hoisting their reads out of this loop (it then spills them).
-        int ldsOffset = 0;
-        asm volatile("" : "+s"(ldsOffset));
-        const f16* sWeights = sParams + ldsOffset;
         // dL/dy -> accumulator layout (fp32 -> fp16), zero outside batch / real channels
         f16x4 dyOut[NT][MTL];
         int validMask = 0;

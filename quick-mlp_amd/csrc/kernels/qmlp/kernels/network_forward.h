@@ -116,11 +116,6 @@ $$CALL_ENCODINGS$$
         const int tile = tile0 + q;
         if (!HAS_STREAMED_LAYERS && tile >= numTiles) break;
         const bool tileValid = tile < numTiles;
-        // The weights in LDS do not change between the tiles; an offset the compiler cannot see
-        // through keeps it from hoisting their reads out of the loops (it then spills them).
-        int ldsOffset = 0;
-        asm volatile("" : "+s"(ldsOffset));
-        const f16* sWeights = sParams + ldsOffset;
         const f16* sTile = sStage + q * (TILE_POINTS * STAGE_STRIDE);
 
         // B operands of the first layer

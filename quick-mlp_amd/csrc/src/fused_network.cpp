@@ -622,21 +622,18 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     std::stringstream callLayers;
     for (size_t i = 0; i < layers_.size(); ++i) {
         const auto& l = layers_[i];
-        // the instruction scheduler stays within one layer (across several it hoists the LDS reads
-        // of all of them to the front and spills them)
-        callLayers << "        __builtin_amdgcn_sched_barrier(0);\n";
         callLayers << "        f16x4 x" << (i + 1) << "[NT][Layer" << i << "::MT];\n";
         if (placement[i] == WEIGHTS_STREAMED)
             callLayers << "        materialize(x" << i << ");\n        __syncthreads();   // the stream buffer is free\n        Layer" << i
                        << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + " << ldsW[i]
                        << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
         if (placement[i] != WEIGHTS_GLOBAL)
-            callLayers << "        Layer" << i << "::template forward<STORE>(sWeights + " << ldsW[i] << ", ";
+            callLayers << "        Layer" << i << "::template forward<STORE, false, HAS_STREAMED_LAYERS>(sParams + " << ldsW[i] << ", ";
         else
-            callLayers << "        Layer" << i << "::template forward<STORE, true>(networkParameters + " << l.weightsStart
+            callLayers << "        Layer" << i << "::template forward<STORE, true, HAS_STREAMED_LAYERS>(networkParameters + " << l.weightsStart
                        << ", ";
         if (l.useBias)
-            callLayers << "sWeights + " << ldsB[i];
+            callLayers << "sParams + " << ldsB[i];
         else
             callLayers << "nullptr";
         callLayers << ", x" << i << ", x" << (i + 1) << ",\n            (STORE && tileValid) ? forwardTmpMemory + ("
@@ -694,9 +691,8 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
         const auto& l = layers_[i];
         const std::string dy = (i == L - 1) ? std::string("dyOut") : "dx" + std::to_string(i + 1);
         const bool needsWeights = i > 0 || needsEncodingAdjoint;
-        callLayers << "        __builtin_amdgcn_sched_barrier(0);\n";
         callLayers << "        f16x4 dx" << i << "[NT][Layer" << i << "::KT];\n";
-        std::string weights = "sWeights + " + std::to_string(ldsW[i]);
+        std::string weights = "sParams + " + std::to_string(ldsW[i]);
         if (placement[i] == WEIGHTS_GLOBAL)
             weights = transposed[i] >= 0 ? "transposedWeights + " + std::to_string(transposed[i]) : "nullptr";
         if (placement[i] == WEIGHTS_STREAMED && needsWeights) {
@@ -706,8 +702,8 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
                        << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
         }
         callLayers << "        Layer" << i << "::template adjoint<HAS_NETWORK_GRADIENTS, "
-                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (placement[i] == WEIGHTS_GLOBAL ? ", true" : "")
-                   << ">(" << weights << ", " << dy
+                   << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (placement[i] == WEIGHTS_GLOBAL ? ", true" : ", false")
+                   << ", HAS_STREAMED_LAYERS>(" << weights << ", " << dy
                    << ", dx" << i << ",\n            forwardTmpMemory + (" << backwardInfo_[i].offsetPre
                    << "ll * numel64 + static_cast<long long>(tileRead) * (" << l.channelsOut << " * TILE_POINTS)),\n"
                    << "            (HAS_NETWORK_GRADIENTS && tileValid) ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut

@@ -93,7 +93,7 @@ def test_networks_whose_weights_exceed_the_lds(widths, act):
     case = Case(identity_cfg(n_in, widths, [act] * len(widths), [True] * len(widths)))
     fwd, bwd = case.net.generated_source("forward"), case.net.generated_source("backward", 7)
     if widths[0] == 512:
-        assert "forward<STORE, true>" in fwd and "transposedWeights +" in bwd
+        assert "forward<STORE, true, " in fwd and "transposedWeights +" in bwd
     else:
         assert "the stream buffer is free" in fwd and "the stream buffer is free" in bwd
     rng = np.random.default_rng(77)

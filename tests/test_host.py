@@ -220,13 +220,13 @@ def test_weights_beyond_the_lds_are_streamed_or_read_from_global_memory():
     fwd, bwd = net.generated_source("forward"), net.generated_source("backward", 1)
     assert "HAS_STREAMED_LAYERS = true" in fwd and "HAS_STREAMED_LAYERS = true" in bwd
     n_streamed = fwd.count("the stream buffer is free")
-    assert n_streamed >= 2 and "forward<STORE, true>" not in fwd
+    assert n_streamed >= 2 and "forward<STORE, true, " not in fwd
     assert net.adjoint_memory(64, 1) == 0
     cfg["network"] = [{"n_out": 512, "bias": False, "activation": "relu"}] * 2 + [{"n_out": 1, "bias": False, "activation": "relu"}]
     big = qmlp.Network(json.dumps(cfg))
     fwd, bwd = big.generated_source("forward"), big.generated_source("backward", 1)
-    assert fwd.count("forward<STORE, true>(networkParameters +") == 1
-    assert bwd.count("true>(transposedWeights +") == 1
+    assert fwd.count("forward<STORE, true, HAS_STREAMED_LAYERS>(networkParameters +") == 1
+    assert bwd.count("true, HAS_STREAMED_LAYERS>(transposedWeights +") == 1
     assert big.adjoint_memory(64, 1) == 512 * 512 * 2                         # the transposed copy
     small = qmlp.Network(json.dumps(BASE))
     assert "HAS_STREAMED_LAYERS = false" in small.generated_source("forward")
