@@ -193,6 +193,10 @@ struct EncodingHashGrid
     __device__ __forceinline__ static void gatherLevel(int l, const float (&pos)[D],
                                                        const table_t* __restrict__ table, float (&feat)[F])
     {
+        // no contraction into fused multiply-adds: the kernels of different shapes (tiles per
+        // wave) would contract differently, and the same point has to give the same bits
+        // whatever the batch size
+#pragma clang fp contract(off)
         const LevelSetup s = setupLevel(l, pos);
         const int R = Cfg::resolution[l];
         const bool hashed = Cfg::hashed[l];

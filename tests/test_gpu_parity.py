@@ -463,6 +463,9 @@ def test_full_size_properties_cfg2():
     assert torch.equal(full, halves)
     perm = torch.randperm(N, device="cuda")
     assert torch.equal(case.net.inference(x[perm].contiguous(), case.params, enc), full[perm])
+    # small batches run kernels of another shape (fewer tiles per wave): same bits per point
+    for n in (1000, 1 << 16, 1 << 18):
+        assert torch.equal(case.net.inference(x[:n], case.params, enc), full[:n])
     sample = np.arange(0, N, 97)
     ref = case.oracle.forward(X[sample], round_mode=1)
     s = np.abs(ref).max()
