@@ -1,0 +1,195 @@
+// Exercises the C++ classes the way the reference's own C++ tests do
+// (tests_cpp/test_against_eigen1.cpp:70-213 of the reference: build a network from JSON,
+// create and initialise the parameter tensor, run inference / forward / adjoint, compare with
+// a plain evaluation on the host). Usage: test_cpp_api [--host]. With --host only the part
+// that needs no GPU runs. Exit code 0 = all checks passed.
+#include <qmlp/fused_network.h>
+#include <qmlp/qmlp.h>
+#include <qmlp/tmp_memory.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+using namespace qmlp;
+
+static int failures = 0;
+#define CHECK(cond)                                                            \
+    do {                                                                       \
+        if (!(cond)) {                                                         \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+            ++failures;                                                        \
+        }                                                                      \
+    } while (0)
+
+static const char* SPEC = R"json({
+    "num_inputs": 5, "num_outputs": 3,
+    "activation_specification": ["qmlp/builtin-activations.json"],
+    "encodings": [{"id": "Identity", "start_in": 0, "n_in": 5}],
+    "network": [
+        {"n_out": 20, "bias": true, "activation": "celu"},
+        {"n_out": 3, "bias": false, "activation": "identity"}
+    ]
+})json";
+
+static float halfToFloat(half h) { return static_cast<float>(h); }   // the host-side half is _Float16
+
+static void hostPart()
+{
+    auto cfg = json::parse(SPEC);
+    FusedNetwork net(cfg, ".");
+    CHECK(net.channelsIn() == 5 && net.channelsOut() == 3 && net.numLayers() == 2);
+    CHECK(net.numEncodings() == 1 && net.encoding(0)->id() == "Identity");
+    // padded layout: W0 (32,16), W1 (16,32), then b0 (32)
+    CHECK(net.networkParameterCount() == 32 * 16 + 16 * 32 + 32);
+    CHECK(net.networkParameterPrecision(Tensor::INFERENCE) == Tensor::HALF);
+    CHECK(net.networkParameterPrecision(Tensor::GRADIENTS) == Tensor::FLOAT);
+    CHECK(net.forwardMemory(100, FusedNetwork::GRADIENTS_INPUT) == size_t(128) * 2 * (16 + 32 + 16));
+    CHECK(FusedNetwork::MATRIX_SIZE == 16 && FusedNetwork::WARP_SIZE == 64);
+    // views into a parameter buffer
+    std::vector<half> dummy(net.networkParameterCount());
+    Tensor w1 = net.networkParameter(1, false, dummy.data(), Tensor::HALF);
+    CHECK(w1.ndim() == 2 && w1.size(0) == 16 && w1.size(1) == 32 && w1.stride(0) == 32);
+    CHECK(static_cast<half*>(w1.rawPtr()) - dummy.data() == 32 * 16);
+    Tensor b0 = net.networkParameter(0, true, dummy.data(), Tensor::HALF);
+    CHECK(b0.ndim() == 1 && b0.size(0) == 32);
+    bool thrown = false;
+    try {
+        auto bad = json::parse(SPEC);
+        bad["num_outputs"] = 4;
+        FusedNetwork n2(bad, ".");
+    } catch (const configuration_error&) {
+        thrown = true;
+    }
+    CHECK(thrown);
+    // the kernels of this network compile for gfx950 without a device
+    net.precompile(FusedNetwork::GRADIENTS_INPUT | FusedNetwork::GRADIENTS_NETWORK_WEIGHTS);
+}
+
+static float celu(float x) { return x > 0 ? x : std::exp(x) - 1; }
+static float celuAdjoint(float x, float adjz) { return x > 0 ? adjz : adjz * std::exp(x); }
+
+static void gpuPart()
+{
+    auto cfg = json::parse(SPEC);
+    auto net = std::make_shared<FusedNetwork>(cfg, ".");
+    const int N = 777, CIN = 5, COUT = 3, H = 32, K = 16;
+    const int P = net->networkParameterCount();
+
+    Tensor params(net->networkParameterPrecision(Tensor::INFERENCE), {P});
+    net->setNetworkParameter(params, Tensor::INFERENCE);
+    std::default_random_engine rng(42);
+    net->initializeInferenceParameters(rng);
+    std::vector<half> hp(P);
+    params.copyToHost(hp.data(), sizeof(half) * P);
+    std::vector<float> p(P);
+    for (int i = 0; i < P; ++i) p[i] = halfToFloat(hp[i]);
+    const float* W0 = p.data();            // (32, 16)
+    const float* W1 = p.data() + H * K;    // (16, 32)
+    const float* b0 = p.data() + 2 * H * K;
+
+    std::vector<float> x(N * CIN), adjOut(N * COUT);
+    std::uniform_real_distribution<float> uni(-1.f, 1.f);
+    for (auto& v : x) v = uni(rng);
+    for (auto& v : adjOut) v = uni(rng) / N;
+    Tensor input(Tensor::FLOAT, {N, CIN}), output(Tensor::FLOAT, {N, COUT}), adjOutput(Tensor::FLOAT, {N, COUT});
+    Tensor adjInput(Tensor::FLOAT, {N, CIN});
+    input.copyFromHost(x.data(), sizeof(float) * x.size());
+    adjOutput.copyFromHost(adjOut.data(), sizeof(float) * adjOut.size());
+    adjInput.zero_();
+    Tensor grads(net->networkParameterPrecision(Tensor::GRADIENTS), {P});
+    grads.zero_();
+    net->setNetworkParameter(grads, Tensor::GRADIENTS);
+
+    // host evaluation in fp32
+    std::vector<float> ref(N * COUT), refAdjIn(N * CIN, 0.f), refGrad(P, 0.f);
+    for (int n = 0; n < N; ++n) {
+        float pre[H], hid[H], dhid[H];
+        for (int o = 0; o < H; ++o) {
+            float a = b0[o];
+            for (int k = 0; k < CIN; ++k) a += W0[o * K + k] * x[n * CIN + k];
+            pre[o] = a;
+            hid[o] = celu(a);
+            dhid[o] = 0.f;
+        }
+        for (int o = 0; o < COUT; ++o) {
+            float a = 0.f;
+            for (int k = 0; k < H; ++k) a += W1[o * H + k] * hid[k];
+            ref[n * COUT + o] = a;
+            const float d = adjOut[n * COUT + o];
+            for (int k = 0; k < H; ++k) {
+                refGrad[H * K + o * H + k] += d * hid[k];
+                dhid[k] += W1[o * H + k] * d;
+            }
+        }
+        for (int o = 0; o < H; ++o) {
+            const float d = celuAdjoint(pre[o], dhid[o]);
+            refGrad[2 * H * K + o] += d;
+            for (int k = 0; k < CIN; ++k) {
+                refGrad[o * K + k] += d * x[n * CIN + k];
+                refAdjIn[n * CIN + k] += W0[o * K + k] * d;
+            }
+        }
+    }
+    auto close = [](float a, float e) { return std::fabs(a - e) <= 1e-3f + 1e-2f * std::fabs(e); };
+
+    net->inference(input, output, nullptr);
+    std::vector<float> out(N * COUT);
+    output.copyToHost(out.data(), sizeof(float) * out.size());
+    int bad = 0;
+    for (size_t i = 0; i < out.size(); ++i) bad += !close(out[i], ref[i]);
+    CHECK(bad == 0);
+
+    const int flags = FusedNetwork::GRADIENTS_INPUT | FusedNetwork::GRADIENTS_NETWORK_WEIGHTS;
+    TmpMemory fwd(net->forwardMemory(input, flags));
+    output.zero_();
+    net->forward(input, output, fwd.get(), nullptr);
+    output.copyToHost(out.data(), sizeof(float) * out.size());
+    bad = 0;
+    for (size_t i = 0; i < out.size(); ++i) bad += !close(out[i], ref[i]);
+    CHECK(bad == 0);
+
+    TmpMemory adj(net->adjointMemory(input, flags));
+    net->adjoint(input, adjOutput, flags, adjInput, fwd.get(), adj.get(), nullptr);
+    std::vector<float> adjIn(N * CIN), grad(P);
+    adjInput.copyToHost(adjIn.data(), sizeof(float) * adjIn.size());
+    grads.copyToHost(grad.data(), sizeof(float) * P);
+    bad = 0;
+    for (size_t i = 0; i < adjIn.size(); ++i) bad += !close(adjIn[i], refAdjIn[i]);
+    CHECK(bad == 0);
+    bad = 0;
+    for (int i = 0; i < P; ++i) bad += !close(grad[i], refGrad[i]);
+    CHECK(bad == 0);
+
+    // gradients accumulate: a second adjoint call doubles them
+    net->adjoint(input, adjOutput, flags, adjInput, fwd.get(), adj.get(), nullptr);
+    grads.copyToHost(grad.data(), sizeof(float) * P);
+    bad = 0;
+    for (int i = 0; i < P; ++i) bad += !close(grad[i], 2 * refGrad[i]);
+    CHECK(bad == 0);
+    net->zeroGradients();
+    grads.copyToHost(grad.data(), sizeof(float) * P);
+    bad = 0;
+    for (int i = 0; i < P; ++i) bad += grad[i] != 0.f;
+    CHECK(bad == 0);
+}
+
+int main(int argc, char** argv)
+{
+    const bool hostOnly = argc > 1 && std::strcmp(argv[1], "--host") == 0;
+    try {
+        QuickMLP::Instance().setLogLevel("error");
+        hostPart();
+        if (!hostOnly) {
+            QuickMLP::Instance().checkHipAvailable();
+            gpuPart();
+        }
+    } catch (const std::exception& e) {
+        std::printf("FAILED with exception: %s\n", e.what());
+        return 2;
+    }
+    std::printf(failures ? "%d check(s) failed\n" : "all checks passed\n", failures);
+    return failures ? 1 : 0;
+}
