@@ -159,6 +159,21 @@ int qmlp_activation_forward(qmlp_activation_t activation, const qmlp_tensor* inp
 int qmlp_activation_adjoint(qmlp_activation_t activation, const qmlp_tensor* input, const qmlp_tensor* adj_output,
                             const qmlp_tensor* adj_input, void* stream);           /* adjoint, :92 */
 
+/* ---- qmlp::Utils (src_cpp/include/qmlp/utils.h:50-85; bound for torch as utils.pullpush_forward
+ * and utils.pullpush_backward in src_cpp/pytorch-bindings/src/bind_utils.cpp:9-40) ---- */
+/* fractionalPullpush, utils.h:65: mask (B,H,W), data and output (B,C,H,W), C < 16, all float
+ * or all double. Returns after the work on 'stream' has finished (the image pyramid is
+ * temporary device memory of the call). */
+int qmlp_utils_pullpush_forward(const qmlp_tensor* mask, const qmlp_tensor* data, const qmlp_tensor* output,
+                                void* stream);
+/* adjointFractionalPullpush, utils.h:80: adds into adj_mask (B,H,W) and adj_data (B,C,H,W),
+ * which the caller zeroes first (bind_utils.cpp:26-27). */
+int qmlp_utils_pullpush_adjoint(const qmlp_tensor* mask, const qmlp_tensor* data, const qmlp_tensor* adj_output,
+                                const qmlp_tensor* adj_mask, const qmlp_tensor* adj_data, void* stream);
+/* Compiles the pull-push kernels for QMLP_FLOAT or QMLP_DOUBLE into the kernel cache without a
+ * device (the reference compiles them on first use, src_cpp/src/utils.cpp:12-35 and :145-180). */
+int qmlp_utils_pullpush_precompile(int precision);
+
 #ifdef __cplusplus
 }
 #endif

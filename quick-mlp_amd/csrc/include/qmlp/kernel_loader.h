@@ -118,13 +118,14 @@ private:
     std::filesystem::path kernelDir_;
     std::vector<std::string> headerNames_;
     std::vector<std::string> headerContents_;
-    std::string headerDigest_;
     std::map<std::string, Entry> modules_;   // key -> module
     std::mutex mutex_;
     int numCompilations_ = 0;
     int numDiskHits_ = 0;
 
     void loadHeaders();
+    /** Digest of the device headers that 'source' includes, directly or through other headers. */
+    std::string includedHeadersDigest(const std::string& source) const;
     std::string cacheKey(const std::string& kernelName, const std::string& source,
                          const std::vector<std::string>& options) const;
     bool loadFromDisk(const std::string& key, Entry& entry);

@@ -7,6 +7,7 @@
 #include <qmlp/fused_network.h>
 #include <qmlp/iencoding.h>
 #include <qmlp/qmlp.h>
+#include <qmlp/utils.h>
 
 #include <cstdlib>
 #include <cstring>
@@ -508,6 +509,33 @@ int qmlp_activation_adjoint(qmlp_activation_t activation, const qmlp_tensor* inp
     QMLP_API_BEGIN
     Tensor adjIn = wrap(adj_input);
     activation->activation->adjoint(wrap(input), wrap(adj_output), adjIn, static_cast<stream_t>(stream));
+    QMLP_API_END
+}
+
+int qmlp_utils_pullpush_forward(const qmlp_tensor* mask, const qmlp_tensor* data, const qmlp_tensor* output,
+                                void* stream)
+{
+    QMLP_API_BEGIN
+    Tensor out = wrap(output);
+    Utils::fractionalPullpush(wrap(mask), wrap(data), out, static_cast<stream_t>(stream));
+    QMLP_API_END
+}
+
+int qmlp_utils_pullpush_adjoint(const qmlp_tensor* mask, const qmlp_tensor* data, const qmlp_tensor* adj_output,
+                                const qmlp_tensor* adj_mask, const qmlp_tensor* adj_data, void* stream)
+{
+    QMLP_API_BEGIN
+    Tensor adjMask = wrap(adj_mask), adjData = wrap(adj_data);
+    Utils::adjointFractionalPullpush(wrap(mask), wrap(data), wrap(adj_output), adjMask, adjData,
+                                     static_cast<stream_t>(stream));
+    QMLP_API_END
+}
+
+int qmlp_utils_pullpush_precompile(int precision)
+{
+    QMLP_API_BEGIN
+    if (precision != QMLP_FLOAT && precision != QMLP_DOUBLE) throw std::runtime_error("precision must be float or double");
+    Utils::precompile(static_cast<Tensor::Precision>(precision));
     QMLP_API_END
 }
 

@@ -143,28 +143,17 @@ void KernelLoader::loadHeaders()
     headerNames_.clear();
     headerContents_.clear();
     std::error_code ec;
-    if (!std::filesystem::is_directory(kernelDir_, ec)) {
-        headerDigest_ = digest("");
-        return;
-    }
+    if (!std::filesystem::is_directory(kernelDir_, ec)) return;
     std::vector<std::filesystem::path> files;
     for (auto it = std::filesystem::recursive_directory_iterator(kernelDir_, ec);
          !ec && it != std::filesystem::recursive_directory_iterator(); it.increment(ec)) {
         if (it->is_regular_file() && it->path().extension() == ".h") files.push_back(it->path());
     }
     std::sort(files.begin(), files.end());
-    std::string all;
     for (const auto& f : files) {
-        std::string rel = std::filesystem::relative(f, kernelDir_).generic_string();
-        std::string content = readFile(f);
-        all += rel;
-        all += '\0';
-        all += content;
-        all += '\0';
-        headerNames_.push_back(rel);
-        headerContents_.push_back(std::move(content));
+        headerNames_.push_back(std::filesystem::relative(f, kernelDir_).generic_string());
+        headerContents_.push_back(readFile(f));
     }
-    headerDigest_ = digest(all);
 }
 
 std::optional<std::string> KernelLoader::findFile(const std::string& name) const
@@ -192,10 +181,50 @@ void KernelLoader::checkHipAvailable() const
     if (!isHipAvailable()) throw hip_error("No HIP device available");
 }
 
+std::string KernelLoader::includedHeadersDigest(const std::string& source) const
+{
+    // transitive closure of the #include lines that name one of the device headers; a header
+    // that the source cannot reach does not enter the key, so editing it keeps the cache
+    std::vector<bool> used(headerNames_.size(), false);
+    std::vector<size_t> todo;
+    auto scan = [&](const std::string& text) {
+        size_t pos = 0;
+        while ((pos = text.find("#include", pos)) != std::string::npos) {
+            pos += 8;
+            const size_t eol = std::min(text.find('\n', pos), text.size());
+            const size_t b = text.find_first_of("<\"", pos);
+            if (b == std::string::npos || b >= eol) continue;
+            const size_t e = text.find_first_of(">\"", b + 1);
+            if (e == std::string::npos || e >= eol) continue;
+            const std::string name = text.substr(b + 1, e - b - 1);
+            for (size_t i = 0; i < headerNames_.size(); ++i)
+                if (!used[i] && headerNames_[i] == name) {
+                    used[i] = true;
+                    todo.push_back(i);
+                }
+        }
+    };
+    scan(source);
+    while (!todo.empty()) {
+        const size_t i = todo.back();
+        todo.pop_back();
+        scan(headerContents_[i]);
+    }
+    std::string all;
+    for (size_t i = 0; i < headerNames_.size(); ++i)   // headerNames_ is sorted
+        if (used[i]) {
+            all += headerNames_[i];
+            all += '\0';
+            all += headerContents_[i];
+            all += '\0';
+        }
+    return digest(all);
+}
+
 std::string KernelLoader::cacheKey(const std::string& kernelName, const std::string& source,
                                    const std::vector<std::string>& options) const
 {
-    std::string all = headerDigest_;
+    std::string all = includedHeadersDigest(source);
     all += '\0';
     all += kernelName;
     all += '\0';

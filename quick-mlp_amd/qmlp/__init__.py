@@ -6,6 +6,7 @@ from ._version import __version__
 from .activation import FusedActivation
 from .encoding import FusedEncoding
 from .network import FusedNetwork, SimulatedNetwork, copy_torch_to_fused
+from . import pullpush   # qmlp.pullpush.pullpush(mask, data), like the reference's module
 from .classes import Activation, Encoding, Network, QuickMLP
 from ._lib import QmlpError, set_kernel_cache_dir, set_log_level
 
@@ -18,5 +19,5 @@ def load_library():
 
 __all__ = [
     "__version__", "load_library", "FusedActivation", "FusedEncoding", "FusedNetwork", "SimulatedNetwork",
-    "copy_torch_to_fused", "Activation", "Encoding", "Network", "QuickMLP", "QmlpError",
+    "copy_torch_to_fused", "pullpush", "Activation", "Encoding", "Network", "QuickMLP", "QmlpError",
     "set_kernel_cache_dir", "set_log_level"]

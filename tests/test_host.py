@@ -295,3 +295,41 @@ def test_line_integration_host_side():
                                    "encodings": [cfg], "network": [{"n_out": 1, "bias": False, "activation": "identity"}]}))
     assert net.num_network_parameters() == 16 * 16
     assert "EncodingLineIntegration<2, 3, qmlp::kernel::LineIntegrationBlendingMode::AVERAGE" in net.generated_source("inference")
+
+
+def test_pullpush_host_side(tmp_path):
+    """Kernels for both dtypes compile without a GPU; the argument checks of
+    Utils::fractionalPullpush (src_cpp/src/utils.cpp:112-135) fire before any device work."""
+    import torch
+    from qmlp import pullpush as qpp
+    from qmlp._lib import check, desc, lib
+    cache = str(tmp_path / "cache")
+    qmlp.set_kernel_cache_dir(cache)
+    try:
+        qpp.precompile(torch.float32)
+        qpp.precompile(torch.float64)
+        assert len(os.listdir(cache)) == 16    # down, up, their adjoints, add and copy for 3 and 4 dimensions; x2 dtypes
+        with pytest.raises(qmlp.QmlpError):
+            qpp.precompile(torch.float16)
+    finally:
+        qmlp.set_kernel_cache_dir(os.environ.get("QMLP_CACHE_DIR", qmlp._lib.DEFAULT_CACHE_DIR))
+
+    def call(mask, data, out=None):
+        out = torch.empty_like(data) if out is None else out
+        check(lib.qmlp_utils_pullpush_forward(desc(mask), desc(data), desc(out), None))
+
+    mask = torch.zeros(1, 4, 4)
+    with pytest.raises(qmlp.QmlpError, match="up to 16 channels, but got 16"):
+        call(mask, torch.zeros(1, 16, 4, 4))
+    with pytest.raises(qmlp.QmlpError, match="mask must have 5 entries at dimension 2"):
+        call(mask, torch.zeros(1, 2, 4, 5))
+    with pytest.raises(qmlp.QmlpError, match="mask must be of type DOUBLE, but is FLOAT"):
+        call(mask, torch.zeros(1, 2, 4, 4, dtype=torch.float64))
+    with pytest.raises(qmlp.QmlpError, match="float or double"):
+        call(mask.half(), torch.zeros(1, 2, 4, 4, dtype=torch.float16))
+    with pytest.raises(qmlp.QmlpError, match="output has the wrong size"):
+        call(mask, torch.zeros(1, 2, 4, 4), torch.zeros(1, 3, 4, 4))
+    with pytest.raises(qmlp.QmlpError, match="3 dimensions"):
+        call(mask[0], torch.zeros(1, 2, 4, 4))
+    with pytest.raises(ValueError, match="GPU tensors only"):
+        qpp.pullpush(mask, torch.zeros(1, 2, 4, 4))
