@@ -22,7 +22,8 @@ const char* scalarName(Tensor::Precision p)
 }
 
 const char* const KERNEL_NAMES[] = {"PullPushDownKernel<$T>", "PullPushUpKernel<$T>", "PullPushAdjointUpKernel<$T>",
-                                    "PullPushAdjointDownKernel<$T>", "PullPushAddKernel<$T, 3>",
+                                    "PullPushAdjointUpGatherKernel<$T>", "PullPushAdjointDownKernel<$T, true>",
+                                    "PullPushAdjointDownKernel<$T, false>", "PullPushAddKernel<$T, 3>",
                                     "PullPushAddKernel<$T, 4>", "PullPushCopyKernel<$T, 3>",
                                     "PullPushCopyKernel<$T, 4>"};
 
@@ -143,6 +144,8 @@ void adjointRecursion(const Tensor& maskInput, const Tensor& dataInput, const Te
     Tensor gradMaskLowPost(dtype, {B, oH, oW}), gradDataLowPost(dtype, {B, C, oH, oW});
     gradMaskLowPost.zeroAsync_(stream);
     gradDataLowPost.zeroAsync_(stream);
+    // what every high-res pixel passes down: C channel terms and one mask term
+    Tensor adjFill(dtype, {B, C + 1, H, W});
     {
         auto fun = pullpushKernel("PullPushAdjointUpKernel<" + t + ">");
         auto mask = accessorOf<const T, 3>(maskInput);
@@ -153,10 +156,18 @@ void adjointRecursion(const Tensor& maskInput, const Tensor& dataInput, const Te
         auto gDataHigh = accessorOf<const T, 4>(gradDataOutput);
         auto gMask = accessorOf<T, 3>(gradMaskInput);
         auto gData = accessorOf<T, 4>(gradDataInput);
+        auto fill = accessorOf<T, 4>(adjFill);
+        launch(fun, static_cast<long long>(B) * H * W, stream,
+               {&mask, &data, &maskLow, &dataLow, &gMaskHigh, &gDataHigh, &gMask, &gData, &fill});
+    }
+    {
+        auto fun = pullpushKernel("PullPushAdjointUpGatherKernel<" + t + ">");
+        auto maskLow = accessorOf<const T, 3>(level.maskLowPost);
+        auto dataLow = accessorOf<const T, 4>(level.dataLowPost);
+        auto fill = accessorOf<const T, 4>(adjFill);
         auto gMaskLow = accessorOf<T, 3>(gradMaskLowPost);
         auto gDataLow = accessorOf<T, 4>(gradDataLowPost);
-        launch(fun, static_cast<long long>(B) * H * W, stream,
-               {&mask, &data, &maskLow, &dataLow, &gMaskHigh, &gDataHigh, &gMask, &gData, &gMaskLow, &gDataLow});
+        launch(fun, static_cast<long long>(B) * oH * oW, stream, {&maskLow, &dataLow, &fill, &gMaskLow, &gDataLow});
     }
     Tensor gradMaskLowPre(dtype, {B, oH, oW}), gradDataLowPre(dtype, {B, C, oH, oW});
     gradMaskLowPre.zeroAsync_(stream);
@@ -164,7 +175,9 @@ void adjointRecursion(const Tensor& maskInput, const Tensor& dataInput, const Te
     adjointRecursion<T>(level.maskLowPre, level.dataLowPre, gradMaskLowPost, gradDataLowPost, gradMaskLowPre,
                         gradDataLowPre, saved, keepAlive, stream);
     {
-        auto fun = pullpushKernel("PullPushAdjointDownKernel<" + t + ">");
+        // windows of neighbouring low-res pixels overlap when a size is odd
+        const bool overlap = (H % 2 != 0) || (W % 2 != 0);
+        auto fun = pullpushKernel("PullPushAdjointDownKernel<" + t + (overlap ? ", true>" : ", false>"));
         auto mask = accessorOf<const T, 3>(maskInput);
         auto data = accessorOf<const T, 4>(dataInput);
         auto gMaskLow = accessorOf<const T, 3>(gradMaskLowPre);
@@ -174,7 +187,7 @@ void adjointRecursion(const Tensor& maskInput, const Tensor& dataInput, const Te
         launch(fun, static_cast<long long>(B) * oH * oW, stream, {&mask, &data, &gMaskLow, &gDataLow, &gMask, &gData});
     }
     for (Tensor* x : {&level.maskLowPre, &level.dataLowPre, &level.maskLowPost, &level.dataLowPost, &gradMaskLowPost,
-                      &gradDataLowPost, &gradMaskLowPre, &gradDataLowPre})
+                      &gradDataLowPost, &gradMaskLowPre, &gradDataLowPre, &adjFill})
         keepAlive.push_back(std::move(*x));
 }
 

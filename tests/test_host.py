@@ -308,7 +308,7 @@ def test_pullpush_host_side(tmp_path):
     try:
         qpp.precompile(torch.float32)
         qpp.precompile(torch.float64)
-        assert len(os.listdir(cache)) == 16    # down, up, their adjoints, add and copy for 3 and 4 dimensions; x2 dtypes
+        assert len(os.listdir(cache)) == 20    # down, up, 4 adjoint kernels, add and copy for 3 and 4 dimensions; x2 dtypes
         with pytest.raises(qmlp.QmlpError):
             qpp.precompile(torch.float16)
     finally:
