@@ -158,6 +158,9 @@ int qmlp_activation_forward(qmlp_activation_t activation, const qmlp_tensor* inp
                             void* stream);                                         /* forward, :81 */
 int qmlp_activation_adjoint(qmlp_activation_t activation, const qmlp_tensor* input, const qmlp_tensor* adj_output,
                             const qmlp_tensor* adj_input, void* stream);           /* adjoint, :92 */
+/* Compiles the standalone kernels into the kernel cache without a device (the reference
+ * compiles them on first use, src_cpp/src/activation.cpp:64-100). */
+int qmlp_activation_precompile(qmlp_activation_t activation);
 
 /* ---- qmlp::Utils (src_cpp/include/qmlp/utils.h:50-85; bound for torch as utils.pullpush_forward
  * and utils.pullpush_backward in src_cpp/pytorch-bindings/src/bind_utils.cpp:9-40) ---- */

@@ -55,6 +55,9 @@ public:
      */
     void adjoint(const Tensor& input, const Tensor& adjOutput, Tensor& adjInput, stream_t stream);
 
+    /** Compiles the two standalone kernels into the kernel cache; needs no GPU. */
+    void precompile();
+
 private:
     std::optional<KernelFunction> forwardKernel_;
     std::optional<KernelFunction> adjointKernel_;

@@ -73,13 +73,19 @@ json Activation::toJson() const
     return json::object({{"id", id()}, {"forward", forward()}, {"adjoint", adjoint()}});
 }
 
-static KernelFunction compileActivationKernel(const Activation& a, const char* kernelName)
+static KernelFunction compileActivationKernel(const Activation& a, const char* kernelName, int extraFlags = 0)
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string codeTemplate = kl->findFile("qmlp/kernels/activation_kernels.h").value();
     replaceAll(codeTemplate, "$$DEFINE_ACTIVATIONS$$", a.code());
     replaceAll(codeTemplate, "$$ACTIVATION_ID$$", a.id());
-    return kl->getKernel(kernelName, codeTemplate, QuickMLP::Instance().getCompileFlags()).value();
+    return kl->getKernel(kernelName, codeTemplate, QuickMLP::Instance().getCompileFlags() | extraFlags).value();
+}
+
+void Activation::precompile()
+{
+    compileActivationKernel(*this, "qmlp::kernel::ActivationForwardKernel", KernelLoader::CompileOnly);
+    compileActivationKernel(*this, "qmlp::kernel::ActivationAdjointKernel", KernelLoader::CompileOnly);
 }
 
 void Activation::forward(const Tensor& input, Tensor& output, stream_t stream)

@@ -512,6 +512,13 @@ int qmlp_activation_adjoint(qmlp_activation_t activation, const qmlp_tensor* inp
     QMLP_API_END
 }
 
+int qmlp_activation_precompile(qmlp_activation_t activation)
+{
+    QMLP_API_BEGIN
+    activation->activation->precompile();
+    QMLP_API_END
+}
+
 int qmlp_utils_pullpush_forward(const qmlp_tensor* mask, const qmlp_tensor* data, const qmlp_tensor* output,
                                 void* stream)
 {

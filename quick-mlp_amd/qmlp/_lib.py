@@ -100,6 +100,7 @@ _SIGNATURES = {
     "qmlp_activation_to_json": [_vp, _pstr],
     "qmlp_activation_forward": [_vp, _TD, _TD, _vp],
     "qmlp_activation_adjoint": [_vp, _TD, _TD, _TD, _vp],
+    "qmlp_activation_precompile": [_vp],
     "qmlp_utils_pullpush_forward": [_TD, _TD, _TD, _vp],
     "qmlp_utils_pullpush_adjoint": [_TD, _TD, _TD, _TD, _TD, _vp],
     "qmlp_utils_pullpush_precompile": [_ci],

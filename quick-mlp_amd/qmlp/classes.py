@@ -83,6 +83,10 @@ class Activation:
     def to_json(self):
         return _lib.get_string(lib.qmlp_activation_to_json, self._handle)
 
+    def precompile(self):
+        """Compiles the standalone kernels into the kernel cache; needs no GPU."""
+        check(lib.qmlp_activation_precompile(self._handle))
+
     def inference(self, input):
         _device_of(input)
         output = torch.empty_like(input)

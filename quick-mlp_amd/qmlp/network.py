@@ -113,6 +113,12 @@ class FusedNetwork(torch.nn.Module):
                           "which most optimizers cannot handle. Pass weight_dtype=torch.float32 to the constructor.")
         return self._network.forward(x, self.weights, list(self.encoding_parameters))
 
+    def __setstate__(self, state):
+        # pickling rebuilds the native network from its specification; take the encodings from
+        # the rebuilt network again instead of stand-alone copies
+        super().__setstate__(state)
+        self._encodings = [self._network.encoding(i) for i in range(self._num_encodings)]
+
     def __repr__(self):
         return f'FusedNetwork("{self._cfg}")'
 

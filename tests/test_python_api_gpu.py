@@ -1,0 +1,296 @@
+"""The PyTorch front end (FusedNetwork, FusedEncoding, FusedActivation) on the GPU, in the
+shape of the reference's Python suite (tests_py/qmlp_tests/test_network_base.py:87-256,
+test_activations.py:8-66, test_encoding.py:10-188, test_network_image.py:13-78).
+
+The comparison partner is plain torch on the same device: ``SimulatedNetwork``
+(torch.nn.Linear + activation modules in half precision) and torch's activation functions.
+Tolerances are the reference suite's: outputs and input gradients rtol 1e-2 / atol 1e-3,
+weight gradients rtol 1e-1 / atol 1e-3, at most 5% of the entries outside (the torch network
+rounds every layer to half, the fused kernels accumulate in fp32).
+"""
+import copy
+import io
+import json
+import os
+import pickle
+
+import numpy as np
+import pytest
+import torch
+
+import qmlp
+from qmlp import FusedActivation, FusedEncoding, FusedNetwork, SimulatedNetwork, copy_torch_to_fused
+
+pytestmark = pytest.mark.gpu
+
+WARM = bool(os.environ.get("QMLP_WARM_CACHE"))
+
+
+def warm_or_gpu(network_cfg=None, activation=None, encoding_cfg=None):
+    """In a CPU cache-warming pass compile what the test needs into the kernel cache and stop."""
+    if WARM:
+        if network_cfg is not None:
+            qmlp.Network(network_cfg).precompile(7)
+        if activation is not None:
+            qmlp.Activation(activation).precompile()
+        if encoding_cfg is not None:
+            enc = qmlp.Encoding(encoding_cfg)
+            for mode in (0, 1, 2, 3):
+                enc.precompile(mode)
+        pytest.skip("kernel cache warmed")
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU in this environment")
+
+
+def network_cfg(c_in, widths, activations, bias=False):
+    return json.dumps({
+        "num_inputs": c_in, "num_outputs": widths[-1],
+        "activation_specification": ["qmlp/builtin-activations.json"],
+        "encodings": [{"id": "Identity", "start_in": 0, "n_in": c_in}],
+        "network": [{"n_out": w, "bias": bias, "activation": a} for w, a in zip(widths, activations)]})
+
+
+def compare_tensors(actual, expected, name, rtol, atol, fail_threshold=0.05):
+    """_compare_tensors of the reference suite (test_network_base.py:56-70)."""
+    actual = actual.detach().cpu().to(torch.float32).numpy()
+    expected = expected.detach().cpu().to(torch.float32).numpy()
+    assert actual.shape == expected.shape, name
+    different = ~np.isclose(actual, expected, rtol=rtol, atol=atol)
+    assert different.mean() <= fail_threshold, "%s: %.2f%% of the entries differ" % (name, 100 * different.mean())
+
+
+def compare_networks(fused, plain, rtol, atol):
+    for layer in range(plain.num_layers()):
+        for bias in ((False, True) if plain.has_bias(layer) else (False,)):
+            want = plain.get_weight(layer, bias, True)
+            got = fused.get_weight(layer, bias, True)
+            got = got[tuple(slice(0, s) for s in want.shape)]      # the fused network pads widths to 16
+            compare_tensors(got, want, "layer %d %s gradient" % (layer, "bias" if bias else "weight"), rtol, atol)
+
+
+def run_network_suite(cfg, batch_sizes=(16, 32, 128, 513, 48621)):
+    """_test_network of the reference suite (test_network_base.py:87-147)."""
+    fused = FusedNetwork(cfg)
+    plain = SimulatedNetwork(cfg).to("cuda")
+    copy_torch_to_fused(fused, plain)
+    n_in, n_out = fused.channels_in(), fused.channels_out()
+    rtol, atol, rtol_wgrad = 1e-2, 1e-3, 1e-1
+    g = torch.Generator(device="cuda").manual_seed(n_in * 100 + n_out)
+    for N in batch_sizes:
+        print("python suite N =", N, flush=True)
+        x = torch.randn((N, n_in), device="cuda", generator=g)
+        grad_output = torch.randn((N, n_out), device="cuda", generator=g)
+        with torch.no_grad():
+            compare_tensors(fused(x), plain(x), "inference, N=%d" % N, rtol, atol)
+        for p in list(plain.parameters()) + list(fused.parameters()):
+            p.grad = None
+        x_plain = x.clone().requires_grad_(True)
+        x_fused = x.clone().requires_grad_(True)
+        y_plain, y_fused = plain(x_plain), fused(x_fused)
+        compare_tensors(y_fused, y_plain, "forward, N=%d" % N, rtol, atol)
+        torch.autograd.backward(y_plain, grad_output)
+        torch.autograd.backward(y_fused, grad_output)
+        compare_tensors(x_fused.grad, x_plain.grad, "input gradients, N=%d" % N, rtol, atol)
+        compare_networks(fused, plain, rtol_wgrad, atol)
+
+
+SINGLE = [(c_in, c_out, act) for c_in in (16, 32, 48) for c_out in (16, 32, 48) for act in ("celu", "identity")]
+
+
+@pytest.mark.parametrize("c_in,c_out,act", SINGLE)
+def test_network_single_layer(c_in, c_out, act):
+    cfg = network_cfg(c_in, [c_out], [act])
+    warm_or_gpu(network_cfg=cfg)
+    run_network_suite(cfg)
+
+
+# a spread over the product the reference loops over (3 x 3 x 3 widths, 2 x 2 activations)
+TWO = [(16, 16, 16, "celu", "celu"), (16, 48, 32, "identity", "celu"), (32, 16, 48, "celu", "identity"),
+       (32, 32, 32, "identity", "identity"), (48, 16, 16, "celu", "identity"), (48, 48, 48, "celu", "celu"),
+       (16, 32, 48, "identity", "identity"), (48, 32, 16, "identity", "celu")]
+
+
+@pytest.mark.parametrize("c_in,c_hidden,c_out,act_hidden,act_last", TWO)
+def test_network_two_layers(c_in, c_hidden, c_out, act_hidden, act_last):
+    cfg = network_cfg(c_in, [c_hidden, c_out], [act_hidden, act_last])
+    warm_or_gpu(network_cfg=cfg)
+    run_network_suite(cfg)
+
+
+THREE = [(16, 16, 16, "celu", "celu"), (32, 48, 16, "celu", "identity"), (48, 32, 48, "identity", "celu"),
+         (16, 48, 32, "identity", "identity"), (48, 16, 32, "celu", "celu")]
+
+
+@pytest.mark.parametrize("c_in,c_hidden,c_out,act_hidden,act_last", THREE)
+def test_network_three_layers(c_in, c_hidden, c_out, act_hidden, act_last):
+    cfg = network_cfg(c_in, [c_hidden, c_hidden, c_out], [act_hidden, act_hidden, act_last])
+    warm_or_gpu(network_cfg=cfg)
+    run_network_suite(cfg, batch_sizes=(32, 513, 48621))
+
+
+def test_network_with_bias_and_unpadded_widths():
+    """Widths that are no multiples of 16 and biased layers (the reference has no bias gradients)."""
+    cfg = network_cfg(5, [20, 24, 3], ["relu", "sine", "identity"], bias=True)
+    warm_or_gpu(network_cfg=cfg)
+    run_network_suite(cfg, batch_sizes=(35, 4267))
+
+
+@pytest.mark.parametrize("name", ["relu", "sine", "celu", "identity"])
+def test_activation_against_torch(name):
+    """_validate_activation of the reference suite (test_activations.py:8-36) on (5, 3) and a larger shape."""
+    warm_or_gpu(activation=name)
+    activ = FusedActivation(name)
+    baseline = FusedActivation.get_activation(name).to(dtype=torch.half, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    for shape in ((5, 3), (1000, 37)):
+        print("activation", name, shape, flush=True)
+        x = torch.randn(shape, dtype=torch.half, device="cuda", generator=g).requires_grad_(True)
+        y = activ(x)
+        y_want = baseline(x)
+        assert torch.allclose(y, y_want, rtol=2e-3, atol=1e-3)
+        target = torch.randn(shape, dtype=torch.half, device="cuda", generator=g)
+        torch.nn.functional.mse_loss(y, target).backward()
+        got = x.grad.detach().clone()
+        x.grad = None
+        torch.nn.functional.mse_loss(baseline(x), target).backward()
+        assert torch.allclose(got, x.grad, rtol=2e-3, atol=1e-4)
+    # strided input and output shapes; empty input
+    xt = torch.randn((37, 64), dtype=torch.half, device="cuda", generator=g).t()
+    assert torch.allclose(activ(xt), baseline(xt), rtol=2e-3, atol=1e-3)
+    assert activ(torch.zeros((0, 4), dtype=torch.half, device="cuda")).shape == (0, 4)
+
+
+def test_inline_activation_and_errors():
+    spec = json.dumps({"id": "square", "forward": "z = __hmul(x, x)",
+                       "adjoint": "adjx = __hmul(__hmul(__float2half(2.0f), x), adjz)"})
+    warm_or_gpu(activation=spec)
+    activ = FusedActivation(spec)
+    x = torch.linspace(-2, 2, 64, dtype=torch.half, device="cuda").reshape(8, 8).requires_grad_(True)
+    y = activ(x)
+    assert torch.allclose(y, x * x, rtol=1e-3, atol=1e-3)
+    y.sum().backward()
+    assert torch.allclose(x.grad, 2 * x.detach(), rtol=1e-3, atol=1e-3)
+    with pytest.raises(RuntimeError, match="HALF"):
+        activ(torch.zeros((4, 4), device="cuda"))
+
+
+GRID_2D = {"id": "HashGrid", "start_in": 0, "n_in": 2, "n_levels": 2, "n_features_per_level": 4,
+           "log2_hashmap_size": -1, "min_resolution": 8, "max_resolution": 16, "combination_mode": "concat",
+           "bounding_box_min": [-1, -1], "bounding_box_size": [2, 2]}
+
+
+def test_encoding_module_autograd_and_gradcheck():
+    """_validate_encoding of the reference suite (test_encoding.py:10-78): shapes, parameter
+    creation, both gradients, and torch.autograd.gradcheck with its loose settings."""
+    cfg = json.dumps(GRID_2D)
+    warm_or_gpu(encoding_cfg=cfg)
+    enc = FusedEncoding(cfg)
+    assert enc.has_parameters() and enc.num_output_channels() == 8 and enc.max_input_channel() == 1
+    params = enc.create_parameter_tensor().requires_grad_(True)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    # the grid is piecewise linear: keep the points away from the cell borders of both levels
+    # (resolutions 8 and 16) so that finite differences stay inside one cell
+    cand = torch.rand((4000, 2), device="cuda", generator=g) * 1.8 - 0.9
+    pos = (cand + 1) / 2
+    inside = torch.ones(len(cand), dtype=torch.bool, device="cuda")
+    for res in (8, 16):
+        frac = (pos * (res - 1)) % 1
+        inside &= ((frac > 0.2) & (frac < 0.8)).all(dim=1)
+    x = cand[inside][:8].clone().requires_grad_(True)
+    assert x.shape == (8, 2)
+    y = enc(x, params)
+    assert y.shape == (8, 8)
+    target = torch.randn(y.shape, device="cuda", generator=g)
+    torch.nn.functional.mse_loss(y, target).backward()
+    assert x.grad.shape == x.shape and params.grad.shape == params.shape
+    assert float(params.grad.abs().sum()) > 0 and float(x.grad.abs().sum()) > 0
+
+    def wrap_input(xd):
+        return enc(xd.to(torch.float32), params.detach()).to(torch.double)
+
+    def wrap_params(pd):
+        return enc(x.detach(), pd.to(params.dtype)).to(torch.double)
+
+    xd = x.detach().to(torch.double).requires_grad_(True)
+    assert torch.autograd.gradcheck(wrap_input, xd, eps=1e-2, atol=1e-1, rtol=1e-1, nondet_tol=1e-3)
+    pd = params.detach().to(torch.double).requires_grad_(True)
+    assert torch.autograd.gradcheck(wrap_params, pd, eps=1e-1, atol=1e-1, nondet_tol=1e-3)
+
+
+def test_identity_encoding_module():
+    cfg = json.dumps({"id": "Identity", "start_in": 1, "n_in": 3})
+    warm_or_gpu(encoding_cfg=cfg)
+    enc = FusedEncoding(cfg)
+    assert not enc.has_parameters() and enc.num_output_channels() == 3 and enc.max_input_channel() == 3
+    x = torch.randn((100, 5), device="cuda").requires_grad_(True)
+    y = enc(x)
+    assert torch.equal(y, x[:, 1:4])        # the stand-alone kernels write fp32, nothing is rounded
+    y.sum().backward()
+    want = torch.zeros_like(x)
+    want[:, 1:4] = 1
+    assert torch.equal(x.grad, want)
+
+
+def fit_cfg(activation, grid):
+    encodings = [{"id": "Identity", "start_in": 0, "n_in": 2}]
+    if grid:
+        encodings.insert(0, dict(GRID_2D, bounding_box_min=[0, 0], bounding_box_size=[1, 1], n_levels=4,
+                                 min_resolution=4, max_resolution=32, n_features_per_level=2))
+    return json.dumps({
+        "num_inputs": 2, "num_outputs": 3,
+        "activation_specification": ["qmlp/builtin-activations.json"],
+        "encodings": encodings,
+        "network": [{"n_out": 32, "bias": True, "activation": activation},
+                    {"n_out": 32, "bias": True, "activation": activation},
+                    {"n_out": 3, "bias": True, "activation": "identity"}]})
+
+
+@pytest.mark.parametrize("activation,grid", [("relu", False), ("sine", False), ("relu", True)])
+def test_fit_an_image_with_adam(activation, grid):
+    """The training loop of test_network_image.py:13-58 (fp32 master weights, Adam) on a
+    synthetic 64 x 64 image: the loss has to fall to about a third of that of the mean image or less."""
+    cfg = fit_cfg(activation, grid)
+    warm_or_gpu(network_cfg=cfg)
+    torch.manual_seed(0)
+    net = FusedNetwork(cfg, weight_dtype=torch.float32)
+    if grid:
+        with torch.no_grad():
+            net.encoding_parameters[0].uniform_(-0.1, 0.1)
+    yy, xx = torch.meshgrid(torch.linspace(0, 1, 64, device="cuda"), torch.linspace(0, 1, 64, device="cuda"), indexing="ij")
+    positions = torch.stack((xx, yy), dim=-1).reshape(-1, 2)
+    target = torch.stack((0.5 + 0.5 * torch.sin(6 * xx), yy * xx, (xx - 0.5) ** 2 + (yy - 0.5) ** 2), dim=-1).reshape(-1, 3)
+    optim = torch.optim.Adam(net.parameters(), lr=1e-2)
+    first = None
+    print("image fit", activation, grid, flush=True)
+    for _ in range(300):
+        optim.zero_grad()
+        loss = torch.nn.functional.mse_loss(net(positions), target)
+        loss.backward()
+        optim.step()
+        first = loss.item() if first is None else first
+    baseline = torch.nn.functional.mse_loss(target.mean(0, keepdim=True).expand_as(target), target).item()
+    assert loss.item() < 0.35 * baseline, (first, loss.item(), baseline)
+
+
+def test_state_dict_pickle_and_deepcopy():
+    """Module state travels like any torch module's; the native object is rebuilt from the
+    specification (the reference pickles its custom classes by cfg, bind_network.cpp:404-410)."""
+    cfg = fit_cfg("relu", True)
+    warm_or_gpu(network_cfg=cfg)
+    net = FusedNetwork(cfg, weight_dtype=torch.float32)
+    with torch.no_grad():
+        net.encoding_parameters[0].normal_(0, 0.1)
+    x = torch.rand((200, 2), device="cuda")
+    with torch.no_grad():
+        want = net(x)
+    other = FusedNetwork(cfg, weight_dtype=torch.float32)
+    other.load_state_dict(net.state_dict())
+    clones = [other, copy.deepcopy(net), pickle.loads(pickle.dumps(net))]
+    buffer = io.BytesIO()
+    torch.save(net, buffer)
+    buffer.seek(0)
+    clones.append(torch.load(buffer, weights_only=False))
+    for clone in clones:
+        with torch.no_grad():
+            assert torch.equal(clone(x), want)
+    assert repr(net).startswith("FusedNetwork(")
