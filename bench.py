@@ -51,7 +51,7 @@ def build_case(cfg_id, n_points, device):
     import qmlp
     from qmlp import baseline_configs as bc
     c = bc.CONFIGS[cfg_id]
-    rng = np.random.default_rng(0)
+    rng = np.random.default_rng(bc.PARAMETER_SEED[cfg_id])
     net = qmlp.Network(json.dumps(c["cfg"]))
     params_np = bc.make_parameters(cfg_id, rng)
     tables_np = []

@@ -102,6 +102,13 @@ def padded_layout(cfg):
     return [tuple(l) for l in layers], n
 
 
+# Seed of numpy's default_rng for the parameters of each configuration. Configuration 5 ends in
+# a ReLU with bias: with most seeds (0 among them) one or both of its outputs are negative
+# before that ReLU for every point, so the output and all gradients are exactly zero; seed 9
+# keeps both outputs alive.
+PARAMETER_SEED = {1: 0, 2: 0, 3: 0, 4: 0, 5: 9}
+
+
 def make_parameters(cfg_id, rng):
     """fp16 network parameters in the flat padded layout: U(+-1/sqrt(fan_in)) ("linear") or
     U(+-sqrt(6/fan_in)/30) ("siren") on the real entries, zeros on the padding."""

@@ -138,9 +138,10 @@ def check_gradients(case, X, adj, flags, got, kinks=False, what="", kink_fractio
     return ref0
 
 
-def baseline_case(cfg_id, table_scale=None, seed=0):
+def baseline_case(cfg_id, table_scale=None, seed=None):
     """A Case for BASELINE config cfg_id with its seeded parameters (and tables)."""
     c = bc.CONFIGS[cfg_id]
+    seed = bc.PARAMETER_SEED[cfg_id] if seed is None else seed
     rng = np.random.default_rng(seed)
     case = Case(c["cfg"], bc.ORACLE_ACTIVATIONS)
     case.set_parameters(bc.make_parameters(cfg_id, rng).astype(np.float32))

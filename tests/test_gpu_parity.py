@@ -417,7 +417,9 @@ def test_baseline_inference(cfg_id, N):
     # O(1) table values: with the published U(+-1e-4) tables every output is below abs 1e-3
     case, rng = baseline_case(cfg_id, table_scale=1.0 if cfg_id in (2, 5) else None)
     X = bc.make_inputs(cfg_id, N, rng)
-    assert_close(case.gpu_inference(X), case.oracle.forward(X), "inference cfg%d" % cfg_id)
+    ref = case.oracle.forward(X)
+    assert (ref != 0).mean() > 0.5, "the comparison would be between zeros"
+    assert_close(case.gpu_inference(X), ref, "inference cfg%d" % cfg_id)
 
 
 @pytest.mark.parametrize("cfg_id", [2, 5])
@@ -444,6 +446,7 @@ def test_baseline_train_step(cfg_id, N):
     adj = _mse_adjoint(out_ref, target) * N      # keep the adjoint O(1) per point
     flags = FLAG_INPUT | FLAG_WEIGHTS | (FLAG_ENC if cfg_id in (3, 5) else 0)
     got = case.gpu_train(X, adj, flags)
+    assert (out_ref != 0).mean() > 0.5 and np.abs(got["grads"]).max() > 0, "the comparison would be between zeros"
     assert_close(got["out"], out_ref, "forward")
     check_gradients(case, X, adj, flags, got, kinks=cfg_id in (3, 5))
 
@@ -492,4 +495,54 @@ def test_full_size_properties_cfg3_train():
     ref = case.oracle.backward(X[sample], adj[sample], FLAG_INPUT, round_mode=1)
     s = np.abs(ref["adj_x"]).max()
     assert_close(a["adj_x"][sample] / s, ref["adj_x"] / s, "sampled input gradients", rel=5e-3, abs_=1e-3,
+                 allowed_fraction=2e-3)
+
+
+@pytest.mark.parametrize("cfg_id,N", [(4, 1 << 20), (5, 1 << 21)])
+def test_full_size_properties_cfg4_cfg5(cfg_id, N):
+    """Configurations 4 and 5 at their benchmark sizes: inference is bit-identical under
+    splits and permutations of the batch and matches the oracle on a sample; the gradients
+    of a train step are additive over a split of the batch (weight and grid gradients are
+    sums over the points) and linear in dL/dy."""
+    case, rng = baseline_case(cfg_id, table_scale=1.0 if cfg_id == 5 else None)
+    X = bc.make_inputs(cfg_id, N, rng)
+    x = torch.from_numpy(X).cuda()
+    enc = case.encoding_parameters()
+    print("full size cfg%d: inference" % cfg_id, flush=True)
+    full = case.net.inference(x, case.params, enc)
+    cut = N // 3 + 5
+    parts = torch.cat([case.net.inference(x[:cut], case.params, enc), case.net.inference(x[cut:], case.params, enc)])
+    assert torch.equal(full, parts)
+    perm = torch.randperm(N, device="cuda")
+    assert torch.equal(case.net.inference(x[perm].contiguous(), case.params, enc), full[perm])
+    sample = np.arange(0, N, 257)
+    ref = case.oracle.forward(X[sample], round_mode=1)
+    assert (ref != 0).mean() > 0.5, "the comparison would be between zeros"
+    s = float(np.abs(ref).max())
+    assert_close(full.cpu().numpy()[sample] / s, ref / s, "sampled oracle check", rel=5e-3, abs_=1e-3,
+                 allowed_fraction=1e-3 if cfg_id == 5 else 0.0)
+
+    print("full size cfg%d: train step" % cfg_id, flush=True)
+    adj = rng.uniform(-1, 1, (N, case.oracle.n_out)).astype(np.float32)
+    flags = FLAG_INPUT | FLAG_WEIGHTS | (FLAG_ENC if cfg_id == 5 else 0)
+    whole = case.gpu_train(X, adj, flags)
+    first = case.gpu_train(X[:cut], adj[:cut], flags)
+    second = case.gpu_train(X[cut:], adj[cut:], flags)
+    assert np.array_equal(whole["out"], np.concatenate([first["out"], second["out"]]))
+    assert np.array_equal(whole["adj_x"], np.concatenate([first["adj_x"], second["adj_x"]]))
+    s = max(float(np.abs(whole["grads"]).max()), 1e-6)
+    assert_close((first["grads"] + second["grads"]) / s, whole["grads"] / s, "additivity of the weight gradients",
+                 rel=1e-3, abs_=1e-4)
+    if cfg_id == 5:
+        t = whole["table_grads"][0]
+        assert_close(first["table_grads"][0] + second["table_grads"][0], t, "additivity of the grid gradients",
+                     rel=1e-3, abs_=1e-4 * np.abs(t).max())
+    doubled = case.gpu_train(X, 2 * adj, flags)
+    assert_close(doubled["grads"] / s, 2 * whole["grads"] / s, "linearity of the weight gradients", rel=1e-2, abs_=1e-3)
+    sample = np.arange(0, N, 1031)
+    ref = case.oracle.backward(X[sample], adj[sample], FLAG_INPUT, round_mode=1)
+    s = max(float(np.abs(ref["adj_x"]).max()), 1e-6)
+    # a few entries in a thousand differ by more: last-bit differences of the half-precision sin / exp
+    # intrinsics (cfg4) and ReLU units switching next to zero (cfg5)
+    assert_close(whole["adj_x"][sample] / s, ref["adj_x"] / s, "sampled input gradients", rel=5e-3, abs_=1e-3,
                  allowed_fraction=2e-3)
