@@ -37,10 +37,14 @@ $$DEFINE_ACTIVATIONS$$
  * \tparam CIN, COUT padded layer widths
  * \tparam BIAS also reduce the bias gradient
  * \tparam InputActivation activation applied to the B operand (previous layer), or passthrough_
- * \tparam MO_CHUNK number of 16-row output tiles one workgroup accumulates; the grid is
- *         (COUT/16/MO_CHUNK) chunks x batch slices, chunk index fastest
+ * \tparam MO_CHUNK number of 16-row output tiles and
+ * \tparam KI_CHUNK number of 16-column input tiles one workgroup accumulates: a workgroup owns a
+ *         MO_CHUNK x KI_CHUNK block of the 16 x 16 tiles of dW. The grid is
+ *         (COUT/16/MO_CHUNK) x (CIN/16/KI_CHUNK) blocks x batch slices, block index fastest.
+ *         Splitting the input channels re-reads dpre, splitting the output channels re-reads
+ *         the input and re-applies its activation; the host picks the cheaper split.
  */
-template <int CIN, int COUT, bool BIAS, typename InputActivation, int MO_CHUNK>
+template <int CIN, int COUT, bool BIAS, typename InputActivation, int MO_CHUNK, int KI_CHUNK>
 __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
     int numTiles,                     // 64-point tiles in the batch
     float* __restrict__ partialWeights,  // slice 0 of this layer's (COUT, CIN) row-major partial sums
@@ -51,9 +55,11 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
 {
     constexpr int KT = CIN / 16;
     constexpr int MT = COUT / 16;
-    constexpr int NCHUNK = MT / MO_CHUNK;
+    constexpr int MCHUNKS = MT / MO_CHUNK;
+    constexpr int KCHUNKS = KT / KI_CHUNK;
+    constexpr int NCHUNK = MCHUNKS * KCHUNKS;
     constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
-    static_assert(MT % MO_CHUNK == 0, "chunk size must divide the number of output tiles");
+    static_assert(MT % MO_CHUNK == 0 && KT % KI_CHUNK == 0, "chunk sizes must divide the numbers of tiles");
 
     const f16* __restrict__ adjPre = reinterpret_cast<const f16*>(adjPreH);
     const f16* __restrict__ input = reinterpret_cast<const f16*>(inputH);
@@ -64,15 +70,17 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
     const int chunk = blockIdx.x % NCHUNK;
     const int slice = blockIdx.x / NCHUNK;
     const int numSlices = gridDim.x / NCHUNK;
-    const int mo0 = chunk * MO_CHUNK;
+    const int mo0 = (chunk % MCHUNKS) * MO_CHUNK;
+    const int ki0 = (chunk / MCHUNKS) * KI_CHUNK;
+    const bool ownsBias = BIAS && ki0 == 0;   // the bias gradient does not depend on the input channels
 
-    f32x4 acc[MO_CHUNK][KT];
+    f32x4 acc[MO_CHUNK][KI_CHUNK];
     f32x4 accBias[MO_CHUNK];
 #pragma unroll
     for (int mo = 0; mo < MO_CHUNK; ++mo) {
         accBias[mo] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int mi = 0; mi < KT; ++mi) acc[mo][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mi = 0; mi < KI_CHUNK; ++mi) acc[mo][mi] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     const f16x8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
 
@@ -82,17 +90,20 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
         const f16* bTile = input + static_cast<long long>(tile) * (CIN * TILE_POINTS);
 #pragma unroll
         for (int kb = 0; kb < TILE_POINTS / 32; ++kb) {
-            f16x8 b[KT];
+            f16x8 b[KI_CHUNK];
 #pragma unroll
-            for (int mi = 0; mi < KT; ++mi) {
-                const f16x8 raw = *reinterpret_cast<const f16x8*>(bTile + (16 * mi + r) * TILE_POINTS + 32 * kb + 8 * g);
-                b[mi] = activationForwardChannel<InputActivation>(raw, 16 * mi + r);
+            for (int mi = 0; mi < KI_CHUNK; ++mi) {
+                const int channel = 16 * (ki0 + mi) + r;
+                const f16x8 raw = *reinterpret_cast<const f16x8*>(bTile + channel * TILE_POINTS + 32 * kb + 8 * g);
+                b[mi] = activationForwardChannel<InputActivation>(raw, channel);
             }
 #pragma unroll
             for (int mo = 0; mo < MO_CHUNK; ++mo) {
                 const f16x8 a = *reinterpret_cast<const f16x8*>(aTile + (16 * (mo0 + mo) + r) * TILE_POINTS + 32 * kb + 8 * g);
 #pragma unroll
-                for (int mi = 0; mi < KT; ++mi) acc[mo][mi] = mfma32(a, b[mi], acc[mo][mi]);
+                for (int mi = 0; mi < KI_CHUNK; ++mi) acc[mo][mi] = mfma32(a, b[mi], acc[mo][mi]);
+                // every block sums the bias gradient (a branch here would split the loop body);
+                // only the blocks of the first input chunk store it
                 if constexpr (BIAS) accBias[mo] = mfma32(a, ones, accBias[mo]);
             }
         }
@@ -100,37 +111,39 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
 
     // combine the waves of the workgroup through LDS, then store the slice's partial sums
     extern __shared__ __align__(16) unsigned char sMemory[];
-    float* sAcc = reinterpret_cast<float*>(sMemory);   // (MO_CHUNK*KT + MO_CHUNK) tiles of 256 floats
-    constexpr int TILES = MO_CHUNK * KT + (BIAS ? MO_CHUNK : 0);
+    float* sAcc = reinterpret_cast<float*>(sMemory);   // (MO_CHUNK*KI_CHUNK + MO_CHUNK) tiles of 256 floats
+    constexpr int TILES = MO_CHUNK * KI_CHUNK + (BIAS ? MO_CHUNK : 0);
     for (int i = threadIdx.x; i < TILES * 256; i += blockDim.x) sAcc[i] = 0.f;
     __syncthreads();
 #pragma unroll
     for (int mo = 0; mo < MO_CHUNK; ++mo) {
 #pragma unroll
-        for (int mi = 0; mi < KT; ++mi)
+        for (int mi = 0; mi < KI_CHUNK; ++mi)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                atomicAdd(&sAcc[(mo * KT + mi) * 256 + (4 * g + i) * 16 + r], acc[mo][mi][i]);
+                atomicAdd(&sAcc[(mo * KI_CHUNK + mi) * 256 + (4 * g + i) * 16 + r], acc[mo][mi][i]);
         if constexpr (BIAS) {
-            if (r == 0) {
+            if (ownsBias && r == 0) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    atomicAdd(&sAcc[(MO_CHUNK * KT + mo) * 256 + 4 * g + i], accBias[mo][i]);
+                    atomicAdd(&sAcc[(MO_CHUNK * KI_CHUNK + mo) * 256 + 4 * g + i], accBias[mo][i]);
             }
         }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < MO_CHUNK * KT * 256; e += blockDim.x) {
+    for (int e = threadIdx.x; e < MO_CHUNK * KI_CHUNK * 256; e += blockDim.x) {
         const int t = e >> 8, within = e & 255;
-        const int mo = t / KT, mi = t - mo * KT;
-        const int row = 16 * (mo0 + mo) + (within >> 4), col = 16 * mi + (within & 15);
+        const int mo = t / KI_CHUNK, mi = t - mo * KI_CHUNK;
+        const int row = 16 * (mo0 + mo) + (within >> 4), col = 16 * (ki0 + mi) + (within & 15);
         partialWeights[static_cast<long long>(slice) * sliceStride + row * CIN + col] = sAcc[e];
     }
     if constexpr (BIAS) {
-        for (int e = threadIdx.x; e < MO_CHUNK * 16; e += blockDim.x) {
-            const int mo = e >> 4;
-            partialBias[static_cast<long long>(slice) * sliceStride + 16 * (mo0 + mo) + (e & 15)]
-                = sAcc[(MO_CHUNK * KT + mo) * 256 + (e & 15)];
+        if (ownsBias) {
+            for (int e = threadIdx.x; e < MO_CHUNK * 16; e += blockDim.x) {
+                const int mo = e >> 4;
+                partialBias[static_cast<long long>(slice) * sliceStride + 16 * (mo0 + mo) + (e & 15)]
+                    = sAcc[(MO_CHUNK * KI_CHUNK + mo) * 256 + (e & 15)];
+            }
         }
     }
 }

@@ -750,22 +750,38 @@ std::string FusedNetwork::weightUpdateSource(int blockSize) const
     return code;
 }
 
-std::string FusedNetwork::weightUpdateKernelName(int layer, int& numChunks) const
+std::string FusedNetwork::weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const
 {
     const auto& l = layers_[layer];
     const int kt = l.channelsIn / MATRIX_SIZE, mt = l.channelsOut / MATRIX_SIZE;
-    // at most 16 accumulator tiles (64 VGPRs) per wave; 32 would halve the re-reads of the input
-    // operand of a 128-wide layer but measured slower (208 VGPRs, half the waves per SIMD)
-    int moChunk = 1;
-    for (int c = 1; c <= mt; ++c)
-        if (mt % c == 0 && c * kt <= 16) moChunk = c;
-    numChunks = mt / moChunk;
+    // A workgroup accumulates a block of mo x ki tiles of dW, at most 16 (64 accumulator
+    // registers per lane; 32 tiles measured slower: half the waves per SIMD). Splitting the
+    // output tiles makes every block read the whole input operand again and re-apply its
+    // activation; splitting the input tiles makes every block read dpre again. Take the split
+    // with the least traffic, the activation counted as half of another read.
+    const double inputCost = layer > 0 ? 1.5 : 1.0;
+    int moChunk = 1, kiChunk = 1;
+    double best = -1;
+    for (int mo = 1; mo <= mt; ++mo) {
+        if (mt % mo != 0) continue;
+        for (int ki = 1; ki <= kt; ++ki) {
+            if (kt % ki != 0 || mo * ki > 16) continue;
+            const double cost = l.channelsOut * static_cast<double>(kt / ki) + inputCost * l.channelsIn * (mt / mo);
+            if (best < 0 || cost < best || (cost == best && mo * ki > moChunk * kiChunk)) {
+                best = cost;
+                moChunk = mo;
+                kiChunk = ki;
+            }
+        }
+    }
+    numChunks = (mt / moChunk) * (kt / kiChunk);
+    tilesPerBlock = moChunk * kiChunk + (l.useBias ? moChunk : 0);
     std::string inputActivation = "qmlp::kernel::activations::passthrough_";
     if (layer > 0) {
         inputActivation = "qmlp::kernel::activations::" + activationTypeName(layer - 1);
     }
-    return format("qmlp::kernel::WeightUpdateKernel<%d, %d, %s, %s, %d>", l.channelsIn, l.channelsOut,
-                  l.useBias ? "true" : "false", inputActivation.c_str(), moChunk);
+    return format("qmlp::kernel::WeightUpdateKernel<%d, %d, %s, %s, %d, %d>", l.channelsIn, l.channelsOut,
+                  l.useBias ? "true" : "false", inputActivation.c_str(), moChunk, kiChunk);
 }
 
 std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFlags)
@@ -884,10 +900,8 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
         ak.layers.resize(layers_.size());
         for (size_t layer = 0; layer < layers_.size(); ++layer) {
             auto& wk = ak.layers[layer];
-            const std::string name = weightUpdateKernelName(static_cast<int>(layer), wk.numChunks);
-            const auto& l = layers_[layer];
-            const int moChunk = l.channelsOut / MATRIX_SIZE / wk.numChunks;
-            const int tiles = moChunk * (l.channelsIn / MATRIX_SIZE) + (l.useBias ? moChunk : 0);
+            int tiles = 0;
+            const std::string name = weightUpdateKernelName(static_cast<int>(layer), wk.numChunks, tiles);
             wk.kernel.blockSize = blockSize;
             wk.kernel.sharedMemorySize = tiles * 256 * static_cast<int>(sizeof(float));
             if (wk.kernel.sharedMemorySize > MaxSharedMemoryBytes())
