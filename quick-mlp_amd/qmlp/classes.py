@@ -175,7 +175,10 @@ class Encoding:
         return _lib.get_int(lib.qmlp_encoding_num_output_channels, self._handle)
 
     def has_parameters(self):
-        return bool(_lib.get_int(lib.qmlp_encoding_has_parameters, self._handle))
+        # fixed by the specification: asked once (this sits on the per-call path of the network)
+        if getattr(self, "_has_parameters", None) is None:
+            self._has_parameters = bool(_lib.get_int(lib.qmlp_encoding_has_parameters, self._handle))
+        return self._has_parameters
 
     def num_parameters(self):
         return _lib.get_int(lib.qmlp_encoding_parameter_count, self._handle)
@@ -376,7 +379,9 @@ class Network:
         check(lib.qmlp_network_set_parallel_streams(self._handle, 1 if enabled else 0))
 
     def num_encodings(self):
-        return _lib.get_int(lib.qmlp_network_num_encodings, self._handle)
+        if getattr(self, "_num_encodings", None) is None:
+            self._num_encodings = _lib.get_int(lib.qmlp_network_num_encodings, self._handle)
+        return self._num_encodings
 
     def encoding(self, idx):
         if idx not in self._encodings:
@@ -389,7 +394,9 @@ class Network:
         return _lib.get_int(lib.qmlp_network_channels_in, self._handle)
 
     def channels_out(self):
-        return _lib.get_int(lib.qmlp_network_channels_out, self._handle)
+        if getattr(self, "_channels_out", None) is None:
+            self._channels_out = _lib.get_int(lib.qmlp_network_channels_out, self._handle)
+        return self._channels_out
 
     def num_layers(self):
         return _lib.get_int(lib.qmlp_network_num_layers, self._handle)
