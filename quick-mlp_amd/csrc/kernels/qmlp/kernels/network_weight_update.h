@@ -8,7 +8,7 @@
 // channel per lane = one 16-byte load in operand layout); in_l is the activation of
 // the previous layer re-applied on the fly, or the stored encoded input for layer 0.
 // Many workgroups reduce disjoint slices of the batch; each wave accumulates in fp32
-// registers, the waves of a workgroup are combined through LDS and the workgroup stores
+// registers, the waves of a workgroup are combined through LDS in a fixed order and the workgroup stores
 // its partial sums (slice-major) without atomics: thousands of atomic additions onto the
 // same few cache lines serialise in the memory system and took ten times longer than
 // the reduction itself. WeightUpdateReduceKernel then adds the partial sums of all slices
@@ -115,22 +115,26 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
     constexpr int TILES = MO_CHUNK * KI_CHUNK + (BIAS ? MO_CHUNK : 0);
     for (int i = threadIdx.x; i < TILES * 256; i += blockDim.x) sAcc[i] = 0.f;
     __syncthreads();
+    // one wave after the other, so that the sum has the same rounding in every run
+    for (int w = 0; w < WAVES; ++w) {
+        if (wave == w) {
 #pragma unroll
-    for (int mo = 0; mo < MO_CHUNK; ++mo) {
+            for (int mo = 0; mo < MO_CHUNK; ++mo) {
 #pragma unroll
-        for (int mi = 0; mi < KI_CHUNK; ++mi)
+                for (int mi = 0; mi < KI_CHUNK; ++mi)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                atomicAdd(&sAcc[(mo * KI_CHUNK + mi) * 256 + (4 * g + i) * 16 + r], acc[mo][mi][i]);
-        if constexpr (BIAS) {
-            if (ownsBias && r == 0) {
+                    for (int i = 0; i < 4; ++i)
+                        sAcc[(mo * KI_CHUNK + mi) * 256 + (4 * g + i) * 16 + r] += acc[mo][mi][i];
+                if constexpr (BIAS) {
+                    if (ownsBias && r == 0) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    atomicAdd(&sAcc[(MO_CHUNK * KI_CHUNK + mo) * 256 + 4 * g + i], accBias[mo][i]);
+                        for (int i = 0; i < 4; ++i) sAcc[(MO_CHUNK * KI_CHUNK + mo) * 256 + 4 * g + i] += accBias[mo][i];
+                    }
+                }
             }
         }
+        __syncthreads();
     }
-    __syncthreads();
     for (int e = threadIdx.x; e < MO_CHUNK * KI_CHUNK * 256; e += blockDim.x) {
         const int t = e >> 8, within = e & 255;
         const int mo = t / KI_CHUNK, mi = t - mo * KI_CHUNK;

@@ -294,3 +294,60 @@ def test_state_dict_pickle_and_deepcopy():
         with torch.no_grad():
             assert torch.equal(clone(x), want)
     assert repr(net).startswith("FusedNetwork(")
+
+
+def test_inference_and_train_step_replay_from_a_hip_graph():
+    """Nothing on the call path allocates, synchronises or clears memory with a memset, so a
+    caller can capture it: inference and a whole train step (forward, backward, weight update,
+    reduce) are recorded once and replayed several times with fresh inputs, with eager work and
+    synchronisations in between; every replay has to give the eager result bit for bit (the
+    grid gradients, summed with atomics, up to fp32 rounding)."""
+    cfg = fit_cfg("relu", True)
+    warm_or_gpu(network_cfg=cfg)
+    net = qmlp.Network(cfg)
+    g = torch.Generator(device="cuda").manual_seed(4)
+    params = ((torch.rand(net.num_network_parameters(), device="cuda", generator=g) - 0.5) * 0.5).half()
+    enc = net.encoding(0)
+    table = (torch.rand(enc.num_parameters(), device="cuda", generator=g) - 0.5).to(enc.parameter_dtype())
+    tables = [table, None]
+    N, flags = 5000, 7
+    x = torch.rand((N, 2), device="cuda", generator=g)
+    adj = torch.rand((N, 3), device="cuda", generator=g)
+    grad_net = torch.zeros(net.num_network_parameters(), device="cuda")
+    grad_table = torch.zeros(enc.num_parameters(), device="cuda")
+    adj_x = torch.zeros_like(x)
+
+    def step():
+        out, tmp = net.forward_raw(x, params, tables, flags)
+        net.adjoint_raw(x, adj, flags, tmp, params, tables, grad_network=grad_net,
+                        grad_encodings=[grad_table, None], adj_input=adj_x)
+        return out, net.inference(x, params, tables)
+
+    def eager():
+        for t in (grad_net, grad_table, adj_x):
+            t.zero_()
+        out, inf = step()
+        torch.cuda.synchronize()
+        return [t.clone() for t in (out, inf, grad_net, grad_table, adj_x)]
+
+    eager()                                   # kernels loaded, occupancy queried
+    graph = torch.cuda.CUDAGraph()
+    for t in (grad_net, grad_table, adj_x):
+        t.zero_()
+    print("hip graph: capture", flush=True)
+    with torch.cuda.graph(graph):
+        out_g, inf_g = step()
+    for replay in range(4):
+        x.copy_(torch.rand((N, 2), device="cuda", generator=g))
+        adj.copy_(torch.rand((N, 3), device="cuda", generator=g))
+        want = eager()                        # eager work and a synchronisation between the replays
+        for t in (grad_net, grad_table, adj_x):
+            t.zero_()                         # a fill kernel, outside of the graph
+        print("hip graph: replay", replay, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [out_g, inf_g, grad_net, grad_table, adj_x]
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), "outputs of replay %d" % replay
+        assert torch.equal(got[2], want[2]), "weight gradients of replay %d" % replay
+        assert torch.allclose(got[3], want[3], rtol=1e-4, atol=1e-6), "grid gradients of replay %d" % replay
+        assert torch.allclose(got[4], want[4], rtol=1e-5, atol=1e-7), "input gradients of replay %d" % replay
