@@ -6,6 +6,7 @@
 #include <qmlp/fused_network.h>
 #include <qmlp/qmlp.h>
 #include <qmlp/tmp_memory.h>
+#include <qmlp/utils.h>
 
 #include <cmath>
 #include <cstdio>
@@ -176,6 +177,59 @@ static void gpuPart()
     CHECK(bad == 0);
 }
 
+// Utils::fractionalPullpush (src_cpp/include/qmlp/utils.h:50-85 of the reference) on closed forms:
+// one known pixel floods a power-of-two image, a full mask returns the data, and the data
+// gradient under a full mask is the output gradient.
+static void pullpushPart()
+{
+    const int B = 2, C = 3, S = 16;
+    std::vector<float> mask(B * S * S, 0.f), data(B * C * S * S), out(B * C * S * S), adjOut(B * C * S * S);
+    std::default_random_engine rng(7);
+    std::uniform_real_distribution<float> uni(-1.f, 1.f);
+    for (auto& v : data) v = uni(rng);
+    for (auto& v : adjOut) v = uni(rng);
+    for (int b = 0; b < B; ++b) mask[(b * S + 5) * S + 11] = 1.f;
+    Tensor tMask(Tensor::FLOAT, {B, S, S}), tData(Tensor::FLOAT, {B, C, S, S}), tOut(Tensor::FLOAT, {B, C, S, S});
+    tMask.copyFromHost(mask.data(), sizeof(float) * mask.size());
+    tData.copyFromHost(data.data(), sizeof(float) * data.size());
+    Utils::fractionalPullpush(tMask, tData, tOut, nullptr);
+    tOut.copyToHost(out.data(), sizeof(float) * out.size());
+    int bad = 0;
+    for (int b = 0; b < B; ++b)
+        for (int c = 0; c < C; ++c) {
+            const float known = data[((b * C + c) * S + 5) * S + 11];
+            for (int i = 0; i < S * S; ++i) bad += std::fabs(out[(b * C + c) * S * S + i] - known) > 1e-5f;
+        }
+    CHECK(bad == 0);
+
+    std::fill(mask.begin(), mask.end(), 1.f);
+    tMask.copyFromHost(mask.data(), sizeof(float) * mask.size());
+    Utils::fractionalPullpush(tMask, tData, tOut, nullptr);
+    tOut.copyToHost(out.data(), sizeof(float) * out.size());
+    bad = 0;
+    for (size_t i = 0; i < out.size(); ++i) bad += out[i] != data[i];
+    CHECK(bad == 0);
+
+    Tensor tAdjOut(Tensor::FLOAT, {B, C, S, S}), tAdjMask(Tensor::FLOAT, {B, S, S}), tAdjData(Tensor::FLOAT, {B, C, S, S});
+    tAdjOut.copyFromHost(adjOut.data(), sizeof(float) * adjOut.size());
+    tAdjMask.zero_();
+    tAdjData.zero_();
+    Utils::adjointFractionalPullpush(tMask, tData, tAdjOut, tAdjMask, tAdjData, nullptr);
+    tAdjData.copyToHost(out.data(), sizeof(float) * out.size());
+    bad = 0;
+    for (size_t i = 0; i < out.size(); ++i) bad += out[i] != adjOut[i];
+    CHECK(bad == 0);
+
+    bool thrown = false;
+    try {
+        Tensor wide(Tensor::FLOAT, {B, 16, S, S}), wideOut(Tensor::FLOAT, {B, 16, S, S});
+        Utils::fractionalPullpush(tMask, wide, wideOut, nullptr);
+    } catch (const std::runtime_error&) {
+        thrown = true;
+    }
+    CHECK(thrown);
+}
+
 int main(int argc, char** argv)
 {
     const bool hostOnly = argc > 1 && std::strcmp(argv[1], "--host") == 0;
@@ -185,6 +239,7 @@ int main(int argc, char** argv)
         if (!hostOnly) {
             QuickMLP::Instance().checkHipAvailable();
             gpuPart();
+            pullpushPart();
         }
     } catch (const std::exception& e) {
         std::printf("FAILED with exception: %s\n", e.what());
