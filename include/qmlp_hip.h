@@ -104,6 +104,11 @@ int qmlp_hip_module_get_global(qmlp_hip_module module, const char* name, void** 
  * (src_cpp/src/fused_network.cpp:473,540). */
 int qmlp_hip_function_occupancy(qmlp_hip_function function, size_t dynamic_lds_bytes,
                                 int block_size_limit, int* block_size, int* min_grid_size);
+/* Workgroups of block_size threads (with dynamic_lds_bytes of dynamic LDS each) that one
+ * compute unit holds at the same time; what the grid of a persistent kernel is sized with.
+ * No counterpart in cuda-kernel-loader (the reference sizes grids with minGridSize()). */
+int qmlp_hip_function_blocks_per_cu(qmlp_hip_function function, int block_size, size_t dynamic_lds_bytes,
+                                    int* blocks_per_cu);
 /* Register / LDS usage of a loaded function (for logging and launch sizing). */
 int qmlp_hip_function_attributes(qmlp_hip_function function, int* num_vgprs, int* static_lds_bytes,
                                  int* max_threads_per_block, int* scratch_bytes);

@@ -363,6 +363,17 @@ int qmlp_hip_function_occupancy(qmlp_hip_function function, size_t dynamic_lds_b
     return 0;
 }
 
+int qmlp_hip_function_blocks_per_cu(qmlp_hip_function function, int block_size, size_t dynamic_lds_bytes,
+                                    int* blocks_per_cu)
+{
+    int blocks = 0;
+    if (int rc = check(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, function->fn, block_size,
+                                                                          dynamic_lds_bytes),
+                       "hipModuleOccupancyMaxActiveBlocksPerMultiprocessor")) return rc;
+    *blocks_per_cu = blocks;
+    return 0;
+}
+
 int qmlp_hip_function_attributes(qmlp_hip_function function, int* num_vgprs, int* static_lds_bytes,
                                  int* max_threads_per_block, int* scratch_bytes)
 {

@@ -77,11 +77,15 @@ int KernelFunction::minGridSize() const
 int KernelFunction::fullGridSize(int blockSize, size_t dynamicLdsBytes) const
 {
     if (!defined()) throw std::runtime_error("KernelFunction is not defined");
-    int block = 0, grid = 0;
-    QMLP_HIP_CALL(qmlp_hip_function_occupancy(function_, dynamicLdsBytes, blockSize, &block, &grid));
-    // the query maximizes threads; rescale the grid if it settled on a smaller block
-    if (block > 0 && block != blockSize) grid = static_cast<int>(static_cast<long long>(grid) * block / blockSize);
-    return std::max(grid, 1);
+    // workgroups that are resident at the same time: per compute unit x compute units
+    int perCu = 0;
+    QMLP_HIP_CALL(qmlp_hip_function_blocks_per_cu(function_, blockSize, dynamicLdsBytes, &perCu));
+    static const int computeUnits = [] {
+        qmlp_hip_device_props props;
+        QMLP_HIP_CALL(qmlp_hip_get_device_props(0, &props));   // one GPU per process
+        return props.compute_units;
+    }();
+    return std::max(perCu, 1) * std::max(computeUnits, 1);
 }
 
 int KernelFunction::numVgprs() const
