@@ -71,6 +71,7 @@ public:
     [[nodiscard]] std::string parameterName() const override;
     [[nodiscard]] Tensor::Precision parameterPrecision(Tensor::Usage usage) const override;
     [[nodiscard]] int parameterCount() const override;
+    [[nodiscard]] int ldsGradientFloats(int maxBytes, int& levels) const override;
     void setParameter(const Tensor& tensor, Tensor::Usage usage) override;
     [[nodiscard]] int fillParameterMemory(char* dst, int dstSize) override;
     void zeroGradients() override;

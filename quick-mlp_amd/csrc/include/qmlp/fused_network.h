@@ -271,6 +271,15 @@ private:
     // name (inside namespace activations) of the activation type of a layer
     std::string activationTypeName(int layer) const;
     int stageBytesPerWave(bool adjoint) const;
+    /** Leading gradient levels of one encoding that the backward kernel sums in LDS. */
+    struct LdsGradients
+    {
+        int levels = 0;      // scatterTile<levels>
+        int floats = 0;      // size of the LDS region
+        int byteOffset = 0;  // of the region in the kernel's dynamic LDS
+    };
+    /** One entry per encoding; returns the LDS bytes of the backward kernel including these regions. */
+    int ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding) const;
     std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);
     void ensureStreams();
 };

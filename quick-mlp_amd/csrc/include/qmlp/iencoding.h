@@ -79,6 +79,18 @@ public:
     virtual void zeroGradients() {}
 
     /**
+     * For the fused backward kernel: how many leading levels (or other leading parts) of the
+     * parameter gradients a workgroup may sum in LDS before adding them to the gradient
+     * tensor, if it has maxBytes of LDS for that. Returns the number of floats needed (0: none)
+     * and sets 'levels', which the device code receives as scatterTile<levels>.
+     */
+    [[nodiscard]] virtual int ldsGradientFloats(int maxBytes, int& levels) const
+    {
+        levels = 0;
+        return 0;
+    }
+
+    /**
      * Standalone forward pass.
      * \param input shape (B, Cin), float32
      * \param output shape (B, >= numOutputChannels()), float32, unit stride along the channels

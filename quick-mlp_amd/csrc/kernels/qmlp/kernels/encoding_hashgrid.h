@@ -408,6 +408,34 @@ struct EncodingHashGrid
         }
     }
 
+    /** Table elements of the first LEVELS levels. */
+    template <int LEVELS>
+    static constexpr int leadingElements()
+    {
+        if constexpr (LEVELS <= 0) return 0;
+        else if constexpr (LEVELS < L) return Cfg::memoryOffset[LEVELS] - Cfg::memoryOffset[0];
+        else return Cfg::ParameterCount - Cfg::memoryOffset[0];
+    }
+
+    /** Float addition in LDS (a native LDS instruction; p must point into LDS). */
+    __device__ __forceinline__ static void ldsAdd(float* p, float v)
+    {
+        typedef __attribute__((address_space(3))) float lds_float;
+        __hip_atomic_fetch_add((lds_float*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+
+    /** Adds the gradients a workgroup has summed in LDS to the gradient tensor (after a barrier). */
+    template <int LEVELS>
+    __device__ __forceinline__ static void flushLdsGradients(const float* ldsGradients, const param_t& params,
+                                                             int thread, int numThreads)
+    {
+        float* __restrict__ grad = params.parametersBackward + Cfg::memoryOffset[0];
+        for (int e = thread; e < leadingElements<LEVELS>(); e += numThreads) {
+            const float v = ldsGradients[e];
+            if (v != 0.f) unsafeAtomicAdd(grad + e, v);
+        }
+    }
+
     /** True if the gradient scatter of a whole tile (scatterTile) is available. */
     static constexpr bool HasTileScatter = detail::isPow2(static_cast<unsigned>(F)) && 2 * F <= WAVE_SIZE;
 
@@ -420,14 +448,18 @@ struct EncodingHashGrid
      * wavefront covers its 64 points in 2*F rounds of 64/(2F) points. Every lane recomputes the level setup of its point; the
      * arithmetic is free next to the atomics.
      *
+     * \tparam LDS_LEVELS the gradients of this many leading levels are first summed in LDS
+     *    (ldsGradients, leadingElements<LDS_LEVELS>() floats, zeroed by the workgroup) and reach
+     *    global memory once per workgroup through flushLdsGradients: a coarse level receives
+     *    many points per cell, so this saves its share of the atomic requests
      * \param index0 index of the first point of the tile
      * \param adjOutput callable (point of the tile 0..63, output channel of this encoding) ->
      *    adjoint of that output as float
      */
-    template <typename AdjFn>
+    template <int LDS_LEVELS = 0, typename AdjFn>
     __device__ __forceinline__ static void scatterTile(int lane, long long index0, long long numel,
                                                        const Tensor2Read<float>& inputs, const AdjFn& adjOutput,
-                                                       const param_t& params)
+                                                       const param_t& params, float* ldsGradients = nullptr)
     {
         constexpr int G = 2 * F;            // lanes per point
         constexpr int PPR = WAVE_SIZE / G;  // points per round
@@ -478,7 +510,11 @@ struct EncodingHashGrid
                         w = w * (hi ? s.f[d] : (1.f - s.f[d]));
                     }
                     if (hashed) idx %= Cfg::hashGridSize[l];
-                    unsafeAtomicAdd(grad + (base + idx * static_cast<unsigned>(F) + static_cast<unsigned>(i)), (w * wk) * adj);
+                    const unsigned element = idx * static_cast<unsigned>(F) + static_cast<unsigned>(i);
+                    if (l < LDS_LEVELS)
+                        ldsAdd(ldsGradients + (base - static_cast<unsigned>(Cfg::memoryOffset[0]) + element), (w * wk) * adj);
+                    else
+                        unsafeAtomicAdd(grad + (base + element), (w * wk) * adj);
                 }
             }
         }

@@ -50,9 +50,9 @@ struct EncodingLineIntegration
 
     /** Never called (HasTileScatter is false); present because the kernels name it in a
      *  discarded `if constexpr` branch of a non-template function, which is still checked. */
-    template <typename AdjFn>
+    template <int LDS_LEVELS = 0, typename AdjFn>
     __device__ __forceinline__ static void scatterTile(int, long long, long long, const Tensor2Read<float>&,
-                                                       const AdjFn&, const param_t&)
+                                                       const AdjFn&, const param_t&, float* = nullptr)
     {
     }
 

@@ -94,6 +94,9 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
 
     // stage the transposed weights in operand order
 $$STAGE_PARAMETERS$$
+    // gradients of coarse grid levels are summed in LDS first (zeroed here, added to the
+    // gradient tensor once per workgroup after the loop over the tiles)
+$$ZERO_LDS_GRADIENTS$$
     __syncthreads();
 
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
@@ -166,6 +169,7 @@ $$CALL_ENCODING_SCATTER$$
             waveLdsSync();
         }
     }
+$$FLUSH_LDS_GRADIENTS$$
 }
 
 QUICKMLP_KERNEL_NAMESPACE_END

@@ -174,6 +174,7 @@ void EncodingHashGrid::fillCode(std::stringstream& code) const
     code << "    static constexpr bool Concat = "
          << (combinationMode_ == LayerCombinationMode::CONCAT ? "true" : "false") << ";\n";
     code << "    static constexpr bool ResolutionFactor = true;\n";
+    code << "    static constexpr int ParameterCount = " << numParameters_ << ";\n";
     code << "    typedef " << (parameterPrecision_ == Tensor::HALF ? "f16" : "float") << " table_t;\n";
     auto emit = [&](const char* type, const char* field, auto getter) {
         code << "    static constexpr " << type << " " << field << "[" << numLevels_ << "] = {";
@@ -202,6 +203,23 @@ Tensor::Precision EncodingHashGrid::parameterPrecision(Tensor::Usage usage) cons
 }
 
 int EncodingHashGrid::parameterCount() const { return numParameters_; }
+
+int EncodingHashGrid::ldsGradientFloats(int maxBytes, int& levels) const
+{
+    levels = 0;
+    // the device code scatters per tile only for these feature counts (HasTileScatter)
+    const int F = numFeaturesPerLevel_;
+    if ((F & (F - 1)) != 0 || 2 * F > 64) return 0;
+    int floats = 0;
+    for (int l = 0; l < numLevels_; ++l) {
+        const int end = l + 1 < numLevels_ ? layers_[l + 1].memoryOffset : numParameters_;
+        const int upTo = end - layers_[0].memoryOffset;
+        if (static_cast<long long>(upTo) * static_cast<long long>(sizeof(float)) > maxBytes) break;
+        levels = l + 1;
+        floats = upTo;
+    }
+    return floats;
+}
 
 void EncodingHashGrid::setParameter(const Tensor& tensor, Tensor::Usage usage)
 {

@@ -645,6 +645,27 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
     return code;
 }
 
+int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding) const
+{
+    perEncoding.assign(encodings_.size(), LdsGradients{});
+    int bytes = ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (blockSize / WARP_SIZE) * stageBytesPerWave(true);
+    if (!(adjointFlags & GRADIENTS_INPUT_ENCODINGS)) return bytes;
+    // Up to 96 KiB of LDS per workgroup in total: a coarse level of a grid fits (16^3 cells with
+    // 2 features: 32 KiB), and a second workgroup per compute unit stays possible.
+    const int limit = std::min(MaxSharedMemoryBytes(), 96 * 1024);
+    for (size_t i = 0; i < encodings_.size(); ++i) {
+        if (!encodings_[i]->hasParameters()) continue;
+        bytes = roundUp(bytes, 16);
+        LdsGradients g;
+        g.floats = encodings_[i]->ldsGradientFloats(limit - bytes, g.levels);
+        if (g.floats <= 0) continue;
+        g.byteOffset = bytes;
+        bytes += g.floats * static_cast<int>(sizeof(float));
+        perEncoding[i] = g;
+    }
+    return bytes;
+}
+
 std::string FusedNetwork::backwardSource(int flags, int blockSize) const
 {
     const bool hasInputGradients = flags & GRADIENTS_INPUT;
@@ -714,12 +735,22 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
     replaceAll(code, "$$HAS_STREAMED_LAYERS$$", anyStreamed ? "true" : "false");
 
-    std::stringstream callEncodings, callScatter;
+    std::stringstream callEncodings, callScatter, zeroLds, flushLds;
+    std::vector<LdsGradients> ldsGradients;
+    ldsGradientLayout(flags, blockSize, ldsGradients);
     int encodingOffset = 0;
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
         const bool parameterGradients = hasEncodingGradients && e->hasParameters();
         const std::string name = e->qualifiedName();
+        const LdsGradients& lg = ldsGradients[encodingIdx];
+        if (lg.levels > 0) {
+            zeroLds << "    float* sGradients" << encodingIdx << " = reinterpret_cast<float*>(sMemory + " << lg.byteOffset
+                    << ");\n    for (int e = threadIdx.x; e < " << lg.floats << "; e += blockDim.x) sGradients"
+                    << encodingIdx << "[e] = 0.f;\n";
+            flushLds << "    " << name << "::template flushLdsGradients<" << lg.levels << ">(sGradients" << encodingIdx
+                     << ", cEncoding" << encodingIdx << ", threadIdx.x, blockDim.x);\n";
+        }
         // encodings with a tile-wide scatter take their parameter gradients out of the per-point call
         const std::string perPointParameterGradients =
             parameterGradients ? "!" + name + "::HasTileScatter" : std::string("false");
@@ -729,15 +760,20 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
                       << ">(encodingInput, adjEncodingOutputK, adjEncodingInput";
         if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
         callEncodings << ");\n                }\n";
-        if (parameterGradients)
+        if (parameterGradients) {
             callScatter << "            if constexpr (" << name << "::HasTileScatter)\n                " << name
-                        << "::scatterTile(lane, static_cast<long long>(tile) * TILE_POINTS, numel, inputs,\n"
+                        << "::template scatterTile<" << lg.levels << ">(lane, static_cast<long long>(tile) * TILE_POINTS, numel, inputs,\n"
                         << "                    [&](int pt, int c) { return static_cast<float>(sStage[stageRow(pt) * STAGE_STRIDE + "
-                        << encodingOffset << " + c]); },\n                    cEncoding" << encodingIdx << ");\n";
+                        << encodingOffset << " + c]); },\n                    cEncoding" << encodingIdx;
+            if (lg.levels > 0) callScatter << ", sGradients" << encodingIdx;
+            callScatter << ");\n";
+        }
         encodingOffset += e->numOutputChannels();
     }
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
     replaceAll(code, "$$CALL_ENCODING_SCATTER$$", callScatter.str());
+    replaceAll(code, "$$ZERO_LDS_GRADIENTS$$", zeroLds.str());
+    replaceAll(code, "$$FLUSH_LDS_GRADIENTS$$", flushLds.str().empty() ? std::string() : "    __syncthreads();\n" + flushLds.str());
     return code;
 }
 
@@ -870,8 +906,10 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
 
     AdjointKernel ak;
     ak.adjoint.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
-    ak.adjoint.sharedMemorySize =
-        ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (ak.adjoint.blockSize / WARP_SIZE) * stageBytesPerWave(true);
+    {
+        std::vector<LdsGradients> ldsGradients;
+        ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients);
+    }
     const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize);
     ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
     {
