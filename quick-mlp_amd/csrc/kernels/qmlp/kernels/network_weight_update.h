@@ -40,7 +40,7 @@ $$DEFINE_ACTIVATIONS$$
  * \tparam MO_CHUNK number of 16-row output tiles and
  * \tparam KI_CHUNK number of 16-column input tiles one workgroup accumulates: a workgroup owns a
  *         MO_CHUNK x KI_CHUNK block of the 16 x 16 tiles of dW. The grid is
- *         (COUT/16/MO_CHUNK) x (CIN/16/KI_CHUNK) blocks x batch slices, block index fastest.
+ *         (COUT/16/MO_CHUNK) x (CIN/16/KI_CHUNK) blocks x batch slices.
  *         Splitting the input channels re-reads dpre, splitting the output channels re-reads
  *         the input and re-applies its activation; the host picks the cheaper split.
  */
@@ -67,9 +67,18 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
     const int wave = threadIdx.x / WAVE_SIZE;
     const int lane = threadIdx.x % WAVE_SIZE;
     const int g = lane >> 4, r = lane & 15;
-    const int chunk = blockIdx.x % NCHUNK;
-    const int slice = blockIdx.x / NCHUNK;
+    // Workgroups are handed to the 8 XCDs in turn. The NCHUNK workgroups that read the same
+    // slice of the batch (different blocks of dW) are therefore placed 8 apart, onto the same
+    // XCD: the operand they share is then read from HBM once and from that XCD's L2 afterwards.
     const int numSlices = gridDim.x / NCHUNK;
+    int chunk, slice;
+    if (NCHUNK > 1 && numSlices % 8 == 0) {
+        chunk = (blockIdx.x / 8) % NCHUNK;
+        slice = (blockIdx.x / (8 * NCHUNK)) * 8 + blockIdx.x % 8;
+    } else {
+        chunk = blockIdx.x % NCHUNK;
+        slice = blockIdx.x / NCHUNK;
+    }
     const int mo0 = (chunk % MCHUNKS) * MO_CHUNK;
     const int ki0 = (chunk / MCHUNKS) * KI_CHUNK;
     const bool ownsBias = BIAS && ki0 == 0;   // the bias gradient does not depend on the input channels
