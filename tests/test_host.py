@@ -333,3 +333,35 @@ def test_pullpush_host_side(tmp_path):
         call(mask[0], torch.zeros(1, 2, 4, 4))
     with pytest.raises(ValueError, match="GPU tensors only"):
         qpp.pullpush(mask, torch.zeros(1, 2, 4, 4))
+
+
+def test_kernel_cache_key_covers_only_the_headers_a_source_includes(tmp_path):
+    """Editing a device header recompiles the kernels that can reach it and no others."""
+    import shutil
+    import subprocess
+    import sys
+    kernels = tmp_path / "kernels"
+    shutil.copytree(os.path.join(ROOT, "quick-mlp_amd", "csrc", "kernels"), kernels)
+    cache = tmp_path / "cache"
+    script = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import torch, qmlp\n"
+        "qmlp.set_log_level('error')\n"
+        "qmlp.Activation('relu').precompile()\n"
+        "qmlp.pullpush.precompile(torch.float32)\n"
+        "print(*qmlp._lib.kernel_cache_stats())\n" % os.path.join(ROOT, "quick-mlp_amd"))
+    env = dict(os.environ, QMLP_KERNEL_DIR=str(kernels), QMLP_CACHE_DIR=str(cache))
+
+    def run():
+        out = subprocess.run([sys.executable, "-c", script], env=env, capture_output=True, text=True, check=True).stdout
+        compiled, hits = (int(v) for v in out.split()[-2:])
+        return compiled, hits
+
+    assert run() == (12, 0)                      # 2 activation kernels + 10 pull-push kernels
+    assert run() == (0, 12)
+    with open(kernels / "qmlp" / "kernels" / "pullpush.h", "a") as f:
+        f.write("\n// edited\n")
+    assert run() == (10, 2)                      # the activation kernels do not include pullpush.h
+    with open(kernels / "qmlp" / "kernels" / "common.h", "a") as f:
+        f.write("\n// edited\n")
+    assert run() == (12, 0)                      # everything includes common.h
