@@ -550,3 +550,25 @@ def test_full_size_properties_cfg4_cfg5(cfg_id, N):
     # intrinsics (cfg4) and ReLU units switching next to zero (cfg5)
     assert_close(whole["adj_x"][sample] / s, ref["adj_x"] / s, "sampled input gradients", rel=5e-3, abs_=1e-3,
                  allowed_fraction=2e-3)
+
+
+def test_batch_with_more_than_2_to_the_31_input_elements():
+    """2^28 points of 16 channels: element offsets beyond 32 bits. The points at both ends and
+    around the 2^31-element mark give the same bits as in a small batch of their own."""
+    case = Case(identity_cfg(16, [16, 1], ["relu", "identity"], [False, False]))
+    rng = np.random.default_rng(5)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    N = 1 << 28
+    print("large batch: %d points" % N, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.rand((N, 16), device="cuda", generator=g) * 2 - 1
+    out = case.net.inference(x, case.params, [None])
+    assert out.shape == (N, 1)
+    mark = (1 << 31) // 16
+    for start in (0, mark - 500, N - 1000):
+        part = x[start:start + 1000].contiguous()
+        assert torch.equal(case.net.inference(part, case.params, [None]), out[start:start + 1000])
+    sample = x[mark - 64:mark + 64].cpu().numpy()
+    assert_close(out[mark - 64:mark + 64].cpu().numpy(), case.oracle.forward(sample), "around the 2^31 mark")
+    del x, out
+    torch.cuda.empty_cache()
