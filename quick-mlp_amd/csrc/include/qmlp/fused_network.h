@@ -240,6 +240,10 @@ private:
     bool hasLargeVariant(bool store) const;
     void compileForwardKernel(bool store, int variant, bool compileOnly = false);
     const CompiledKernel& forwardKernelFor(bool store, int numTiles);
+    /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
+    int gatherChunkPoints(const CompiledKernel& ck) const;
+    /** inference (store = false) or forward with stored intermediates, in one or several launches. */
+    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane) const;
@@ -247,7 +251,7 @@ private:
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const;
     void fillEncodingsAndActivations(std::string& codeTemplate) const;
-    int forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane = nullptr) const;
+    int forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane = nullptr, int fixedPointsPerLane = 0) const;
     int weightUpdateBlockSize() const;
     // number of batch slices whose partial weight gradients are kept in the adjoint memory
     int weightUpdateSlices(int numTiles) const;

@@ -48,6 +48,8 @@ public:
     [[nodiscard]] int minGridSize() const;
     /** Blocks of 'blockSize' threads with 'dynamicLdsBytes' that fill the device once. */
     [[nodiscard]] int fullGridSize(int blockSize, size_t dynamicLdsBytes) const;
+    /** Compute units of the device. */
+    [[nodiscard]] static int computeUnits();
     [[nodiscard]] int numVgprs() const;
     [[nodiscard]] int scratchBytes() const;
 

@@ -36,7 +36,9 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     const Tensor2Read<float> inputs,  //shape (numel, Cin)
     Tensor2RW<float> outputs,         //shape (numel, Cout)
     const half* __restrict__ networkParametersH,
-    half* __restrict__ forwardTmpMemoryH
+    half* __restrict__ forwardTmpMemoryH,
+    int tmpTileOffset,                // STORE: index of this launch's first tile in the whole batch
+    int tmpNumTiles                   // STORE: tiles of the whole batch (a batch may be cut into several launches)
     $$ENCODING_PARAMETERS$$)
 {
     constexpr int NUM_INPUTS = $$NUM_INPUTS$$;            // raw input channels
@@ -70,7 +72,8 @@ $$STAGE_PARAMETERS$$
     __syncthreads();
 
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
-    const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
+    // the regions of the temporary memory are laid out for the whole batch
+    const long long numel64 = static_cast<long long>(tmpNumTiles) * TILE_POINTS;
     (void)numel64;
     for (int tileBase = blockIdx.x * WAVES * PPL; tileBase < numTiles; tileBase += gridDim.x * WAVES * PPL)
     {
@@ -116,6 +119,8 @@ $$CALL_ENCODINGS$$
         const int tile = tile0 + q;
         if (!HAS_STREAMED_LAYERS && tile >= numTiles) break;
         const bool tileValid = tile < numTiles;
+        const int tmpTile = tile + tmpTileOffset;
+        (void)tmpTile;
         const f16* sTile = sStage + q * (TILE_POINTS * STAGE_STRIDE);
 
         // B operands of the first layer
@@ -128,7 +133,7 @@ $$CALL_ENCODINGS$$
 
         if (STORE && tileValid) {
             // encoded input, channel-major per tile, for the weight update of layer 0
-            f16* encTile = forwardTmpMemory + static_cast<long long>(tile) * (CHANNELS_IN * TILE_POINTS);
+            f16* encTile = forwardTmpMemory + static_cast<long long>(tmpTile) * (CHANNELS_IN * TILE_POINTS);
 #pragma unroll
             for (int t = 0; t < KT0; ++t)
 #pragma unroll

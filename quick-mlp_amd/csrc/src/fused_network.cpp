@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <limits>
 #include <sstream>
 #include <unordered_set>
 
@@ -502,7 +503,7 @@ int FusedNetwork::stageBytesPerWave(bool adjoint) const
     return TILE_POINTS * (c + (rotated ? 0 : STAGE_PAD)) * static_cast<int>(sizeof(half));
 }
 
-int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane) const
+int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLane, int fixedPointsPerLane) const
 {
     int blockSize = DEFAULT_BLOCK_SIZE;
     if (overwrite > 0) {
@@ -524,8 +525,9 @@ int FusedNetwork::forwardBlockSize(int overwrite, bool adjoint, int* pointsPerLa
         // should still fit on a compute unit.
         bool gathers = false;
         for (const auto& e : encodings_) gathers = gathers || e->hasParameters();
-        ppl = compileOptions_.pointsPerLane > 0 ? compileOptions_.pointsPerLane : (gathers ? 2 : 1);
-        const int budget = compileOptions_.pointsPerLane > 0 ? maxLds : maxLds / 2;
+        const int fixed = fixedPointsPerLane > 0 ? fixedPointsPerLane : compileOptions_.pointsPerLane;
+        ppl = fixed > 0 ? fixed : (gathers ? 2 : 1);
+        const int budget = fixed > 0 ? maxLds : maxLds / 2;
         while (ppl > 1 && paramBytes + (blockSize / WARP_SIZE) * ppl * stageBytesPerWave(adjoint) > budget) --ppl;
         *pointsPerLane = ppl;
     }
@@ -637,7 +639,7 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
         else
             callLayers << "nullptr";
         callLayers << ", x" << i << ", x" << (i + 1) << ",\n            (STORE && tileValid) ? forwardTmpMemory + ("
-                   << backwardInfo_[i].offsetPre << "ll * numel64 + static_cast<long long>(tile) * ("
+                   << backwardInfo_[i].offsetPre << "ll * numel64 + static_cast<long long>(tmpTile) * ("
                    << l.channelsOut << " * TILE_POINTS)) : nullptr, lane);\n";
     }
     callLayers << "        auto& xOut = x" << layers_.size() << ";\n";
@@ -857,9 +859,10 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
     if (slot.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
+    // the narrow shape is sized like a network with one tile per wave (smaller workgroups when
+    // the weights allow it: a small batch then spreads over more compute units)
     ck.blockSize = forwardBlockSize(store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference,
-                                    false, &ck.pointsPerLane);
-    if (variant == VARIANT_NARROW) ck.pointsPerLane = 1;
+                                    false, &ck.pointsPerLane, variant == VARIANT_NARROW ? 1 : 0);
     if (variant == VARIANT_LARGE) {
         ck.blockSize = 2 * DEFAULT_BLOCK_SIZE;
         ck.pointsPerLane = 4;
@@ -881,19 +884,31 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
 const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles)
 {
     const int s = store ? 1 : 0;
-    if (hasLargeVariant(store)) {
-        compileForwardKernel(store, VARIANT_LARGE);
-        const auto& large = forwardKernels_[s][VARIANT_LARGE].value();
-        if (divUp(numTiles, (large.blockSize / WARP_SIZE) * large.pointsPerLane) >= large.fullGrid) return large;
-    }
     compileForwardKernel(store, VARIANT_DEFAULT);
     const auto& wide = forwardKernels_[s][VARIANT_DEFAULT].value();
-    if (wide.pointsPerLane == 1) return wide;
-    // several tiles per wave only pay off while they still fill most of the compute units
-    const int waves = wide.blockSize / WARP_SIZE;
-    if (2 * divUp(numTiles, waves * wide.pointsPerLane) >= wide.fullGrid) return wide;
-    compileForwardKernel(store, VARIANT_NARROW);
-    return forwardKernels_[s][VARIANT_NARROW].value();
+    if (wide.pointsPerLane == 1) return wide;   // no gathers, or a pinned shape: one kernel
+    // Kernels that take more tiles per wave are faster per point, but the time grows in steps
+    // of one workgroup per compute unit, whether all compute units have one or not. Measured on
+    // a 16-level hash grid, per step: 4 waves x 1 tile 26 us (2^16 points), 8 waves x 2 tiles
+    // 82 us (2^18 points), 8 waves x 4 tiles 153 us (2^19 points). Take the shape with the
+    // least estimated time = steps x points per step x relative cost per point.
+    const CompiledKernel* best = nullptr;
+    double bestCost = 0;
+    const int computeUnits = KernelFunction::computeUnits();
+    auto consider = [&](int variant, double costPerPoint) {
+        compileForwardKernel(store, variant);
+        const auto& k = forwardKernels_[s][variant].value();
+        const long long stepTiles = static_cast<long long>(computeUnits) * (k.blockSize / WARP_SIZE) * k.pointsPerLane;
+        const double cost = static_cast<double>(divUp<long long>(numTiles, stepTiles)) * stepTiles * costPerPoint;
+        if (!best || cost < bestCost) {
+            best = &k;
+            bestCost = cost;
+        }
+    };
+    if (hasLargeVariant(store)) consider(VARIANT_LARGE, 1.0);
+    consider(VARIANT_DEFAULT, 1.075);
+    consider(VARIANT_NARROW, 1.39);
+    return *best;
 }
 
 void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
@@ -970,6 +985,20 @@ void FusedNetwork::precompile(int adjointFlags)
 
 // ------------------------------------------------------------------ launches
 
+int FusedNetwork::gatherChunkPoints(const CompiledKernel& ck) const
+{
+    // The workgroups of a launch walk the levels of a grid side by side, which keeps the table
+    // of the level in use in L2. Over many passes they drift apart and several level tables
+    // compete for the L2: cfg2 at 2^24 points took 602 ps per point in one launch, against 288
+    // at 2^20. Batches of a network that gathers are therefore cut into launches of two
+    // passes each; a launch boundary brings the workgroups back in step.
+    bool gathers = false;
+    for (const auto& e : encodings_) gathers = gathers || e->hasParameters();
+    if (!gathers) return std::numeric_limits<int>::max();
+    const long long pass = static_cast<long long>(KernelFunction::computeUnits()) * (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * TILE_POINTS;
+    return static_cast<int>(std::min<long long>(2 * pass, std::numeric_limits<int>::max()));
+}
+
 std::vector<char> FusedNetwork::encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage)
 {
     storage.clear();
@@ -997,18 +1026,34 @@ void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t strea
     CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
     if (numel == 0) return;
 
-    const int numTiles = divUp(numel, TILE_POINTS);
-    const auto& ck = forwardKernelFor(false, numTiles);
-    const int waves = ck.blockSize / WARP_SIZE;
-    const int grid = std::min(divUp(numTiles, waves * ck.pointsPerLane), ck.fullGrid);
-    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
-    auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
+    launchForward(false, input, output, nullptr, stream);
+}
+
+void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream)
+{
+    const int numel = input.size(0);
+    int tmpNumTiles = divUp(numel, TILE_POINTS);
+    const auto inputAll = input.accessor<kernel::Tensor2Read<float>>();
+    const auto outputAll = output.accessor<kernel::Tensor2RW<float>>();
     const half* networkParams = parametersInference_.dataPtr<half>();
-    half* tmpMemory = nullptr;
-    std::vector<void*> args = {&numel, &inputAcc, &outputAcc, &networkParams, &tmpMemory};
-    std::vector<std::vector<char>> storage;
-    encodingArguments(args, storage);
-    ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+    for (long long start = 0; start < numel;) {
+        // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
+        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)));
+        int count = static_cast<int>(std::min<long long>(gatherChunkPoints(ck), numel - start));
+        auto inputAcc = inputAll;
+        auto outputAcc = outputAll;
+        inputAcc.data_ += start * inputAll.strides_[0];
+        outputAcc.data_ += start * outputAll.strides_[0];
+        inputAcc.sizes_[0] = outputAcc.sizes_[0] = count;
+        int tmpTileOffset = static_cast<int>(start / TILE_POINTS);
+        const int waves = ck.blockSize / WARP_SIZE;
+        const int grid = std::min(divUp(divUp(count, TILE_POINTS), waves * ck.pointsPerLane), ck.fullGrid);
+        std::vector<void*> args = {&count, &inputAcc, &outputAcc, &networkParams, &tmpMemory, &tmpTileOffset, &tmpNumTiles};
+        std::vector<std::vector<char>> storage;
+        encodingArguments(args, storage);
+        ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+        start += count;
+    }
 }
 
 size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlags)
@@ -1040,18 +1085,7 @@ void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory,
     CHECK_ERROR(tmpMemory != nullptr, "forward() needs temporary memory of forwardMemory() bytes");
     CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemory) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
 
-    const int numTiles = divUp(numel, TILE_POINTS);
-    const auto& ck = forwardKernelFor(true, numTiles);
-    const int waves = ck.blockSize / WARP_SIZE;
-    const int grid = std::min(divUp(numTiles, waves * ck.pointsPerLane), ck.fullGrid);
-    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
-    auto outputAcc = output.accessor<kernel::Tensor2RW<float>>();
-    const half* networkParams = parametersInference_.dataPtr<half>();
-    half* tmpMemoryHalf = static_cast<half*>(tmpMemory);
-    std::vector<void*> args = {&numel, &inputAcc, &outputAcc, &networkParams, &tmpMemoryHalf};
-    std::vector<std::vector<char>> storage;
-    encodingArguments(args, storage);
-    ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+    launchForward(true, input, output, static_cast<half*>(tmpMemory), stream);
 }
 
 void FusedNetwork::zeroGradients()

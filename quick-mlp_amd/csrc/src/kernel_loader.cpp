@@ -80,12 +80,17 @@ int KernelFunction::fullGridSize(int blockSize, size_t dynamicLdsBytes) const
     // workgroups that are resident at the same time: per compute unit x compute units
     int perCu = 0;
     QMLP_HIP_CALL(qmlp_hip_function_blocks_per_cu(function_, blockSize, dynamicLdsBytes, &perCu));
-    static const int computeUnits = [] {
+    return std::max(perCu, 1) * computeUnits();
+}
+
+int KernelFunction::computeUnits()
+{
+    static const int value = [] {
         qmlp_hip_device_props props;
         QMLP_HIP_CALL(qmlp_hip_get_device_props(0, &props));   // one GPU per process
-        return props.compute_units;
+        return std::max(props.compute_units, 1);
     }();
-    return std::max(perCu, 1) * std::max(computeUnits, 1);
+    return value;
 }
 
 int KernelFunction::numVgprs() const

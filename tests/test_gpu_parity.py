@@ -572,3 +572,38 @@ def test_batch_with_more_than_2_to_the_31_input_elements():
     assert_close(out[mark - 64:mark + 64].cpu().numpy(), case.oracle.forward(sample), "around the 2^31 mark")
     del x, out
     torch.cuda.empty_cache()
+
+
+def test_grid_network_batches_that_take_several_launches():
+    """Networks that gather are run in launches of at most two steps of the resident workgroups
+    (2^20 points for configuration 2). A longer batch has to give the same bits as its parts
+    cut anywhere else, and the intermediates of a forward pass in several launches have to
+    serve the backward pass: gradients are additive over a split of the batch."""
+    case, rng = baseline_case(3, table_scale=1.0)
+    N = (1 << 20) + (1 << 19) + 1000
+    X = bc.make_inputs(3, N, rng)
+    x = torch.from_numpy(X).cuda()
+    enc = case.encoding_parameters()
+    print("several launches: inference of %d points" % N, flush=True)
+    whole = case.net.inference(x, case.params, enc)
+    cut = 700001
+    parts = torch.cat([case.net.inference(x[:cut], case.params, enc), case.net.inference(x[cut:], case.params, enc)])
+    assert torch.equal(whole, parts)
+    sample = np.arange(0, N, 4099)
+    ref = case.oracle.forward(X[sample], round_mode=1)
+    s = float(np.abs(ref).max())
+    assert_close(whole.cpu().numpy()[sample] / s, ref / s, "sampled oracle check", rel=5e-3, abs_=1e-3, allowed_fraction=1e-3)
+
+    print("several launches: train step", flush=True)
+    adj = rng.uniform(-1, 1, (N, 1)).astype(np.float32)
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    a = case.gpu_train(X, adj, flags)
+    b = case.gpu_train(X[:cut], adj[:cut], flags)
+    c = case.gpu_train(X[cut:], adj[cut:], flags)
+    assert np.array_equal(a["out"], np.concatenate([b["out"], c["out"]]))
+    assert np.array_equal(a["adj_x"], np.concatenate([b["adj_x"], c["adj_x"]]))
+    s = float(np.abs(a["grads"]).max())
+    assert_close((b["grads"] + c["grads"]) / s, a["grads"] / s, "additivity of the weight gradients", rel=1e-3, abs_=1e-4)
+    t = a["table_grads"][0]
+    assert_close(b["table_grads"][0] + c["table_grads"][0], t, "additivity of the grid gradients", rel=1e-3,
+                 abs_=1e-4 * float(np.abs(t).max()))
