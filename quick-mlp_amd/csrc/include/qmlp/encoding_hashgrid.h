@@ -72,6 +72,7 @@ public:
     [[nodiscard]] Tensor::Precision parameterPrecision(Tensor::Usage usage) const override;
     [[nodiscard]] int parameterCount() const override;
     [[nodiscard]] int ldsGradientFloats(int maxBytes, int& levels) const override;
+    [[nodiscard]] int numSweptTables() const override { return numLevels_; }
     void setParameter(const Tensor& tensor, Tensor::Usage usage) override;
     [[nodiscard]] int fillParameterMemory(char* dst, int dstSize) override;
     void zeroGradients() override;

@@ -84,6 +84,13 @@ public:
      * tensor, if it has maxBytes of LDS for that. Returns the number of floats needed (0: none)
      * and sets 'levels', which the device code receives as scatterTile<levels>.
      */
+    /**
+     * Number of parameter tables that the fused forward kernel sweeps one after the other
+     * (the levels of a grid). With two or more, the workgroups of a launch should stay in
+     * step so that only the table in use occupies the L2; 0 for encodings without tables.
+     */
+    [[nodiscard]] virtual int numSweptTables() const { return 0; }
+
     [[nodiscard]] virtual int ldsGradientFloats(int maxBytes, int& levels) const
     {
         levels = 0;
