@@ -334,6 +334,35 @@ def test_fused_grid_network_against_oracle(precision):
     assert got_e["adj_x"] is None and got_e["grads"] is None
 
 
+def test_network_with_two_grids_against_oracle():
+    """Two grid encodings in one network (a 2-D hashed one with 4 features and a small dense 3-D one
+    whose gradients are all summed in LDS first) next to an identity encoding."""
+    grid_a = _grid_cfg(dict(n_in=2, n_levels=5, n_features_per_level=4, log2_hashmap_size=9, min_resolution=4,
+                            max_resolution=96), "half", start=0)
+    grid_b = _grid_cfg(dict(n_in=3, n_levels=2, n_features_per_level=2, log2_hashmap_size=-1, min_resolution=5,
+                            max_resolution=9), "float", start=2)
+    cfg = {"num_inputs": 5, "num_outputs": 2, "activation_specification": ["qmlp/builtin-activations.json"],
+           "encodings": [grid_a, grid_b, {"id": "Identity", "start_in": 1, "n_in": 3}],
+           "network": [{"n_out": 48, "bias": True, "activation": "sine"},
+                       {"n_out": 32, "bias": False, "activation": "celu"},
+                       {"n_out": 2, "bias": True, "activation": "identity"}]}
+    case = Case(cfg)
+    rng = np.random.default_rng(31)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    for i in (0, 1):
+        case.set_table(i, rng.uniform(-1, 1, case.oracle.encodings[i][1].n_params))
+    N = 7001
+    lo = np.array(grid_a["bounding_box_min"] + grid_b["bounding_box_min"], np.float32)
+    sz = np.array(grid_a["bounding_box_size"] + grid_b["bounding_box_size"], np.float32)
+    X = (lo + sz * rng.uniform(-0.05, 1.05, (N, 5))).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+    assert_close(case.gpu_inference(X), case.oracle.forward(X), "inference")
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    got = case.gpu_train(X, adj, flags)
+    assert_close(got["out"], case.oracle.forward(X), "forward")
+    check_gradients(case, X, adj, flags, got)
+
+
 # ---------------------------------------------------------------------------- line integration
 def _line_cfg(blending, precision="float", start=0):
     child = {"id": "HashGrid", "start_in": 0, "n_in": 3, "n_levels": 4, "n_features_per_level": 2,
