@@ -272,7 +272,8 @@ void FusedNetwork::initializeInferenceParameters(std::default_random_engine& rng
     std::vector<half> dataHost(static_cast<size_t>(parametersInference_.numel()), static_cast<half>(0));
     for (int layer = 0; layer < numLayers(); ++layer) {
         const auto& l = layers_[layer];
-        const float bound = 1.0f / std::sqrt(static_cast<float>(l.channelsIn));
+        // std::sqrt of an int is evaluated in double, as in the reference (fused_network.cpp:294)
+        const float bound = static_cast<float>(1.0f / std::sqrt(static_cast<double>(l.channelsIn)));
         std::uniform_real_distribution<float> distr1(-bound, +bound);
         Tensor weights = networkParameter(layer, false, dataHost.data(), Tensor::HALF);
         for (int32_t i = 0; i < weights.size(0); ++i)
