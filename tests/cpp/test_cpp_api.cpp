@@ -87,6 +87,26 @@ static void gpuPart()
     params.copyToHost(hp.data(), sizeof(half) * P);
     std::vector<float> p(P);
     for (int i = 0; i < P; ++i) p[i] = halfToFloat(hp[i]);
+    {
+        // the draw order of initializeInferenceParameters (src_cpp/src/fused_network.cpp:280-312 of
+        // the reference): per layer the weight matrix row by row, then the bias, one engine,
+        // U(-1/sqrt(padded fan-in), +1/sqrt(padded fan-in)) rounded to half
+        std::default_random_engine again(42);
+        std::vector<float> expected(P, 0.f);
+        const int fanIn[2] = {K, H}, fanOut[2] = {H, K};
+        const int weightStart[2] = {0, H * K}, biasStart[2] = {2 * H * K, -1};
+        for (int layer = 0; layer < 2; ++layer) {
+            const float bound = static_cast<float>(1.0f / std::sqrt(static_cast<double>(fanIn[layer])));
+            std::uniform_real_distribution<float> distr(-bound, +bound);
+            for (int i = 0; i < fanOut[layer] * fanIn[layer]; ++i)
+                expected[weightStart[layer] + i] = halfToFloat(static_cast<half>(distr(again)));
+            if (biasStart[layer] >= 0)
+                for (int i = 0; i < fanOut[layer]; ++i) expected[biasStart[layer] + i] = halfToFloat(static_cast<half>(distr(again)));
+        }
+        int different = 0;
+        for (int i = 0; i < P; ++i) different += p[i] != expected[i];
+        CHECK(different == 0);
+    }
     const float* W0 = p.data();            // (32, 16)
     const float* W1 = p.data() + H * K;    // (16, 32)
     const float* b0 = p.data() + 2 * H * K;
