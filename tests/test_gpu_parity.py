@@ -203,6 +203,9 @@ GRID_SPECS = [
          combination_mode="add"),
     dict(n_in=5, n_levels=2, n_features_per_level=2, log2_hashmap_size=8, min_resolution=2, max_resolution=7),
     dict(n_in=6, n_levels=2, n_features_per_level=1, log2_hashmap_size=12, min_resolution=2, max_resolution=5),
+    # many features per entry: 32 and 64 lanes share one point in the gradient scatter
+    dict(n_in=2, n_levels=2, n_features_per_level=16, log2_hashmap_size=6, min_resolution=3, max_resolution=12),
+    dict(n_in=2, n_levels=1, n_features_per_level=32, log2_hashmap_size=-1, min_resolution=5, max_resolution=5),
 ]
 
 
@@ -360,6 +363,31 @@ def test_network_with_two_grids_against_oracle():
     flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
     got = case.gpu_train(X, adj, flags)
     assert_close(got["out"], case.oracle.forward(X), "forward")
+    check_gradients(case, X, adj, flags, got)
+
+
+@pytest.mark.parametrize("features,levels", [(16, 2), (32, 1), (1, 6)])
+def test_fused_network_with_wide_and_narrow_grid_entries(features, levels):
+    """1, 16 and 32 features per entry in the fused kernels: 2, 32 and 64 lanes share a point
+    when the grid gradients are scattered."""
+    grid = _grid_cfg(dict(n_in=2, n_levels=levels, n_features_per_level=features, log2_hashmap_size=7,
+                          min_resolution=3, max_resolution=3 if levels == 1 else 40), "half", start=0)
+    cfg = {"num_inputs": 2, "num_outputs": 2, "activation_specification": ["qmlp/builtin-activations.json"],
+           "encodings": [grid],
+           "network": [{"n_out": 32, "bias": True, "activation": "celu"},
+                       {"n_out": 2, "bias": False, "activation": "identity"}]}
+    case = Case(cfg)
+    rng = np.random.default_rng(features)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    case.set_table(0, rng.uniform(-1, 1, case.oracle.encodings[0][1].n_params))
+    N = 3001
+    lo = np.array(grid["bounding_box_min"], np.float32)
+    sz = np.array(grid["bounding_box_size"], np.float32)
+    X = (lo + sz * rng.uniform(0, 1, (N, 2))).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+    assert_close(case.gpu_inference(X), case.oracle.forward(X), "inference")
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    got = case.gpu_train(X, adj, flags)
     check_gradients(case, X, adj, flags, got)
 
 
