@@ -135,26 +135,30 @@ _PRECISION_OF = {torch.float32: QMLP_FLOAT, torch.float16: QMLP_HALF, torch.floa
 DTYPE_OF = {QMLP_FLOAT: torch.float32, QMLP_HALF: torch.float16, QMLP_DOUBLE: torch.float64}
 
 
+# one pack call per descriptor: field-by-field assignment of a ctypes structure costs more than
+# the launch of a small kernel
+_PACK = {n: __import__("struct").Struct("<Qii%di%dx%di%dx" % (n, 4 * (4 - n), n, 4 * (4 - n))) for n in range(1, 5)}
+
+
 def desc(t):
     """Tensor descriptor of a torch tensor (None -> undefined tensor)."""
-    d = TensorDesc()
     if t is None:
-        return d
+        return TensorDesc()
+    n = t.dim()
     if t.dtype not in _PRECISION_OF:
         raise TypeError("unsupported dtype %s" % t.dtype)
-    if t.dim() < 1 or t.dim() > 4:
+    if n < 1 or n > 4:
         raise ValueError("tensors must have 1 to 4 dimensions")
-    d.data = t.data_ptr()
-    d.precision = _PRECISION_OF[t.dtype]
-    d.ndim = t.dim()
-    for i in range(t.dim()):
-        d.sizes[i] = t.shape[i]
-        d.strides[i] = t.stride(i)
-    return d
+    return TensorDesc.from_buffer_copy(_PACK[n].pack(t.data_ptr(), _PRECISION_OF[t.dtype], n, *t.shape, *t.stride()))
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def current_stream(device=None):
     """Handle of torch's current HIP stream as a void*."""
+    if _raw_stream is not None and isinstance(device, torch.device) and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))      # no Stream object: this sits on every call
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
