@@ -199,6 +199,12 @@ class Encoding:
         return torch.empty((self.num_parameters(),), dtype=self.parameter_dtype(True), device=device)
 
     def set_parameter(self, tensor, gradients=False):
+        if not gradients:
+            # binding the same memory again changes nothing: skipped, this sits on every call of a network
+            key = None if tensor is None else (tensor.data_ptr(), tensor.numel(), tensor.dtype)
+            if key is not None and key == getattr(self, "_bound_inference", None):
+                return
+            self._bound_inference = key
         check(lib.qmlp_encoding_set_parameter(self._handle, desc(tensor),
                                               QMLP_GRADIENTS if gradients else QMLP_INFERENCE))
 
@@ -412,6 +418,7 @@ class Network:
         """Default (torch.nn.Linear style) initialization of the fp16 tensor 'dst'."""
         with self._mutex:
             check(lib.qmlp_network_set_parameter(self._handle, desc(dst), QMLP_INFERENCE))
+            self._bound_inference = (dst.data_ptr(), dst.numel(), dst.dtype)
             seed = int(torch.randint(2 ** 31 - 1, (1,)).item())
             check(lib.qmlp_network_initialize_inference_parameters(self._handle, seed))
 
@@ -450,7 +457,10 @@ class Network:
 
     def _set_network_parameters(self, network_parameters, encoding_parameters):
         if network_parameters is not None:
-            check(lib.qmlp_network_set_parameter(self._handle, desc(network_parameters), QMLP_INFERENCE))
+            key = (network_parameters.data_ptr(), network_parameters.numel(), network_parameters.dtype)
+            if key != getattr(self, "_bound_inference", None):
+                check(lib.qmlp_network_set_parameter(self._handle, desc(network_parameters), QMLP_INFERENCE))
+                self._bound_inference = key
         m = min(len(encoding_parameters), self.num_encodings())
         for i in range(m):
             p = encoding_parameters[i]
