@@ -11,10 +11,25 @@ from .classes import Activation, Encoding, Network, QuickMLP
 from ._lib import QmlpError, set_kernel_cache_dir, set_log_level
 
 
+_torch_classes = None
+
+
 def load_library():
-    """Kept for API compatibility: the native library is loaded when the package is imported."""
-    from . import _lib
-    return _lib.LIB_PATH
+    """Registers the torch custom classes ``torch.classes.qmlp_cu.{QuickMLP, Network, Encoding,
+    Activation, utils}`` (like ``load_library`` of the reference, src_py/qmlp/import_library.py:5-39)
+    and returns that namespace. The modules of this package do not need them (they call the C ABI
+    directly); scripted or traced modules that are to be saved with TorchScript do."""
+    global _torch_classes
+    if _torch_classes is None:
+        import os
+        import torch
+        from . import _lib
+        path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libqmlp_torch.so")
+        if not os.path.exists(path):
+            raise ImportError("%s has not been built: make -C quick-mlp_amd/csrc/torch (or __graft_entry__.build())" % path)
+        torch.classes.load_library(path)
+        _torch_classes = torch.classes.qmlp_cu
+    return _torch_classes
 
 
 __all__ = [
