@@ -31,10 +31,19 @@ class FusedActivation(torch.nn.Module):
             return torch.nn.Identity()
         raise ValueError("Unknown or user-specified activation")
 
-    def __init__(self, cfg: str):
+    def __init__(self, cfg: str, scriptable: bool = False):
+        """
+        :param scriptable: hold the torch custom class ``torch.classes.qmlp_cu.Activation`` instead
+            of the ctypes mirror, so that the module can be traced or scripted and saved with
+            TorchScript like the reference's module (same kernels and numbers either way)
+        """
         super().__init__()
         self._cfg = cfg
-        self._activation = Activation(cfg)
+        if scriptable:
+            from . import load_library
+            self._activation = load_library().Activation(cfg)
+        else:
+            self._activation = Activation(cfg)
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         """(batch, channels) half -> (batch, channels) half, with autograd support."""

@@ -16,16 +16,25 @@ class FusedEncoding(torch.nn.Module):
     Mirrors src_py/qmlp/encoding.py:9-123 of the reference.
     """
 
-    def __init__(self, cfg_or_impl):
+    def __init__(self, cfg_or_impl, scriptable: bool = False):
+        """
+        :param scriptable: with a JSON string, hold the torch custom class
+            ``torch.classes.qmlp_cu.Encoding`` instead of the ctypes mirror, so that the module can
+            be traced or scripted and saved with TorchScript like the reference's module
+        """
         super().__init__()
         if isinstance(cfg_or_impl, str):
             self._cfg = cfg_or_impl
-            self._encoding = Encoding(cfg_or_impl)
-        elif isinstance(cfg_or_impl, Encoding):
+            if scriptable:
+                from . import load_library
+                self._encoding = load_library().Encoding(cfg_or_impl)
+            else:
+                self._encoding = Encoding(cfg_or_impl)
+        elif isinstance(cfg_or_impl, Encoding) or isinstance(cfg_or_impl, torch.ScriptObject):
             self._cfg = cfg_or_impl.to_json()
             self._encoding = cfg_or_impl
         else:
-            raise TypeError("expected a json string or a qmlp.Encoding")
+            raise TypeError("expected a json string, a qmlp.Encoding or a torch.classes.qmlp_cu.Encoding")
         self._max_input_channel = self._encoding.max_input_channel()
         self._num_output_channels = self._encoding.num_output_channels()
         self._has_parameters = self._encoding.has_parameters()
@@ -44,7 +53,10 @@ class FusedEncoding(torch.nn.Module):
     def create_parameter_tensor(self, device="cuda") -> torch.Tensor:
         """A normally-distributed parameter tensor of the right size and dtype."""
         assert self.has_parameters()
-        t = self._encoding.create_inference_parameters(device)
+        if isinstance(self._encoding, Encoding):
+            t = self._encoding.create_inference_parameters(device)
+        else:
+            t = self._encoding.create_inference_parameters().to(device)
         tmp = torch.empty(t.shape, dtype=torch.float32, device=t.device)
         torch.nn.init.normal_(tmp)
         t.copy_(tmp)

@@ -17,22 +17,33 @@ class FusedNetwork(torch.nn.Module):
     (the reference passes an empty list), and the static size queries work.
     """
 
-    def __init__(self, cfg: str, parent: str = ".", weight_dtype=torch.float16, device="cuda"):
+    def __init__(self, cfg: str, parent: str = ".", weight_dtype=torch.float16, device="cuda", scriptable: bool = False):
         """
         :param cfg: the network specification as a JSON string
         :param parent: folder relative to which activation files named in the
             specification are resolved
         :param weight_dtype: dtype of the master weights (float32 for training with
             optimizers that cannot step fp16 tensors)
+        :param scriptable: hold the torch custom class ``torch.classes.qmlp_cu.Network`` instead of
+            the ctypes mirror, so that the module can be traced and saved with TorchScript like the
+            reference's module (same kernels and numbers either way)
         """
         super().__init__()
         self._cfg = cfg
         self._parent = parent
-        self._network = Network(cfg, parent)
+        self._scriptable = scriptable
+        if scriptable:
+            from . import load_library
+            self._network = load_library().Network(cfg, parent)
+        else:
+            self._network = Network(cfg, parent)
+        # plain integers: a traced forward() may not call integer methods of the custom class
+        self._channels_in = self._network.channels_in()
         self._num_output_channels = self._network.channels_out()
         self._num_layers = self._network.num_layers()
 
-        weights = self._network.create_inference_parameters(device)
+        weights = (self._network.create_inference_parameters().to(device) if scriptable
+                   else self._network.create_inference_parameters(device))
         self._network.initialize_inference_parameters(weights)
         self.weights = torch.nn.Parameter(weights.to(weight_dtype), requires_grad=True)
 
@@ -45,7 +56,7 @@ class FusedNetwork(torch.nn.Module):
             self._encodings.append(e)
             self._max_input_channel = max(self._max_input_channel, e.max_input_channel())
             if e.has_parameters():
-                p = e.create_inference_parameters(device)
+                p = e.create_inference_parameters().to(device) if scriptable else e.create_inference_parameters(device)
                 torch.zero_(p)
                 params.append(torch.nn.Parameter(p, requires_grad=True))
             else:
@@ -75,16 +86,16 @@ class FusedNetwork(torch.nn.Module):
         self._network.set_parallel_streams(v)
 
     def num_encodings(self) -> int:
-        return self._network.num_encodings()
+        return self._num_encodings
 
     def encoding(self, index: int) -> FusedEncoding:
         return FusedEncoding(self._encodings[index])
 
     def channels_in(self) -> int:
-        return self._network.channels_in()
+        return self._channels_in
 
     def channels_out(self) -> int:
-        return self._network.channels_out()
+        return self._num_output_channels
 
     def num_layers(self) -> int:
         return self._num_layers
@@ -112,6 +123,12 @@ class FusedNetwork(torch.nn.Module):
             warnings.warn("Training a network with 16-bit master weights: the gradient tensor is 16-bit as well, "
                           "which most optimizers cannot handle. Pass weight_dtype=torch.float32 to the constructor.")
         return self._network.forward(x, self.weights, list(self.encoding_parameters))
+
+    def __getstate__(self):
+        state = super().__getstate__() if hasattr(super(), "__getstate__") else self.__dict__.copy()
+        state = dict(state)
+        state["_encodings"] = None      # handles into the native network: taken again after unpickling
+        return state
 
     def __setstate__(self, state):
         # pickling rebuilds the native network from its specification; take the encodings from

@@ -180,3 +180,54 @@ def test_pullpush_class():
     gm, gd = Q.utils.pullpush_backward(mask, data.detach(), torch.ones_like(out))
     assert torch.equal(data.grad, gd) and gm.shape == mask.shape
     assert torch.equal(Q.utils.pullpush_forward(mask, data.detach()), out.detach())
+
+
+@pytest.mark.gpu
+def test_scriptable_modules_trace_save_and_load(tmp_path):
+    """FusedActivation / FusedEncoding / FusedNetwork with scriptable=True hold the torch custom
+    classes: torch.jit.trace -> freeze -> save -> load as in the reference's module tests, and the
+    same numbers as the default modules."""
+    _gpu_or_skip()
+    g = torch.Generator(device="cuda").manual_seed(3)
+
+    act = qmlp.FusedActivation("sine", scriptable=True).eval()
+    x = torch.randn((5, 3), device="cuda", generator=g, dtype=torch.float16)
+    traced = torch.jit.freeze(torch.jit.trace(act, (x,)))
+    torch.jit.save(traced, str(tmp_path / "act.pt"))
+    assert torch.equal(torch.jit.load(str(tmp_path / "act.pt"))(x), qmlp.FusedActivation("sine")(x))
+
+    enc = qmlp.FusedEncoding(GRID_CFG, scriptable=True).eval()
+    table = enc.create_parameter_tensor()
+    pos = torch.rand((64, 2), device="cuda", generator=g) * 1.8 - 0.9
+    traced = torch.jit.freeze(torch.jit.trace(enc, (pos, table)))
+    torch.jit.save(traced, str(tmp_path / "enc.pt"))
+    assert torch.equal(torch.jit.load(str(tmp_path / "enc.pt"))(pos, table), qmlp.FusedEncoding(GRID_CFG)(pos, table))
+
+    torch.manual_seed(0)
+    net = qmlp.FusedNetwork(NETWORK_CFG, weight_dtype=torch.float32, scriptable=True)
+    plain = qmlp.FusedNetwork(NETWORK_CFG, weight_dtype=torch.float32)
+    plain.load_state_dict(net.state_dict())
+    xin = torch.randn((500, 16), device="cuda", generator=g)
+    adj = torch.randn((500, 16), device="cuda", generator=g)
+    outs = []
+    for module in (net, plain):
+        xi = xin.clone().requires_grad_(True)
+        y = module(xi)
+        y.backward(adj)
+        outs.append((y.detach(), xi.grad, module.weights.grad.clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    net.eval()
+    with torch.no_grad():
+        traced = torch.jit.trace(net, (xin,))
+    torch.jit.save(traced, str(tmp_path / "net.pt"))
+    loaded = torch.jit.load(str(tmp_path / "net.pt"))
+    with torch.no_grad():
+        assert torch.equal(loaded(xin), outs[1][0])
+    # pickling and deepcopy of the module that holds the custom class
+    import copy
+    import pickle
+    for clone in (copy.deepcopy(net), pickle.loads(pickle.dumps(net))):
+        with torch.no_grad():
+            assert torch.equal(clone(xin), outs[1][0])
+        assert clone.encoding(0).num_output_channels() == 16
