@@ -31,7 +31,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 # 256 MiB device copy of --copy-calibration: x2.000 and x1.000 on MI355X). The summary
 # with the commands is kept under profiles/. Workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2-inference": {"points": 1 << 20, "fetch": 355535.7 * 1024 * 2.0, "write": 30209.1 * 1024 * 1.0},
+    "cfg2-inference": {"points": 1 << 20, "fetch": 106149.0 * 1024 * 2.0, "write": 8192.0 * 1024 * 1.0},
 }
 
 WORKLOADS = {

@@ -49,6 +49,11 @@ public:
         //together (level by level for grid encodings). If <=0, the library chooses.
         int pointsPerLane = -1;
 
+        // If true (default), networks with grid encodings and at most 32 encoded channels get a
+        // kernel shape whose encoded rows wait in registers instead of LDS: a wavefront then
+        // takes 8 tiles at once, and 2^20 points are one sweep over the level tables.
+        bool registerStaging = true;
+
         // Accepted for compatibility; the LDS layouts of this implementation are
         // bank-conflict free for 64 lanes by construction and need no skew.
         bool skewSharedMemory = false;
@@ -98,7 +103,7 @@ private:
         int fullGrid = 0;
     };
     // [store intermediates][variant], see ForwardVariant
-    std::optional<CompiledKernel> forwardKernels_[2][3];
+    std::optional<CompiledKernel> forwardKernels_[2][4];
 
     struct AdjointLayerInfo
     {
@@ -236,8 +241,14 @@ private:
     // encodings on batches that still fill the device that way (fewer sweeps over the level
     // tables); DEFAULT: 4 wavefronts, 2 tiles each with grid encodings; NARROW: one tile per
     // wavefront for small batches.
-    enum ForwardVariant { VARIANT_DEFAULT = 0, VARIANT_NARROW = 1, VARIANT_LARGE = 2 };
+    // REGISTERS: 8 wavefronts whose encoded rows wait in registers (up to 8 tiles each) and pass
+    // through one LDS staging tile per wavefront: one sweep over the level tables per 2^20 points.
+    enum ForwardVariant { VARIANT_DEFAULT = 0, VARIANT_NARROW = 1, VARIANT_LARGE = 2, VARIANT_REGISTERS = 3 };
     bool hasLargeVariant(bool store) const;
+    /** Tiles per wavefront of the REGISTERS shape, 0 if the network has none. */
+    int registerVariantTiles(bool store) const;
+    /** Workgroup size and tiles per wavefront of a shape of the forward kernel. */
+    void forwardShape(bool store, int variant, int& blockSize, int& pointsPerLane) const;
     void compileForwardKernel(bool store, int variant, bool compileOnly = false);
     const CompiledKernel& forwardKernelFor(bool store, int numTiles);
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
@@ -246,7 +257,7 @@ private:
     void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 
-    std::string forwardSource(int blockSize, int pointsPerLane) const;
+    std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false) const;
     std::string backwardSource(int flags, int blockSize) const;
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const;

@@ -91,6 +91,16 @@ public:
      */
     [[nodiscard]] virtual int numSweptTables() const { return 0; }
 
+    /**
+     * 32-bit registers that the gathers of one point from one table occupy while they are in
+     * flight (all corners of a cell); 0 for encodings that gather nothing. The fused forward
+     * kernel keeps the gathers of several points per lane in flight and sizes that number by it.
+     */
+    [[nodiscard]] virtual int gatherRegistersPerPoint() const { return 0; }
+
+    /** Output channels that the device code writes together (the features of a grid entry). */
+    [[nodiscard]] virtual int channelsWrittenTogether() const { return 1; }
+
     [[nodiscard]] virtual int ldsGradientFloats(int maxBytes, int& levels) const
     {
         levels = 0;

@@ -75,6 +75,75 @@ struct StageRowArray
     }
 };
 
+/**
+ * Encoded rows of PPL points of a lane that wait in registers, two halves per 32-bit register,
+ * one register vector per point. The point index has to be a compile-time constant once the
+ * loops over the points are unrolled; the register of a point may be selected by a value that
+ * is uniform over the wavefront (a level counter): that is one indexed register move.
+ */
+template <typename T, int PPL, int C>
+struct PackedRegisterRows
+{
+    static_assert(sizeof(T) == 2, "two values per register");
+    typedef unsigned int Vector __attribute__((ext_vector_type(C / 2)));
+    Vector data_[PPL];
+};
+
+/** The rows of PackedRegisterRows from channel OFFSET on: rows[q][i] = value. */
+template <typename T, int PPL, int C, int OFFSET>
+struct PackedRegisterRowsView
+{
+    typedef T ValueType;
+    typedef PackedRegisterRows<T, PPL, C> Rows;
+    struct Element
+    {
+        typename Rows::Vector& vector_;
+        int channel_;
+        __device__ __forceinline__ void operator=(T v) const
+        {
+            const unsigned int bits = __builtin_bit_cast(unsigned short, v);
+            const unsigned int old = vector_[channel_ >> 1];
+            vector_[channel_ >> 1] = (channel_ & 1) ? ((old & 0xffffu) | (bits << 16)) : ((old & 0xffff0000u) | bits);
+        }
+    };
+    struct Row
+    {
+        typedef T ValueType;
+        Rows& rows_;
+        int q_;
+        __device__ __forceinline__ Element operator[](int i) const { return Element{rows_.data_[q_], i + OFFSET}; }
+    };
+    Rows& rows_;
+    __device__ __forceinline__ Row operator[](int q) const { return Row{rows_, q}; }
+};
+
+/** rows[q][i] = a, rows[q][i + 1] = b for an even channel i. */
+template <typename Rows, typename T>
+__device__ __forceinline__ void storePair(Rows& rows, int q, int i, T a, T b)
+{
+    rows[q][i] = a;
+    rows[q][i + 1] = b;
+}
+template <typename T, int PPL, int C, int OFFSET>
+__device__ __forceinline__ void storePair(PackedRegisterRowsView<T, PPL, C, OFFSET>& rows, int q, int i, T a, T b)
+{
+    static_assert(OFFSET % 2 == 0, "pairs start at even channels");
+    const unsigned int lo = __builtin_bit_cast(unsigned short, a), hi = __builtin_bit_cast(unsigned short, b);
+    rows.rows_.data_[q][(i + OFFSET) >> 1] = lo | (hi << 16);
+}
+
+/** Element type of a set of output rows: a C array of row views, or PackedRegisterRowsView. */
+template <typename Rows>
+struct RowsValueType
+{
+    typedef typename Rows::ValueType Type;
+};
+template <typename Row, int N>
+struct RowsValueType<Row[N]>
+{
+    typedef typename Row::ValueType Type;
+};
+
 /** Strided global row. */
 template <typename T>
 struct StridedArray

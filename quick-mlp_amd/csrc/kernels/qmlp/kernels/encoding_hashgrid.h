@@ -278,11 +278,10 @@ struct EncodingHashGrid
      * any starts level l+1, so that the workgroups of the device sweep through the level
      * tables together and a level's table stays in L2 while it is in use.
      */
-    template <int PPL, typename I, typename O>
-    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], O (&outputs)[PPL],
-                                                        const param_t& params)
+    template <int PPL, typename I, typename Os>
+    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], Os& outputs, const param_t& params)
     {
-        typedef typename O::ValueType O_t;
+        typedef typename RowsValueType<Os>::Type O_t;
         float pos[PPL][D];
 #pragma unroll
         for (int q = 0; q < PPL; ++q) unitPosition(inputs[q], params, pos[q]);
@@ -298,7 +297,11 @@ struct EncodingHashGrid
             for (int q = 0; q < PPL; ++q) gatherLevel(l, pos[q], params.parametersForward, feat[q]);
 #pragma unroll
             for (int q = 0; q < PPL; ++q) {
-                if constexpr (Cfg::Concat) {
+                if constexpr (Cfg::Concat && F % 2 == 0) {
+#pragma unroll
+                    for (int i = 0; i < F; i += 2)
+                        storePair(outputs, q, l * F + i, fcast<O_t>(feat[q][i]), fcast<O_t>(feat[q][i + 1]));
+                } else if constexpr (Cfg::Concat) {
 #pragma unroll
                     for (int i = 0; i < F; ++i) outputs[q][l * F + i] = fcast<O_t>(feat[q][i]);
                 } else {

@@ -20,11 +20,14 @@ struct EncodingIdentity
         for (int i = 0; i < NumChannels; ++i) output[i] = fcast<O_t>(input[i + StartChannel]);
     }
 
-    template <int PPL, typename I, typename O>
-    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], O (&outputs)[PPL])
+    template <int PPL, typename I, typename Os>
+    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], Os& outputs)
     {
 #pragma unroll
-        for (int q = 0; q < PPL; ++q) forward(inputs[q], outputs[q]);
+        for (int q = 0; q < PPL; ++q) {
+            auto row = outputs[q];
+            forward(inputs[q], row);
+        }
     }
 
     template <bool EvaluateInputGradients, bool EvaluateParameterGradients, typename I, typename O, typename AdjI>

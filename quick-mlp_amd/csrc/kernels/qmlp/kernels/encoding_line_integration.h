@@ -130,12 +130,14 @@ struct EncodingLineIntegration
         for (int i = 0; i < NumOutputs; ++i) output[i] = fcast<O_t>(accu[i]);
     }
 
-    template <int PPL, typename I, typename O>
-    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], O (&outputs)[PPL],
-                                                        const param_t& params)
+    template <int PPL, typename I, typename Os>
+    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], Os& outputs, const param_t& params)
     {
 #pragma unroll 1
-        for (int q = 0; q < PPL; ++q) forward(inputs[q], outputs[q], params);
+        for (int q = 0; q < PPL; ++q) {
+            auto row = outputs[q];
+            forward(inputs[q], row, params);
+        }
     }
 
     template <bool EvaluateInputGradients, bool EvaluateParameterGradients, typename I, typename O, typename AdjI>

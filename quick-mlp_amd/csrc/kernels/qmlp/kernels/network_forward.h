@@ -25,6 +25,19 @@ namespace activations
 $$DEFINE_ACTIVATIONS$$
 }
 
+/** Points the staging rows of the PPL points of a lane at the wave's LDS staging tiles. */
+template <typename T, int C, int PPL>
+__device__ __forceinline__ void bindEncodingRow(StageRowArray<T, C> (&rows)[PPL], T* stage, int q, int lane)
+{
+    rows[q].row_ = stage + (q * TILE_POINTS + stageRow(lane)) * StageLayout<C>::Stride;
+    rows[q].rotation_ = StageLayout<C>::rotation(stageRow(lane));
+    rows[q].offset_ = 0;
+}
+template <typename T, int PPL, int C, int OFFSET>
+__device__ __forceinline__ void bindEncodingRow(PackedRegisterRowsView<T, PPL, C, OFFSET>&, T*, int, int)
+{
+}
+
 /**
  * \tparam STORE false: inference. true: additionally stores, per 64-point tile and
  *   channel-major, the encoded network input and the pre-activations of every layer
@@ -52,6 +65,11 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     constexpr int LDS_PARAM_HALVES = $$LDS_PARAM_HALVES$$;
     constexpr int WAVES = $$BLOCK_SIZE$$ / WAVE_SIZE;
     constexpr int PPL = $$POINTS_PER_LANE$$;              // tiles a wave encodes together
+    // true: the encoded rows of the PPL tiles wait in registers and go through one LDS staging
+    // tile per wave, one after the other (the register file holds more points than the LDS);
+    // false: every tile has its own staging rows in LDS
+    constexpr bool REGISTER_STAGING = $$REGISTER_STAGING$$;
+    constexpr int STAGED_TILES = REGISTER_STAGING ? 1 : PPL;
     // Some layers' weights are staged into a shared LDS buffer right before the layer runs:
     // the wavefronts of the workgroup then walk the tiles and layers in lockstep (workgroup
     // barriers inside the loops), wavefronts without a tile compute on zero rows.
@@ -65,7 +83,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     const int wave = threadIdx.x / WAVE_SIZE;
     const int lane = threadIdx.x % WAVE_SIZE;
     const int g = lane >> 4, r = lane & 15;
-    f16* sStage = sParams + LDS_PARAM_HALVES + wave * (PPL * TILE_POINTS * STAGE_STRIDE);
+    f16* sStage = sParams + LDS_PARAM_HALVES + wave * (STAGED_TILES * TILE_POINTS * STAGE_STRIDE);
 
     // stage the weights in operand order, then the biases
 $$STAGE_PARAMETERS$$
@@ -83,17 +101,17 @@ $$STAGE_PARAMETERS$$
         // encodings: PPL points per lane (one of each tile), each into its staging row.
         // Rows outside the batch are evaluated at the origin and zeroed afterwards so that
         // no NaN enters the matrix cores.
+        PackedRegisterRows<f16, REGISTER_STAGING ? PPL : 1, CHANNELS_IN> encodedRegisters;
+        (void)encodedRegisters;
         {
             StaticArray<float, NUM_INPUTS> encodingInput[PPL];
-            StageRowArray<f16, CHANNELS_IN> encodingOutput[PPL];
+            $$ENCODING_OUTPUT_ROWS$$
             bool valid[PPL];
 #pragma unroll
             for (int q = 0; q < PPL; ++q) {
                 const int index = (tile0 + q) * TILE_POINTS + lane;
                 valid[q] = index < numel;
-                encodingOutput[q].row_ = sStage + (q * TILE_POINTS + stageRow(lane)) * STAGE_STRIDE;
-                encodingOutput[q].rotation_ = Stage::rotation(stageRow(lane));
-                encodingOutput[q].offset_ = 0;
+                bindEncodingRow(encodingOutput, sStage, q, lane);
 #pragma unroll
                 for (int i = 0; i < NUM_INPUTS; ++i)
                     encodingInput[q][i] = valid[q] ? inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
@@ -113,7 +131,7 @@ $$CALL_ENCODINGS$$
         }
         waveLdsSync();
 
-#pragma unroll 1
+$$TILE_LOOP_PRAGMA$$
         for (int q = 0; q < PPL; ++q)
         {
         const int tile = tile0 + q;
@@ -121,7 +139,19 @@ $$CALL_ENCODINGS$$
         const bool tileValid = tile < numTiles;
         const int tmpTile = tile + tmpTileOffset;
         (void)tmpTile;
-        const f16* sTile = sStage + q * (TILE_POINTS * STAGE_STRIDE);
+        const f16* sTile = sStage + (REGISTER_STAGING ? 0 : q) * (TILE_POINTS * STAGE_STRIDE);
+        if (REGISTER_STAGING) {
+            // the lane's row of this tile: registers -> staging row, 8 bytes at a time
+            if (q > 0) waveLdsSync();   // the operands of the previous tile have been read
+#pragma unroll
+            for (int chunk = 0; chunk < CHANNELS_IN / 4; ++chunk) {
+                typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+                const u32x2 v = {encodedRegisters.data_[REGISTER_STAGING ? q : 0][2 * chunk],
+                                 encodedRegisters.data_[REGISTER_STAGING ? q : 0][2 * chunk + 1]};
+                *reinterpret_cast<u32x2*>(sStage + Stage::chunkOffset(stageRow(lane), chunk)) = v;
+            }
+            waveLdsSync();
+        }
 
         // B operands of the first layer
         f16x4 x0[NT][KT0];

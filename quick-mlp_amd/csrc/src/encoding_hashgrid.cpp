@@ -204,6 +204,12 @@ Tensor::Precision EncodingHashGrid::parameterPrecision(Tensor::Usage usage) cons
 
 int EncodingHashGrid::parameterCount() const { return numParameters_; }
 
+int EncodingHashGrid::gatherRegistersPerPoint() const
+{
+    const int entryBytes = numFeaturesPerLevel_ * (parameterPrecision_ == Tensor::HALF ? 2 : 4);
+    return std::max(1, ((1 << dimension_) * entryBytes + 3) / 4);
+}
+
 int EncodingHashGrid::ldsGradientFloats(int maxBytes, int& levels) const
 {
     levels = 0;

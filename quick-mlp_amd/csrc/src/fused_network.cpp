@@ -71,6 +71,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         compileOptions_.pointsPerLane = options.value("points_per_lane", compileOptions_.pointsPerLane);
         if (compileOptions_.pointsPerLane > 8)
             throw configuration_error("points_per_lane must be at most 8, but is %d", compileOptions_.pointsPerLane);
+        compileOptions_.registerStaging = options.value("register_staging", compileOptions_.registerStaging);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
             options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
@@ -575,13 +576,16 @@ static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
     return ss.str();
 }
 
-std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
+std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool registerStaging) const
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string code = kl->findFile("qmlp/kernels/network_forward.h").value();
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
     replaceAll(code, "$$POINTS_PER_LANE$$", std::to_string(pointsPerLane));
+    replaceAll(code, "$$REGISTER_STAGING$$", registerStaging ? "true" : "false");
+    // rows in registers are indexed by the tile: that loop has to be unrolled
+    replaceAll(code, "$$TILE_LOOP_PRAGMA$$", registerStaging ? "#pragma unroll" : "#pragma unroll 1");
     std::vector<int> ldsW, ldsB;
     int streamOffset = -1;
     replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(false, ldsW, ldsB, &streamOffset)));
@@ -610,12 +614,19 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane) const
 
     std::stringstream callEncodings;
     int encodingOffset = 0;
+    replaceAll(code, "$$ENCODING_OUTPUT_ROWS$$",
+               registerStaging ? "PackedRegisterRowsView<f16, PPL, CHANNELS_IN, 0> encodingOutput{encodedRegisters};"
+                               : "StageRowArray<f16, CHANNELS_IN> encodingOutput[PPL];");
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
-        callEncodings << "            {\n                StageRowArray<f16, CHANNELS_IN> encodingOutputK[PPL];\n"
-                      << "#pragma unroll\n                for (int q = 0; q < PPL; ++q) encodingOutputK[q] = encodingOutput[q] + "
-                      << encodingOffset << ";\n                " << e->qualifiedName()
-                      << "::template forwardBatch<PPL>(encodingInput, encodingOutputK";
+        if (registerStaging)
+            callEncodings << "            {\n                PackedRegisterRowsView<f16, PPL, CHANNELS_IN, " << encodingOffset
+                          << "> encodingOutputK{encodedRegisters};\n                ";
+        else
+            callEncodings << "            {\n                StageRowArray<f16, CHANNELS_IN> encodingOutputK[PPL];\n"
+                          << "#pragma unroll\n                for (int q = 0; q < PPL; ++q) encodingOutputK[q] = encodingOutput[q] + "
+                          << encodingOffset << ";\n                ";
+        callEncodings << e->qualifiedName() << "::template forwardBatch<PPL>(encodingInput, encodingOutputK";
         if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
         callEncodings << ");\n            }\n";
         encodingOffset += e->numOutputChannels();
@@ -854,25 +865,69 @@ bool FusedNetwork::hasLargeVariant(bool store) const
     return gathers && lds <= MaxSharedMemoryBytes();
 }
 
+int FusedNetwork::registerVariantTiles(bool store) const
+{
+    const int overwrite = store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference;
+    if (overwrite > 0 || compileOptions_.pointsPerLane > 0 || !compileOptions_.registerStaging) return 0;
+    bool gathers = false;
+    int channelOffset = 0;
+    for (const auto& e : encodings_) {
+        const int offset = channelOffset;
+        channelOffset += e->numOutputChannels();
+        gathers = gathers || e->hasParameters();
+        if (!e->hasParameters()) continue;
+        // a register holds two channels: the features of a level have to fill whole registers
+        if (offset % 2 != 0 || e->channelsWrittenTogether() % 2 != 0) return 0;
+        // The shape pays through fewer sweeps over the tables of a multi-level grid (only
+        // grids write their rows with indices that resolve to registers). The gathers of
+        // all 8 points of a lane are in flight together: beyond 64 registers for them the
+        // compiler spills (a dense 4-D grid with 8 features: 1.5 KB of scratch per lane and
+        // 1.9 times the time of the LDS shape).
+        if (e->numSweptTables() < 2 || 8 * e->gatherRegistersPerPoint() > 64) return 0;
+    }
+    if (!gathers) return 0;
+    // a wavefront of a workgroup of 8 has 256 registers: half of them hold encoded rows (two
+    // channels per register), the layers need the rest
+    int widest = 0;
+    for (const auto& l : layers_) widest = std::max(widest, std::max(l.channelsIn, l.channelsOut));
+    if (widest > 64) return 0;
+    for (int p : weightPlacement(false))
+        if (p != WEIGHTS_RESIDENT) return 0;
+    const int tiles = std::min(8, 256 / layers_[0].channelsIn);
+    const int lds = ldsParamHalves(false) * static_cast<int>(sizeof(half)) + 8 * stageBytesPerWave(false);
+    if (tiles < 8 || lds > MaxSharedMemoryBytes()) return 0;
+    return tiles;
+}
+
+void FusedNetwork::forwardShape(bool store, int variant, int& blockSize, int& pointsPerLane) const
+{
+    // the narrow shape is sized like a network with one tile per wave (smaller workgroups when
+    // the weights allow it: a small batch then spreads over more compute units)
+    blockSize = forwardBlockSize(store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference,
+                                 false, &pointsPerLane, variant == VARIANT_NARROW ? 1 : 0);
+    if (variant == VARIANT_LARGE) {
+        blockSize = 2 * DEFAULT_BLOCK_SIZE;
+        pointsPerLane = 4;
+    }
+    if (variant == VARIANT_REGISTERS) {
+        blockSize = 2 * DEFAULT_BLOCK_SIZE;
+        pointsPerLane = registerVariantTiles(store);
+    }
+}
+
 void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnly)
 {
     auto& slot = forwardKernels_[store ? 1 : 0][variant];
     if (slot.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
-    // the narrow shape is sized like a network with one tile per wave (smaller workgroups when
-    // the weights allow it: a small batch then spreads over more compute units)
-    ck.blockSize = forwardBlockSize(store ? compileOptions_.overwriteBlocksizeForward : compileOptions_.overwriteBlocksizeInference,
-                                    false, &ck.pointsPerLane, variant == VARIANT_NARROW ? 1 : 0);
-    if (variant == VARIANT_LARGE) {
-        ck.blockSize = 2 * DEFAULT_BLOCK_SIZE;
-        ck.pointsPerLane = 4;
-    }
+    forwardShape(store, variant, ck.blockSize, ck.pointsPerLane);
+    const bool registerStaging = variant == VARIANT_REGISTERS;
     ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
-        + (ck.blockSize / WARP_SIZE) * ck.pointsPerLane * stageBytesPerWave(false);
+        + (ck.blockSize / WARP_SIZE) * (registerStaging ? 1 : ck.pointsPerLane) * stageBytesPerWave(false);
     ck.fun = kl->getKernel(store ? "qmlp::kernel::NetworkKernelInferenceAndForward<true>"
                                  : "qmlp::kernel::NetworkKernelInferenceAndForward<false>",
-                           forwardSource(ck.blockSize, ck.pointsPerLane), loaderFlags(compileOnly)).value();
+                           forwardSource(ck.blockSize, ck.pointsPerLane, registerStaging), loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
     QuickMLP::Instance().getLogger()->debug(
@@ -885,31 +940,40 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
 const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles)
 {
     const int s = store ? 1 : 0;
-    compileForwardKernel(store, VARIANT_DEFAULT);
-    const auto& wide = forwardKernels_[s][VARIANT_DEFAULT].value();
-    if (wide.pointsPerLane == 1) return wide;   // no gathers, or a pinned shape: one kernel
+    {
+        int blockSize = 0, pointsPerLane = 1;
+        forwardShape(store, VARIANT_DEFAULT, blockSize, pointsPerLane);
+        if (pointsPerLane == 1) {   // no gathers, or a pinned shape: one kernel
+            compileForwardKernel(store, VARIANT_DEFAULT);
+            return forwardKernels_[s][VARIANT_DEFAULT].value();
+        }
+    }
     // Kernels that take more tiles per wave are faster per point, but the time grows in steps
     // of one workgroup per compute unit, whether all compute units have one or not. Measured on
     // a 16-level hash grid, per step: 4 waves x 1 tile 26 us (2^16 points), 8 waves x 2 tiles
     // 82 us (2^18 points), 8 waves x 4 tiles 153 us (2^19 points). Take the shape with the
     // least estimated time = steps x points per step x relative cost per point.
-    const CompiledKernel* best = nullptr;
+    // Only the shape that wins is compiled.
+    int best = -1;
     double bestCost = 0;
     const int computeUnits = KernelFunction::computeUnits();
     auto consider = [&](int variant, double costPerPoint) {
-        compileForwardKernel(store, variant);
-        const auto& k = forwardKernels_[s][variant].value();
-        const long long stepTiles = static_cast<long long>(computeUnits) * (k.blockSize / WARP_SIZE) * k.pointsPerLane;
+        int blockSize = 0, pointsPerLane = 1;
+        forwardShape(store, variant, blockSize, pointsPerLane);
+        const long long stepTiles = static_cast<long long>(computeUnits) * (blockSize / WARP_SIZE) * pointsPerLane;
         const double cost = static_cast<double>(divUp<long long>(numTiles, stepTiles)) * stepTiles * costPerPoint;
-        if (!best || cost < bestCost) {
-            best = &k;
+        if (best < 0 || cost < bestCost) {
+            best = variant;
             bestCost = cost;
         }
     };
+    // measured 258 ps per point against 288 for 8 waves x 4 tiles (16-level hash grid, 2^20 points)
+    if (registerVariantTiles(store) > 0) consider(VARIANT_REGISTERS, 0.9);
     if (hasLargeVariant(store)) consider(VARIANT_LARGE, 1.0);
     consider(VARIANT_DEFAULT, 1.075);
     consider(VARIANT_NARROW, 1.39);
-    return *best;
+    compileForwardKernel(store, best);
+    return forwardKernels_[s][best].value();
 }
 
 void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
@@ -980,6 +1044,7 @@ void FusedNetwork::precompile(int adjointFlags)
         forwardBlockSize(-1, false, &ppl);
         if (ppl > 1) compileForwardKernel(store, VARIANT_NARROW, true);
         if (hasLargeVariant(store)) compileForwardKernel(store, VARIANT_LARGE, true);
+        if (registerVariantTiles(store) > 0) compileForwardKernel(store, VARIANT_REGISTERS, true);
     }
     if (adjointFlags > 0) compileBackwardKernel(adjointFlags, true);
 }

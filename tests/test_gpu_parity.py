@@ -3,6 +3,8 @@ oracle on the same seeded inputs. Shapes follow the reference's own tests
 (tests_cpp/test_against_eigen1.cpp:26-61, test_against_eigen2.cpp:17-28,
 tests_py/qmlp_tests/test_network_base.py:87-256). Tolerance of every floating point
 comparison: rel 1e-2 / abs 1e-3 against the fp32 oracle, no entry may exceed it."""
+import json
+
 import numpy as np
 import pytest
 import torch
@@ -664,3 +666,36 @@ def test_grid_network_batches_that_take_several_launches():
     t = a["table_grads"][0]
     assert_close(b["table_grads"][0] + c["table_grads"][0], t, "additivity of the grid gradients", rel=1e-3,
                  abs_=1e-4 * float(np.abs(t).max()))
+
+
+def test_rows_staged_in_registers_give_the_same_bits_as_rows_staged_in_lds():
+    """A multi-level grid with at most 32 encoded channels gets a kernel shape whose encoded rows
+    wait in registers (8 tiles per wavefront). It has to agree bit for bit with the shapes that
+    stage in LDS (``register_staging: false``): inference, the forward pass whose intermediates
+    feed the backward pass, on one pass and on two passes of the resident workgroups, ragged."""
+    c = bc.CONFIGS[3]
+    cases = []
+    for on in (True, False):
+        cfg = json.loads(json.dumps(c["cfg"]))
+        cfg.setdefault("options", {})["register_staging"] = on
+        rng = np.random.default_rng(5)
+        case = Case(cfg, bc.ORACLE_ACTIVATIONS)
+        case.set_parameters(bc.make_parameters(3, rng).astype(np.float32))
+        case.set_table(0, bc.make_table(3, case.oracle.encodings[0][1].n_params, rng, 1.0))
+        cases.append(case)
+    reg, lds = cases
+    rng = np.random.default_rng(6)
+    for N in ((1 << 20) - 37, (1 << 21) - 64 * 700 - 5):
+        print("register staging: %d points" % N, flush=True)
+        X = bc.make_inputs(3, N, rng)
+        a = reg.gpu_inference(X)
+        b = lds.gpu_inference(X)
+        assert np.abs(a).max() > 0.1 and np.array_equal(a, b)
+    N = (1 << 20) - 37
+    adj = rng.uniform(-1, 1, (N, 1)).astype(np.float32)
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    ga, gb = reg.gpu_train(X[:N], adj, flags), lds.gpu_train(X[:N], adj, flags)
+    for key in ("out", "adj_x", "grads"):
+        assert np.array_equal(ga[key], gb[key]), key
+    t = gb["table_grads"][0]
+    assert_close(ga["table_grads"][0], t, "grid gradients (atomics)", rel=1e-3, abs_=1e-4 * float(np.abs(t).max()))
