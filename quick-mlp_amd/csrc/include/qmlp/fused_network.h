@@ -104,6 +104,8 @@ private:
     };
     // [store intermediates][variant], see ForwardVariant
     std::optional<CompiledKernel> forwardKernels_[2][4];
+    // set once the compiled REGISTERS shape turned out to spill heavily: it is not used then
+    bool registerShapeSpills_[2] = {false, false};
 
     struct AdjointLayerInfo
     {

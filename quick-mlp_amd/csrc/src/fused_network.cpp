@@ -19,6 +19,7 @@ constexpr int TILE_POINTS = 64;          // points per wavefront tile
 constexpr int DEFAULT_BLOCK_SIZE = 256;  // 4 wavefronts
 constexpr int MAX_WEIGHT_UPDATE_SLICES = 512;  // batch slices with partial weight gradients
 constexpr int STAGE_PAD = 8;             // halves of padding per staging row
+constexpr int MAX_REGISTER_SHAPE_SCRATCH = 512;   // bytes per lane, see forwardKernelFor
 
 int gfx950LdsBytes() { return 160 * 1024; }
 } // namespace
@@ -880,10 +881,11 @@ int FusedNetwork::registerVariantTiles(bool store) const
         if (offset % 2 != 0 || e->channelsWrittenTogether() % 2 != 0) return 0;
         // The shape pays through fewer sweeps over the tables of a multi-level grid (only
         // grids write their rows with indices that resolve to registers). The gathers of
-        // all 8 points of a lane are in flight together: beyond 64 registers for them the
-        // compiler spills (a dense 4-D grid with 8 features: 1.5 KB of scratch per lane and
-        // 1.9 times the time of the LDS shape).
-        if (e->numSweptTables() < 2 || 8 * e->gatherRegistersPerPoint() > 64) return 0;
+        // all 8 points of a lane are in flight together: far beyond 64 registers for them
+        // the compiler spills (fp32 entries, 128 registers: 32 spilled registers and 18 %
+        // faster than the LDS shape; a dense 4-D grid with 8 features, 512 registers: 1.5 KB
+        // of scratch per lane and 1.9 times the time of the LDS shape).
+        if (e->numSweptTables() < 2 || 8 * e->gatherRegistersPerPoint() > 128) return 0;
     }
     if (!gathers) return 0;
     // a wavefront of a workgroup of 8 has 256 registers: half of them hold encoded rows (two
@@ -968,11 +970,19 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
         }
     };
     // measured 258 ps per point against 288 for 8 waves x 4 tiles (16-level hash grid, 2^20 points)
-    if (registerVariantTiles(store) > 0) consider(VARIANT_REGISTERS, 0.9);
+    if (registerVariantTiles(store) > 0 && !registerShapeSpills_[s]) consider(VARIANT_REGISTERS, 0.9);
     if (hasLargeVariant(store)) consider(VARIANT_LARGE, 1.0);
     consider(VARIANT_DEFAULT, 1.075);
     consider(VARIANT_NARROW, 1.39);
     compileForwardKernel(store, best);
+    if (best == VARIANT_REGISTERS && forwardKernels_[s][best].value().fun.scratchBytes() > MAX_REGISTER_SHAPE_SCRATCH) {
+        // the compiler did not get the rows and the gathers into the registers: a kernel that
+        // spills this much is slower than the shapes that stage in LDS
+        QuickMLP::Instance().getLogger()->debug("the forward kernel with rows in registers spills %d bytes per lane, not used",
+                                                forwardKernels_[s][best].value().fun.scratchBytes());
+        registerShapeSpills_[s] = true;
+        return forwardKernelFor(store, numTiles);
+    }
     return forwardKernels_[s][best].value();
 }
 

@@ -668,7 +668,8 @@ def test_grid_network_batches_that_take_several_launches():
                  abs_=1e-4 * float(np.abs(t).max()))
 
 
-def test_rows_staged_in_registers_give_the_same_bits_as_rows_staged_in_lds():
+@pytest.mark.parametrize("precision", ["half", "float"])
+def test_rows_staged_in_registers_give_the_same_bits_as_rows_staged_in_lds(precision):
     """A multi-level grid with at most 32 encoded channels gets a kernel shape whose encoded rows
     wait in registers (8 tiles per wavefront). It has to agree bit for bit with the shapes that
     stage in LDS (``register_staging: false``): inference, the forward pass whose intermediates
@@ -678,6 +679,7 @@ def test_rows_staged_in_registers_give_the_same_bits_as_rows_staged_in_lds():
     for on in (True, False):
         cfg = json.loads(json.dumps(c["cfg"]))
         cfg.setdefault("options", {})["register_staging"] = on
+        cfg["encodings"][0]["parameter_precision"] = precision
         rng = np.random.default_rng(5)
         case = Case(cfg, bc.ORACLE_ACTIVATIONS)
         case.set_parameters(bc.make_parameters(3, rng).astype(np.float32))
