@@ -252,7 +252,12 @@ private:
     /** Workgroup size and tiles per wavefront of a shape of the forward kernel. */
     void forwardShape(bool store, int variant, int& blockSize, int& pointsPerLane) const;
     void compileForwardKernel(bool store, int variant, bool compileOnly = false);
-    const CompiledKernel& forwardKernelFor(bool store, int numTiles);
+    /**
+     * The kernel shape for the next launch over a batch of numTiles tiles and, in launchTiles,
+     * how many of them that launch should take (whole steps of a large shape first; the caller
+     * asks again for the rest).
+     */
+    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr);
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */

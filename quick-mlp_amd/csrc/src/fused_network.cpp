@@ -939,9 +939,10 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
     slot = std::move(ck);
 }
 
-const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles)
+const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles)
 {
     const int s = store ? 1 : 0;
+    if (launchTiles) *launchTiles = numTiles;
     {
         int blockSize = 0, pointsPerLane = 1;
         forwardShape(store, VARIANT_DEFAULT, blockSize, pointsPerLane);
@@ -953,27 +954,51 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
     // Kernels that take more tiles per wave are faster per point, but the time grows in steps
     // of one workgroup per compute unit, whether all compute units have one or not. Measured on
     // a 16-level hash grid, per step: 4 waves x 1 tile 26 us (2^16 points), 8 waves x 2 tiles
-    // 82 us (2^18 points), 8 waves x 4 tiles 153 us (2^19 points). Take the shape with the
-    // least estimated time = steps x points per step x relative cost per point.
-    // Only the shape that wins is compiled.
-    int best = -1;
-    double bestCost = 0;
+    // 82 us (2^18 points), 8 waves x 4 tiles 153 us (2^19 points), 8 waves x 8 tiles with the
+    // rows in registers 271 us (2^20 points). Estimated time of a shape = steps x points per
+    // step x relative cost per point. A batch first gets whole steps of the cheapest shape
+    // that it fills (at most two per launch, see gatherChunkPoints), what is left the shape
+    // with the least estimated time; the caller comes back for the rest. Only shapes that
+    // are used are compiled.
+    struct Shape { int variant; long long stepTiles; double costPerPoint; };
+    std::vector<Shape> shapes;
     const int computeUnits = KernelFunction::computeUnits();
     auto consider = [&](int variant, double costPerPoint) {
         int blockSize = 0, pointsPerLane = 1;
         forwardShape(store, variant, blockSize, pointsPerLane);
-        const long long stepTiles = static_cast<long long>(computeUnits) * (blockSize / WARP_SIZE) * pointsPerLane;
-        const double cost = static_cast<double>(divUp<long long>(numTiles, stepTiles)) * stepTiles * costPerPoint;
-        if (best < 0 || cost < bestCost) {
-            best = variant;
-            bestCost = cost;
-        }
+        shapes.push_back({variant, static_cast<long long>(computeUnits) * (blockSize / WARP_SIZE) * pointsPerLane, costPerPoint});
     };
     // measured 258 ps per point against 288 for 8 waves x 4 tiles (16-level hash grid, 2^20 points)
     if (registerVariantTiles(store) > 0 && !registerShapeSpills_[s]) consider(VARIANT_REGISTERS, 0.9);
     if (hasLargeVariant(store)) consider(VARIANT_LARGE, 1.0);
     consider(VARIANT_DEFAULT, 1.075);
     consider(VARIANT_NARROW, 1.39);
+    auto wholeBatch = [&](long long tiles, int& variant) {
+        double bestCost = 0;
+        variant = -1;
+        for (const auto& sh : shapes) {
+            const double cost = static_cast<double>(divUp<long long>(tiles, sh.stepTiles)) * sh.stepTiles * sh.costPerPoint;
+            if (variant < 0 || cost < bestCost) {
+                variant = sh.variant;
+                bestCost = cost;
+            }
+        }
+        return tiles > 0 ? bestCost : 0.0;
+    };
+    int best = -1;
+    double bestCost = wholeBatch(numTiles, best);
+    for (const auto& sh : shapes) {
+        const long long steps = numTiles / sh.stepTiles;
+        if (steps < 1) continue;
+        int unused = -1;
+        const double cost = static_cast<double>(steps * sh.stepTiles) * sh.costPerPoint
+            + wholeBatch(numTiles - steps * sh.stepTiles, unused);
+        if (cost < bestCost) {
+            best = sh.variant;
+            bestCost = cost;
+            if (launchTiles) *launchTiles = static_cast<int>(steps * sh.stepTiles);
+        }
+    }
     compileForwardKernel(store, best);
     if (best == VARIANT_REGISTERS && forwardKernels_[s][best].value().fun.scratchBytes() > MAX_REGISTER_SHAPE_SCRATCH) {
         // the compiler did not get the rows and the gathers into the registers: a kernel that
@@ -981,7 +1006,7 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
         QuickMLP::Instance().getLogger()->debug("the forward kernel with rows in registers spills %d bytes per lane, not used",
                                                 forwardKernels_[s][best].value().fun.scratchBytes());
         registerShapeSpills_[s] = true;
-        return forwardKernelFor(store, numTiles);
+        return forwardKernelFor(store, numTiles, launchTiles);
     }
     return forwardKernels_[s][best].value();
 }
@@ -1115,8 +1140,10 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     const half* networkParams = parametersInference_.dataPtr<half>();
     for (long long start = 0; start < numel;) {
         // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
-        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)));
-        int count = static_cast<int>(std::min<long long>(gatherChunkPoints(ck), numel - start));
+        int launchTiles = 0;
+        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles);
+        int count = static_cast<int>(std::min<long long>(
+            {static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS, numel - start}));
         auto inputAcc = inputAll;
         auto outputAcc = outputAll;
         inputAcc.data_ += start * inputAll.strides_[0];
