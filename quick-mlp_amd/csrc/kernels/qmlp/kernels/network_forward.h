@@ -101,7 +101,7 @@ $$STAGE_PARAMETERS$$
         // encodings: PPL points per lane (one of each tile), each into its staging row.
         // Rows outside the batch are evaluated at the origin and zeroed afterwards so that
         // no NaN enters the matrix cores.
-        PackedRegisterRows<f16, REGISTER_STAGING ? PPL : 1, CHANNELS_IN> encodedRegisters;
+        PackedRegisterRows<f16, REGISTER_STAGING ? PPL : 1, CHANNELS_IN> encodedRegisters = {};   // halves are merged into it
         (void)encodedRegisters;
         {
             StaticArray<float, NUM_INPUTS> encodingInput[PPL];
