@@ -54,6 +54,15 @@ public:
         // takes 8 tiles at once, and 2^20 points are one sweep over the level tables.
         bool registerStaging = true;
 
+        // Inference only: evaluate the points slab by slab of a dense grid that exceeds the L2
+        // (a counting sort of the batch in front of the fused kernel, see point_order.h; the
+        // results are those of the order given). <0 (default): the library decides from the
+        // encodings and the batch size; 0: never; >0: whenever an encoding offers a slab key.
+        // The sorted copy of the inputs lives in device memory that the network allocates on
+        // the first such call and keeps (grown when a larger batch comes); calls of one
+        // network on several streams at once would share it.
+        int sortPoints = -1;
+
         // Accepted for compatibility; the LDS layouts of this implementation are
         // bank-conflict free for 64 lanes by construction and need no skew.
         bool skewSharedMemory = false;
@@ -106,6 +115,23 @@ private:
     std::optional<CompiledKernel> forwardKernels_[2][4];
     // set once the compiled REGISTERS shape turned out to spill heavily: it is not used then
     bool registerShapeSpills_[2] = {false, false};
+
+    // counting sort of the batch by grid slab in front of the inference kernel
+    struct PointOrder
+    {
+        std::optional<KernelFunction> count, scan, scatter;
+        Tensor workspace;           // sorted inputs (floats), order (ints), slab totals and per-chunk histograms (ints)
+        long long capacity = 0;     // points the workspace holds
+    };
+    PointOrder pointOrder_;
+    /** Batches of at least this many points are sorted when sortPoints < 0. */
+    static constexpr int SORT_POINTS_MIN_BATCH = 1 << 20;
+    /**
+     * Sorts the batch by the slab key of the first encoding that offers one.
+     * \return false if the batch stays as it is; else sortedInput views the sorted copy and
+     *   order holds, per row of it, the row of the caller's batch
+     */
+    bool sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream);
 
     struct AdjointLayerInfo
     {

@@ -4,6 +4,7 @@
 #include "json.h"
 #include "kernel_loader.h"
 #include "tensor.h"
+#include <qmlp/kernels/point_order_key.h>
 
 #include <functional>
 #include <optional>
@@ -97,6 +98,18 @@ public:
      * kernel keeps the gathers of several points per lane in flight and sizes that number by it.
      */
     [[nodiscard]] virtual int gatherRegistersPerPoint() const { return 0; }
+
+    /**
+     * Encodings that gather from a table too large for the L2 of one accelerator die, and whose
+     * gathers are close in memory for points that are close in space (dense grids), fill in how
+     * points are assigned to slabs of that table and return true: the fused inference kernel
+     * then evaluates the points slab by slab.
+     */
+    [[nodiscard]] virtual bool pointOrderKey(kernel::PointOrderKey& key) const
+    {
+        (void)key;
+        return false;
+    }
 
     /** Output channels that the device code writes together (the features of a grid entry). */
     [[nodiscard]] virtual int channelsWrittenTogether() const { return 1; }

@@ -51,7 +51,8 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     const half* __restrict__ networkParametersH,
     half* __restrict__ forwardTmpMemoryH,
     int tmpTileOffset,                // STORE: index of this launch's first tile in the whole batch
-    int tmpNumTiles                   // STORE: tiles of the whole batch (a batch may be cut into several launches)
+    int tmpNumTiles,                  // STORE: tiles of the whole batch (a batch may be cut into several launches)
+    const int* __restrict__ pointOrder  // null, or per row of inputs the row of outputs it belongs to (inputs sorted by grid slab)
     $$ENCODING_PARAMETERS$$)
 {
     constexpr int NUM_INPUTS = $$NUM_INPUTS$$;            // raw input channels
@@ -178,6 +179,12 @@ $$CALL_NETWORK_LAYERS$$
 
         // output: lane holds channels 16m+4g+i of the points 4r+nt
         const int actualChannelsOut = outputs.sizes_[1];
+        long long outputRow[NT];   // -1: outside the batch
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int p = tile * TILE_POINTS + 4 * r + nt;
+            outputRow[nt] = p < numel ? (pointOrder ? pointOrder[p] : p) : -1;
+        }
 #pragma unroll
         for (int m = 0; m < MTL; ++m)
 #pragma unroll
@@ -186,10 +193,8 @@ $$CALL_NETWORK_LAYERS$$
                 if (c < actualChannelsOut) {
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
-                        const int p = tile * TILE_POINTS + 4 * r + nt;
-                        if (p < numel)
-                            outputs.data_[static_cast<long long>(p) * outputs.strides_[0]
-                                          + static_cast<long long>(c) * outputs.strides_[1]]
+                        if (outputRow[nt] >= 0)
+                            outputs.data_[outputRow[nt] * outputs.strides_[0] + static_cast<long long>(c) * outputs.strides_[1]]
                                 = static_cast<float>(xOut[nt][m][i]);
                     }
                 }

@@ -1,0 +1,202 @@
+// Orders the points of a batch by the slab of a dense grid they fall into, so that the
+// wavefronts that run side by side gather from the same few megabytes of the table and
+// find them in L1 / L2. A counting sort over at most 1024 slabs in three launches, without
+// atomics on device memory (a first version reserved the ranges with one returning atomic per
+// slab and workgroup: 256 workgroups on the same 64 cache lines took 120 us):
+//   PointOrderCount   one histogram per workgroup (summed in LDS) over its chunk of the batch,
+//   PointOrderScan    per slab, the running sum over the workgroups (in place) and the total,
+//   PointOrderScatter scans the totals into slab offsets, sorts its chunk in LDS and writes
+//                     it to slab offset + running sum + rank in the chunk: a copy of the
+//                     input rows in sorted order and, per sorted position, the index of the
+//                     point in the caller's batch.
+// The order of the points of one chunk inside a slab depends on the timing of the wavefronts;
+// the fused kernel evaluates every point on its own, so its results do not.
+// No counterpart in the reference, which evaluates the points in the order given.
+
+#include <qmlp/kernels/common.h>
+#include <qmlp/kernels/point_order_key.h>
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+constexpr int POINT_ORDER_MAX_SLABS = 1024;
+constexpr int POINT_ORDER_BLOCK = 1024;
+constexpr int POINT_ORDER_POINTS_PER_THREAD = 8;    // a workgroup's chunk: 8192 points (offsets in it take 13 bits)
+
+/** Slab of the point in row `index`: the two leading grid coordinates, clamped to the box. */
+__device__ __forceinline__ int pointOrderSlab(const Tensor2Read<float>& inputs, long long index, const PointOrderKey& key)
+{
+    const float* row = inputs.data_ + index * inputs.strides_[0];
+    const float p0 = (row[static_cast<long long>(key.channel0) * inputs.strides_[1]] - key.min0) * key.scale0;
+    // the comparisons are false for NaN, which then lands in slab 0
+    int s = p0 > 0.f ? static_cast<int>(fminf(p0, static_cast<float>(key.slabs0 - 1))) : 0;
+    if (key.slabs1 > 1) {
+        const float p1 = (row[static_cast<long long>(key.channel1) * inputs.strides_[1]] - key.min1) * key.scale1;
+        const int s1 = p1 > 0.f ? static_cast<int>(fminf(p1, static_cast<float>(key.slabs1 - 1))) : 0;
+        s = s * key.slabs1 + s1;
+    }
+    return s;
+}
+
+/** histogram: (workgroups, POINT_ORDER_MAX_SLABS), every entry is written. */
+__global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderCount(
+    int numel, const Tensor2Read<float> inputs, const PointOrderKey key, int* __restrict__ histogram)
+{
+    __shared__ int sCount[POINT_ORDER_MAX_SLABS];
+    sCount[threadIdx.x] = 0;
+    __syncthreads();
+    const long long chunk = static_cast<long long>(blockIdx.x) * (POINT_ORDER_BLOCK * POINT_ORDER_POINTS_PER_THREAD);
+#pragma unroll
+    for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
+        const long long index = chunk + k * POINT_ORDER_BLOCK + threadIdx.x;
+        if (index < numel) atomicAdd(&sCount[pointOrderSlab(inputs, index, key)], 1);
+    }
+    __syncthreads();
+    histogram[blockIdx.x * POINT_ORDER_MAX_SLABS + threadIdx.x] = sCount[threadIdx.x];
+}
+
+/**
+ * histogram[w][slab] becomes the number of points of the slab in the chunks before w,
+ * totals[slab] their number in all chunks. A workgroup takes 64 slabs (one per lane); its 16
+ * wavefronts take a sixteenth of the chunks each: sum, exchange through LDS, running sum.
+ */
+__global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScan(int chunks, int* __restrict__ histogram, int* __restrict__ totals)
+{
+    constexpr int WAVES = POINT_ORDER_BLOCK / WAVE_SIZE;
+    constexpr int BATCH = 16;   // loads in flight
+    __shared__ int sPartial[WAVES][WAVE_SIZE];
+    const int lane = threadIdx.x % WAVE_SIZE, wave = threadIdx.x / WAVE_SIZE;
+    const int slab = blockIdx.x * WAVE_SIZE + lane;
+    const int perWave = (chunks + WAVES - 1) / WAVES;
+    const int begin = min(wave * perWave, chunks), end = min(begin + perWave, chunks);
+    int sum = 0;
+    for (int w0 = begin; w0 < end; w0 += BATCH) {
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j)
+            if (w0 + j < end) sum += histogram[(w0 + j) * POINT_ORDER_MAX_SLABS + slab];
+    }
+    sPartial[wave][lane] = sum;
+    __syncthreads();
+    int running = 0;
+    for (int q = 0; q < wave; ++q) running += sPartial[q][lane];
+    if (wave == WAVES - 1) totals[slab] = running + sum;
+    for (int w0 = begin; w0 < end; w0 += BATCH) {
+        int v[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) v[j] = w0 + j < end ? histogram[(w0 + j) * POINT_ORDER_MAX_SLABS + slab] : 0;
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+            if (w0 + j < end) histogram[(w0 + j) * POINT_ORDER_MAX_SLABS + slab] = running;
+            running += v[j];
+        }
+    }
+}
+
+/** Exclusive scan over the POINT_ORDER_MAX_SLABS values held one per thread of the workgroup. */
+__device__ __forceinline__ int pointOrderBlockScan(int value, int* sWaveSum)
+{
+    const int lane = threadIdx.x % WAVE_SIZE, wave = threadIdx.x / WAVE_SIZE;
+    int inclusive = value;
+#pragma unroll
+    for (int d = 1; d < WAVE_SIZE; d *= 2) {
+        const int other = __shfl_up(inclusive, d, WAVE_SIZE);
+        if (lane >= d) inclusive += other;
+    }
+    __syncthreads();   // sWaveSum may still be read from a previous scan
+    if (lane == WAVE_SIZE - 1) sWaveSum[wave] = inclusive;
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += sWaveSum[w];
+    return before + inclusive - value;
+}
+
+/** The channels of one input row; one 16-byte load where the layout allows it. */
+template <int MAX_CHANNELS>
+__device__ __forceinline__ void pointOrderLoadRow(const Tensor2Read<float>& inputs, long long index, bool vector4, float (&row)[MAX_CHANNELS])
+{
+    const float* src = inputs.data_ + index * inputs.strides_[0];
+    if (vector4) {
+        const float4 v = *reinterpret_cast<const float4*>(src);
+        row[0] = v.x; row[1] = v.y; row[2] = v.z; row[3] = v.w;
+    } else {
+#pragma unroll
+        for (int c = 0; c < MAX_CHANNELS; ++c)
+            row[c] = c < inputs.sizes_[1] ? src[static_cast<long long>(c) * inputs.strides_[1]] : 0.f;
+    }
+}
+
+/**
+ * The workgroup first sorts the indices of its chunk by slab in LDS, then walks the sorted
+ * chunk with consecutive lanes on consecutive positions, so that the stores of a wavefront
+ * fall into a few runs (a scatter straight from the unsorted chunk sent every lane's stores
+ * to a line of their own and took 80 us for 2^21 points).
+ * \tparam MAX_CHANNELS at least the number of input channels (4, 8, 16)
+ */
+template <int MAX_CHANNELS>
+__global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
+    int numel, const Tensor2Read<float> inputs, const PointOrderKey key,
+    const int* __restrict__ histogram,  // as PointOrderScan left it
+    const int* __restrict__ totals,
+    float* __restrict__ sortedInputs,   // (numel, inputs.sizes_[1]), dense, 16-byte aligned
+    int* __restrict__ order)            // (numel): sorted position -> index in the batch
+{
+    constexpr int CHUNK = POINT_ORDER_BLOCK * POINT_ORDER_POINTS_PER_THREAD;
+    __shared__ int sStart[POINT_ORDER_MAX_SLABS];        // first position of the chunk's points of a slab in the sorted batch
+    __shared__ int sCount[POINT_ORDER_MAX_SLABS];
+    __shared__ int sLocalStart[POINT_ORDER_MAX_SLABS];   // the same inside the sorted chunk
+    __shared__ int sWaveSum[POINT_ORDER_BLOCK / WAVE_SIZE];
+    __shared__ unsigned int sSorted[CHUNK];              // sorted chunk: slab << 16 | offset of the point in the chunk
+    const int t = threadIdx.x;
+
+    sCount[t] = 0;
+    const int total = totals[t];
+    const int slabStart = pointOrderBlockScan(total, sWaveSum);   // holds a barrier after sCount = 0
+    sStart[t] = slabStart + histogram[blockIdx.x * POINT_ORDER_MAX_SLABS + t];
+
+    const long long chunk = static_cast<long long>(blockIdx.x) * CHUNK;
+    const int chunkPoints = static_cast<int>(min(static_cast<long long>(CHUNK), numel - chunk));
+    int slab[POINT_ORDER_POINTS_PER_THREAD], rank[POINT_ORDER_POINTS_PER_THREAD];
+#pragma unroll
+    for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
+        const int j = k * POINT_ORDER_BLOCK + t;
+        slab[k] = 0;
+        rank[k] = 0;
+        if (j < chunkPoints) {
+            slab[k] = pointOrderSlab(inputs, chunk + j, key);
+            rank[k] = atomicAdd(&sCount[slab[k]], 1);
+        }
+    }
+    __syncthreads();
+    sLocalStart[t] = pointOrderBlockScan(sCount[t], sWaveSum);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
+        const int j = k * POINT_ORDER_BLOCK + t;
+        if (j < chunkPoints) sSorted[sLocalStart[slab[k]] + rank[k]] = static_cast<unsigned int>(slab[k]) << 16 | static_cast<unsigned int>(j);
+    }
+    __syncthreads();
+
+    const int channels = inputs.sizes_[1];
+    const bool vector4 = channels == 4 && inputs.strides_[1] == 1 && inputs.strides_[0] % 4 == 0
+        && reinterpret_cast<unsigned long long>(inputs.data_) % 16 == 0;
+#pragma unroll 4
+    for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
+        const int j = k * POINT_ORDER_BLOCK + t;
+        if (j >= chunkPoints) continue;
+        const unsigned int entry = sSorted[j];
+        const long long index = chunk + (entry & 0xffffu);
+        const int s = static_cast<int>(entry >> 16);
+        float row[MAX_CHANNELS];
+        pointOrderLoadRow<MAX_CHANNELS>(inputs, index, vector4, row);
+        const long long position = sStart[s] + (j - sLocalStart[s]);
+        order[position] = static_cast<int>(index);
+        if (vector4) {
+            *reinterpret_cast<float4*>(sortedInputs + position * 4) = make_float4(row[0], row[1], row[2], row[3]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < MAX_CHANNELS; ++c)
+                if (c < channels) sortedInputs[position * channels + c] = row[c];
+        }
+    }
+}
+
+QUICKMLP_KERNEL_NAMESPACE_END

@@ -73,6 +73,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         if (compileOptions_.pointsPerLane > 8)
             throw configuration_error("points_per_lane must be at most 8, but is %d", compileOptions_.pointsPerLane);
         compileOptions_.registerStaging = options.value("register_staging", compileOptions_.registerStaging);
+        compileOptions_.sortPoints = options.value("sort_points", compileOptions_.sortPoints);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
             options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
@@ -1082,6 +1083,16 @@ void FusedNetwork::precompile(int adjointFlags)
         if (registerVariantTiles(store) > 0) compileForwardKernel(store, VARIANT_REGISTERS, true);
     }
     if (adjointFlags > 0) compileBackwardKernel(adjointFlags, true);
+    kernel::PointOrderKey key{};
+    for (const auto& e : encodings_)
+        if (compileOptions_.sortPoints != 0 && e->pointOrderKey(key)) {
+            auto kl = QuickMLP::Instance().kernelLoader();
+            const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
+            const std::string scatter = "PointOrderScatter<" + std::to_string(channelsIn_ <= 4 ? 4 : channelsIn_ <= 8 ? 8 : 16) + ">";
+            for (const std::string& name : {std::string("PointOrderCount"), std::string("PointOrderScan"), scatter})
+                kl->getKernel("qmlp::kernel::" + name, source, loaderFlags(true));
+            break;
+        }
 }
 
 // ------------------------------------------------------------------ launches
@@ -1135,8 +1146,12 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
 {
     const int numel = input.size(0);
     int tmpNumTiles = divUp(numel, TILE_POINTS);
-    const auto inputAll = input.accessor<kernel::Tensor2Read<float>>();
+    auto inputAll = input.accessor<kernel::Tensor2Read<float>>();
     const auto outputAll = output.accessor<kernel::Tensor2RW<float>>();
+    // inference of a network with a large dense grid: rows of the input sorted by grid slab,
+    // every row of the result written where its point stands in the caller's batch
+    const int* orderAll = nullptr;
+    const bool sorted = !store && sortPoints(input, inputAll, orderAll, stream);
     const half* networkParams = parametersInference_.dataPtr<half>();
     for (long long start = 0; start < numel;) {
         // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
@@ -1147,17 +1162,78 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
         auto inputAcc = inputAll;
         auto outputAcc = outputAll;
         inputAcc.data_ += start * inputAll.strides_[0];
-        outputAcc.data_ += start * outputAll.strides_[0];
+        if (!sorted) outputAcc.data_ += start * outputAll.strides_[0];
         inputAcc.sizes_[0] = outputAcc.sizes_[0] = count;
+        const int* order = sorted ? orderAll + start : nullptr;
         int tmpTileOffset = static_cast<int>(start / TILE_POINTS);
         const int waves = ck.blockSize / WARP_SIZE;
         const int grid = std::min(divUp(divUp(count, TILE_POINTS), waves * ck.pointsPerLane), ck.fullGrid);
-        std::vector<void*> args = {&count, &inputAcc, &outputAcc, &networkParams, &tmpMemory, &tmpTileOffset, &tmpNumTiles};
+        std::vector<void*> args = {&count, &inputAcc, &outputAcc, &networkParams, &tmpMemory, &tmpTileOffset, &tmpNumTiles, &order};
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
         start += count;
     }
+}
+
+bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream)
+{
+    const int numel = input.size(0);
+    if (compileOptions_.sortPoints == 0 || (compileOptions_.sortPoints < 0 && numel < SORT_POINTS_MIN_BATCH)) return false;
+    kernel::PointOrderKey key{};
+    bool found = false;
+    for (const auto& e : encodings_)
+        if (e->pointOrderKey(key)) {
+            found = true;
+            break;
+        }
+    const int channels = input.size(1);
+    if (!found || channels > 16) return false;
+    const int maxChannels = channels <= 4 ? 4 : channels <= 8 ? 8 : 16;
+
+    auto& po = pointOrder_;
+    if (!po.scatter.has_value()) {
+        auto kl = QuickMLP::Instance().kernelLoader();
+        const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
+        po.scan = kl->getKernel("qmlp::kernel::PointOrderScan", source, loaderFlags(false)).value();
+        po.count = kl->getKernel("qmlp::kernel::PointOrderCount", source, loaderFlags(false)).value();
+        po.scatter = kl->getKernel("qmlp::kernel::PointOrderScatter<" + std::to_string(maxChannels) + ">", source, loaderFlags(false)).value();
+    }
+    constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 8 * BLOCK;   // as in point_order.h
+    if (po.capacity < numel) {
+        // words: sorted inputs, order, one histogram per chunk, totals
+        const long long words = static_cast<long long>(numel) * (channels + 1) + (divUp(numel, CHUNK) + 1ll) * SLABS;
+        CHECK_ERROR(words <= std::numeric_limits<int32_t>::max(), "Batch too large to be sorted by grid slab, set the option sort_points to 0");
+        po.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
+        po.capacity = numel;
+    }
+    float* sortedData = po.workspace.dataPtr<float>();
+    int* orderData = reinterpret_cast<int*>(sortedData + po.capacity * channels);   // the sorted rows come first: 16-byte aligned
+    int* totals = orderData + po.capacity;
+    int* histogram = totals + SLABS;
+
+    int count = numel;
+    auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+    int chunks = divUp(numel, CHUNK);
+    {
+        void* args[] = {&count, &inputAcc, &key, &histogram};
+        po.count.value().launch(chunks, BLOCK, 0, stream, args);
+    }
+    {
+        void* args[] = {&chunks, &histogram, &totals};
+        po.scan.value().launch(SLABS / WARP_SIZE, BLOCK, 0, stream, args);
+    }
+    {
+        void* args[] = {&count, &inputAcc, &key, &histogram, &totals, &sortedData, &orderData};
+        po.scatter.value().launch(chunks, BLOCK, 0, stream, args);
+    }
+    sortedInput.data_ = sortedData;
+    sortedInput.sizes_[0] = numel;
+    sortedInput.sizes_[1] = channels;
+    sortedInput.strides_[0] = channels;
+    sortedInput.strides_[1] = 1;
+    order = orderData;
+    return true;
 }
 
 size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlags)
@@ -1351,6 +1427,9 @@ void FusedNetwork::clearCachedKernels()
     for (auto& perStore : forwardKernels_)
         for (auto& k : perStore) k = {};
     for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i) backwardKernel_[i] = {};
+    pointOrder_.scan = {};
+    pointOrder_.count = {};
+    pointOrder_.scatter = {};
 }
 
 QUICKMLP_NAMESPACE_END

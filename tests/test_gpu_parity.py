@@ -701,3 +701,47 @@ def test_rows_staged_in_registers_give_the_same_bits_as_rows_staged_in_lds(preci
         assert np.array_equal(ga[key], gb[key]), key
     t = gb["table_grads"][0]
     assert_close(ga["table_grads"][0], t, "grid gradients (atomics)", rel=1e-3, abs_=1e-4 * float(np.abs(t).max()))
+
+
+def test_inference_sorted_by_grid_slab_gives_the_same_bits_as_the_order_given():
+    """A network with a dense grid larger than the L2 evaluates large inference batches slab by
+    slab of the grid (``sort_points``; a counting sort in front of the fused kernel). Every
+    point is evaluated on its own, so the result has to agree bit for bit with the batch
+    evaluated as given: uniform points, ragged sizes, points that all fall into one slab,
+    points outside the box and NaN coordinates (slab 0), a batch that grows between calls, and
+    a small batch against the CPU oracle."""
+    c = bc.CONFIGS[5]
+    cases = []
+    for mode in (1, 0):
+        cfg = json.loads(json.dumps(c["cfg"]))
+        cfg.setdefault("options", {})["sort_points"] = mode
+        rng = np.random.default_rng(11)
+        case = Case(cfg, bc.ORACLE_ACTIVATIONS)
+        case.set_parameters(bc.make_parameters(5, rng).astype(np.float32))
+        case.set_table(0, bc.make_table(5, case.oracle.encodings[0][1].n_params, rng, 1.0))
+        cases.append(case)
+    sorted_, plain = cases
+    rng = np.random.default_rng(12)
+    for N in (1, 63, 8191, 8193, (1 << 18) + 77, (1 << 21) - 5):
+        print("sorted by slab: %d points" % N, flush=True)
+        X = bc.make_inputs(5, N, rng)
+        a, b = sorted_.gpu_inference(X), plain.gpu_inference(X)
+        assert np.array_equal(a, b)
+        assert N < 64 or np.abs(a).max() > 0.01
+    N = 50000
+    X = bc.make_inputs(5, N, rng)
+    X[:, 0] = 0.5                     # one slab of the leading coordinate
+    X[:, 1] = X[:, 1] * 0.01 + 0.3    # one or two of the second
+    X[::7, 0] = -3.0                  # outside the box: clamped
+    X[::11, 1] = 17.0
+    assert np.array_equal(sorted_.gpu_inference(X), plain.gpu_inference(X))
+    assert_close(sorted_.gpu_inference(X[:4096]), sorted_.oracle.forward(X[:4096]), "sorted inference against the oracle")
+    X[::5, 0] = np.nan
+    a, b = sorted_.gpu_inference(X), plain.gpu_inference(X)
+    assert np.array_equal(np.isnan(a), np.isnan(b)) and np.array_equal(a[~np.isnan(a)], b[~np.isnan(b)])
+    # strided input rows
+    wide = torch.rand((70000, 7), device="cuda")
+    view = wide[:, 2:6]
+    a = sorted_.net.inference(view, sorted_.params, sorted_.encoding_parameters())
+    b = plain.net.inference(view.contiguous(), plain.params, plain.encoding_parameters())
+    assert torch.equal(a, b)
