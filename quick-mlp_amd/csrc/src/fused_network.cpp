@@ -1203,7 +1203,7 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     if (po.capacity < numel) {
         // words: sorted inputs, order, one histogram per chunk, totals
         const long long words = static_cast<long long>(numel) * (channels + 1) + (divUp(numel, CHUNK) + 1ll) * SLABS;
-        CHECK_ERROR(words <= std::numeric_limits<int32_t>::max(), "Batch too large to be sorted by grid slab, set the option sort_points to 0");
+        if (words > std::numeric_limits<int32_t>::max()) return false;   // beyond one tensor: the batch stays as it is
         po.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
         po.capacity = numel;
     }

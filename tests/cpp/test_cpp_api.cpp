@@ -67,6 +67,34 @@ static void hostPart()
     CHECK(thrown);
     // the kernels of this network compile for gfx950 without a device
     net.precompile(FusedNetwork::GRADIENTS_INPUT | FusedNetwork::GRADIENTS_NETWORK_WEIGHTS);
+
+    // Which grids offer a slab key for sorting inference batches: a dense 32^4 grid with 8 fp16
+    // features (16.8 MB) does, in 31 x 31 slabs of one cell over its box [1,3] x [0,4];
+    // a 16-level hash grid whose dense levels are small does not, nor does a small dense grid.
+    {
+        auto dense = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 1, "n_in": 4,
+            "n_levels": 1, "n_features_per_level": 8, "log2_hashmap_size": -1, "min_resolution": 32, "max_resolution": 32,
+            "combination_mode": "concat", "bounding_box_min": [1, 0, 0, 0], "bounding_box_size": [2, 4, 1, 1],
+            "parameter_precision": "half"})json"));
+        kernel::PointOrderKey key{};
+        CHECK(dense->pointOrderKey(key));
+        CHECK(key.channel0 == 1 && key.channel1 == 2 && key.slabs0 == 31 && key.slabs1 == 31);
+        CHECK(key.min0 == 1.f && key.min1 == 0.f && key.scale0 == 15.5f && key.scale1 == 7.75f);
+        auto hashed = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 0, "n_in": 3,
+            "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 19, "min_resolution": 16, "max_resolution": 4096,
+            "combination_mode": "concat", "bounding_box_min": [0, 0, 0], "bounding_box_size": [1, 1, 1]})json"));
+        CHECK(!hashed->pointOrderKey(key));
+        auto small = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 0, "n_in": 3,
+            "n_levels": 1, "n_features_per_level": 2, "log2_hashmap_size": -1, "min_resolution": 64, "max_resolution": 64,
+            "combination_mode": "concat", "bounding_box_min": [0, 0, 0], "bounding_box_size": [1, 1, 1]})json"));
+        CHECK(!small->pointOrderKey(key));
+        // a wide dense 3-D grid: 300 cells per coordinate in 30 slabs of 10 cells
+        auto wide = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 0, "n_in": 3,
+            "n_levels": 1, "n_features_per_level": 2, "log2_hashmap_size": -1, "min_resolution": 301, "max_resolution": 301,
+            "combination_mode": "concat", "bounding_box_min": [0, 0, 0], "bounding_box_size": [1, 1, 1]})json"));
+        CHECK(wide->pointOrderKey(key));
+        CHECK(key.slabs0 == 30 && key.slabs1 == 30 && key.scale0 == 30.f);
+    }
 }
 
 static float celu(float x) { return x > 0 ? x : std::exp(x) - 1; }
