@@ -91,6 +91,9 @@ $$STAGE_PARAMETERS$$
     __syncthreads();
 
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
+    const bool inputRowsAreVectors = inputs.strides_[1] == 1 && inputs.strides_[0] % NUM_INPUTS == 0
+        && reinterpret_cast<unsigned long long>(inputs.data_) % (NUM_INPUTS * sizeof(float)) == 0;
+    (void)inputRowsAreVectors;
     // the regions of the temporary memory are laid out for the whole batch
     const long long numel64 = static_cast<long long>(tmpNumTiles) * TILE_POINTS;
     (void)numel64;
@@ -113,11 +116,25 @@ $$STAGE_PARAMETERS$$
                 const int index = (tile0 + q) * TILE_POINTS + lane;
                 valid[q] = index < numel;
                 bindEncodingRow(encodingOutput, sStage, q, lane);
+                const float* inputRow = inputs.data_ + static_cast<long long>(index) * inputs.strides_[0];
+                if ((NUM_INPUTS == 2 || NUM_INPUTS == 4) && inputRowsAreVectors) {
+                    // the channels of a row lie side by side: one load per point
+                    if (NUM_INPUTS == 4) {
+                        const float4 v = valid[q] ? *reinterpret_cast<const float4*>(inputRow) : make_float4(0.f, 0.f, 0.f, 0.f);
+                        encodingInput[q][0] = v.x;
+                        encodingInput[q][NUM_INPUTS > 1 ? 1 : 0] = v.y;
+                        encodingInput[q][NUM_INPUTS > 2 ? 2 : 0] = v.z;
+                        encodingInput[q][NUM_INPUTS > 3 ? 3 : 0] = v.w;
+                    } else {
+                        const float2 v = valid[q] ? *reinterpret_cast<const float2*>(inputRow) : make_float2(0.f, 0.f);
+                        encodingInput[q][0] = v.x;
+                        encodingInput[q][NUM_INPUTS > 1 ? 1 : 0] = v.y;
+                    }
+                } else {
 #pragma unroll
-                for (int i = 0; i < NUM_INPUTS; ++i)
-                    encodingInput[q][i] = valid[q] ? inputs.data_[static_cast<long long>(index) * inputs.strides_[0]
-                                                                  + static_cast<long long>(i) * inputs.strides_[1]]
-                                                   : 0.f;
+                    for (int i = 0; i < NUM_INPUTS; ++i)
+                        encodingInput[q][i] = valid[q] ? inputRow[static_cast<long long>(i) * inputs.strides_[1]] : 0.f;
+                }
             }
 $$CALL_ENCODINGS$$
 #pragma unroll
@@ -185,20 +202,43 @@ $$CALL_NETWORK_LAYERS$$
             const int p = tile * TILE_POINTS + 4 * r + nt;
             outputRow[nt] = p < numel ? (pointOrder ? pointOrder[p] : p) : -1;
         }
+        // two or four output channels that lie side by side in memory leave as one store per
+        // point (the lanes of group 0 hold channels 0..3 of their points)
+        const bool rowsOfFloat2 = actualChannelsOut == 2 && outputs.strides_[1] == 1 && outputs.strides_[0] % 2 == 0
+            && reinterpret_cast<unsigned long long>(outputs.data_) % 8 == 0;
+        const bool rowsOfFloat4 = actualChannelsOut == 4 && outputs.strides_[1] == 1 && outputs.strides_[0] % 4 == 0
+            && reinterpret_cast<unsigned long long>(outputs.data_) % 16 == 0;
+        if (rowsOfFloat2 || rowsOfFloat4) {
+            if (g == 0) {
 #pragma unroll
-        for (int m = 0; m < MTL; ++m)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int c = 16 * m + 4 * g + i;
-                if (c < actualChannelsOut) {
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        if (outputRow[nt] >= 0)
-                            outputs.data_[outputRow[nt] * outputs.strides_[0] + static_cast<long long>(c) * outputs.strides_[1]]
-                                = static_cast<float>(xOut[nt][m][i]);
-                    }
+                for (int nt = 0; nt < NT; ++nt) {
+                    if (outputRow[nt] < 0) continue;
+                    float* row = outputs.data_ + outputRow[nt] * outputs.strides_[0];
+                    if (rowsOfFloat2)
+                        *reinterpret_cast<float2*>(row) =
+                            make_float2(static_cast<float>(xOut[nt][0][0]), static_cast<float>(xOut[nt][0][1]));
+                    else
+                        *reinterpret_cast<float4*>(row) =
+                            make_float4(static_cast<float>(xOut[nt][0][0]), static_cast<float>(xOut[nt][0][1]),
+                                        static_cast<float>(xOut[nt][0][2]), static_cast<float>(xOut[nt][0][3]));
                 }
             }
+        } else {
+#pragma unroll
+            for (int m = 0; m < MTL; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int c = 16 * m + 4 * g + i;
+                    if (c < actualChannelsOut) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) {
+                            if (outputRow[nt] >= 0)
+                                outputs.data_[outputRow[nt] * outputs.strides_[0] + static_cast<long long>(c) * outputs.strides_[1]]
+                                    = static_cast<float>(xOut[nt][m][i]);
+                        }
+                    }
+                }
+        }
         }
         waveLdsSync();   // the staging rows are overwritten by the next group of tiles
     }
