@@ -102,6 +102,10 @@ $$ZERO_LDS_GRADIENTS$$
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
     const int actualChannelsOut = adjOutputs.sizes_[1];
+    const bool adjOutputRowsOfFloat2 = actualChannelsOut == 2 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 2 == 0
+        && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 8 == 0;
+    const bool adjOutputRowsOfFloat4 = actualChannelsOut == 4 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 4 == 0
+        && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 16 == 0;
     for (int tileBase = blockIdx.x * WAVES; tileBase < numTiles; tileBase += gridDim.x * WAVES)
     {
         const int tile = tileBase + wave;
@@ -117,17 +121,40 @@ $$ZERO_LDS_GRADIENTS$$
             const int p = tile * TILE_POINTS + 4 * r + nt;
             const bool pv = p < numel;
             validMask |= pv ? (1 << nt) : 0;
+            if (adjOutputRowsOfFloat2 || adjOutputRowsOfFloat4) {
+                // two or four channels side by side in memory: one load per point (lane group 0
+                // holds channels 0..3 of its points, everything else is zero)
 #pragma unroll
-            for (int m = 0; m < MTL; ++m)
+                for (int m = 0; m < MTL; ++m)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int c = 16 * m + 4 * g + i;
-                    float v = 0.f;
-                    if (pv && c < actualChannelsOut)
-                        v = adjOutputs.data_[static_cast<long long>(p) * adjOutputs.strides_[0]
-                                             + static_cast<long long>(c) * adjOutputs.strides_[1]];
-                    dyOut[nt][m][i] = static_cast<f16>(v);
+                    for (int i = 0; i < 4; ++i) dyOut[nt][m][i] = static_cast<f16>(0);
+                if (pv && g == 0) {
+                    const float* row = adjOutputs.data_ + static_cast<long long>(p) * adjOutputs.strides_[0];
+                    if (adjOutputRowsOfFloat4) {
+                        const float4 v = *reinterpret_cast<const float4*>(row);
+                        dyOut[nt][0][0] = static_cast<f16>(v.x);
+                        dyOut[nt][0][1] = static_cast<f16>(v.y);
+                        dyOut[nt][0][2] = static_cast<f16>(v.z);
+                        dyOut[nt][0][3] = static_cast<f16>(v.w);
+                    } else {
+                        const float2 v = *reinterpret_cast<const float2*>(row);
+                        dyOut[nt][0][0] = static_cast<f16>(v.x);
+                        dyOut[nt][0][1] = static_cast<f16>(v.y);
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int m = 0; m < MTL; ++m)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int c = 16 * m + 4 * g + i;
+                        float v = 0.f;
+                        if (pv && c < actualChannelsOut)
+                            v = adjOutputs.data_[static_cast<long long>(p) * adjOutputs.strides_[0]
+                                                 + static_cast<long long>(c) * adjOutputs.strides_[1]];
+                        dyOut[nt][m][i] = static_cast<f16>(v);
+                    }
+            }
         }
 
         // layers, last to first
@@ -157,10 +184,21 @@ $$CALL_NETWORK_LAYERS$$
 $$CALL_ENCODINGS$$
 
                 if constexpr (HAS_INPUT_GRADIENTS) {
+                    float* adjRow = adjInputs.data_ + static_cast<long long>(index) * adjInputs.strides_[0];
+                    if (NUM_INPUTS == 4 && adjInputs.strides_[1] == 1 && adjInputs.strides_[0] % 4 == 0
+                        && reinterpret_cast<unsigned long long>(adjInputs.data_) % 16 == 0) {
+                        // the four channels of a row side by side: one load and one store
+                        float4 v = *reinterpret_cast<float4*>(adjRow);
+                        v.x += adjEncodingInput[0];
+                        v.y += adjEncodingInput[NUM_INPUTS > 1 ? 1 : 0];
+                        v.z += adjEncodingInput[NUM_INPUTS > 2 ? 2 : 0];
+                        v.w += adjEncodingInput[NUM_INPUTS > 3 ? 3 : 0];
+                        *reinterpret_cast<float4*>(adjRow) = v;
+                    } else {
 #pragma unroll
-                    for (int i = 0; i < NUM_INPUTS; ++i)
-                        adjInputs.data_[static_cast<long long>(index) * adjInputs.strides_[0]
-                                        + static_cast<long long>(i) * adjInputs.strides_[1]] += adjEncodingInput[i];
+                        for (int i = 0; i < NUM_INPUTS; ++i)
+                            adjRow[static_cast<long long>(i) * adjInputs.strides_[1]] += adjEncodingInput[i];
+                    }
                 }
             }
 
