@@ -91,8 +91,9 @@ $$STAGE_PARAMETERS$$
     __syncthreads();
 
     const int numTiles = (numel + TILE_POINTS - 1) / TILE_POINTS;
-    const bool inputRowsAreVectors = inputs.strides_[1] == 1 && inputs.strides_[0] % NUM_INPUTS == 0
-        && reinterpret_cast<unsigned long long>(inputs.data_) % (NUM_INPUTS * sizeof(float)) == 0;
+    constexpr int INPUT_VECTOR = NUM_INPUTS % 4 == 0 ? 4 : 2;   // floats per load
+    const bool inputRowsAreVectors = inputs.strides_[1] == 1 && inputs.strides_[0] % INPUT_VECTOR == 0
+        && reinterpret_cast<unsigned long long>(inputs.data_) % (INPUT_VECTOR * sizeof(float)) == 0;
     (void)inputRowsAreVectors;
     // the regions of the temporary memory are laid out for the whole batch
     const long long numel64 = static_cast<long long>(tmpNumTiles) * TILE_POINTS;
@@ -117,14 +118,17 @@ $$STAGE_PARAMETERS$$
                 valid[q] = index < numel;
                 bindEncodingRow(encodingOutput, sStage, q, lane);
                 const float* inputRow = inputs.data_ + static_cast<long long>(index) * inputs.strides_[0];
-                if ((NUM_INPUTS == 2 || NUM_INPUTS == 4) && inputRowsAreVectors) {
-                    // the channels of a row lie side by side: one load per point
-                    if (NUM_INPUTS == 4) {
-                        const float4 v = valid[q] ? *reinterpret_cast<const float4*>(inputRow) : make_float4(0.f, 0.f, 0.f, 0.f);
-                        encodingInput[q][0] = v.x;
-                        encodingInput[q][NUM_INPUTS > 1 ? 1 : 0] = v.y;
-                        encodingInput[q][NUM_INPUTS > 2 ? 2 : 0] = v.z;
-                        encodingInput[q][NUM_INPUTS > 3 ? 3 : 0] = v.w;
+                if ((NUM_INPUTS == 2 || NUM_INPUTS % 4 == 0) && inputRowsAreVectors) {
+                    // the channels of a row lie side by side: 16 (or 8) bytes per load
+                    if (NUM_INPUTS % 4 == 0) {
+#pragma unroll
+                        for (int i = 0; i + 3 < NUM_INPUTS; i += 4) {
+                            const float4 v = valid[q] ? *reinterpret_cast<const float4*>(inputRow + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+                            encodingInput[q][i] = v.x;
+                            encodingInput[q][i + 1] = v.y;
+                            encodingInput[q][i + 2] = v.z;
+                            encodingInput[q][i + 3] = v.w;
+                        }
                     } else {
                         const float2 v = valid[q] ? *reinterpret_cast<const float2*>(inputRow) : make_float2(0.f, 0.f);
                         encodingInput[q][0] = v.x;
@@ -202,25 +206,32 @@ $$CALL_NETWORK_LAYERS$$
             const int p = tile * TILE_POINTS + 4 * r + nt;
             outputRow[nt] = p < numel ? (pointOrder ? pointOrder[p] : p) : -1;
         }
-        // two or four output channels that lie side by side in memory leave as one store per
-        // point (the lanes of group 0 hold channels 0..3 of their points)
+        // output channels that lie side by side in memory leave four at a time (a lane holds
+        // channels 16m+4g .. +3 of its points), rows of two channels as one 8-byte store
         const bool rowsOfFloat2 = actualChannelsOut == 2 && outputs.strides_[1] == 1 && outputs.strides_[0] % 2 == 0
             && reinterpret_cast<unsigned long long>(outputs.data_) % 8 == 0;
-        const bool rowsOfFloat4 = actualChannelsOut == 4 && outputs.strides_[1] == 1 && outputs.strides_[0] % 4 == 0
+        const bool rowsOfFloat4 = actualChannelsOut % 4 == 0 && outputs.strides_[1] == 1 && outputs.strides_[0] % 4 == 0
             && reinterpret_cast<unsigned long long>(outputs.data_) % 16 == 0;
-        if (rowsOfFloat2 || rowsOfFloat4) {
+        if (rowsOfFloat4) {
+#pragma unroll
+            for (int m = 0; m < MTL; ++m) {
+                const int c = 16 * m + 4 * g;
+                if (c >= actualChannelsOut) continue;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    if (outputRow[nt] < 0) continue;
+                    *reinterpret_cast<float4*>(outputs.data_ + outputRow[nt] * outputs.strides_[0] + c) =
+                        make_float4(static_cast<float>(xOut[nt][m][0]), static_cast<float>(xOut[nt][m][1]),
+                                    static_cast<float>(xOut[nt][m][2]), static_cast<float>(xOut[nt][m][3]));
+                }
+            }
+        } else if (rowsOfFloat2) {
             if (g == 0) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     if (outputRow[nt] < 0) continue;
-                    float* row = outputs.data_ + outputRow[nt] * outputs.strides_[0];
-                    if (rowsOfFloat2)
-                        *reinterpret_cast<float2*>(row) =
-                            make_float2(static_cast<float>(xOut[nt][0][0]), static_cast<float>(xOut[nt][0][1]));
-                    else
-                        *reinterpret_cast<float4*>(row) =
-                            make_float4(static_cast<float>(xOut[nt][0][0]), static_cast<float>(xOut[nt][0][1]),
-                                        static_cast<float>(xOut[nt][0][2]), static_cast<float>(xOut[nt][0][3]));
+                    *reinterpret_cast<float2*>(outputs.data_ + outputRow[nt] * outputs.strides_[0]) =
+                        make_float2(static_cast<float>(xOut[nt][0][0]), static_cast<float>(xOut[nt][0][1]));
                 }
             }
         } else {
