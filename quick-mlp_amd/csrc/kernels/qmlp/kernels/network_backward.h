@@ -104,7 +104,7 @@ $$ZERO_LDS_GRADIENTS$$
     const int actualChannelsOut = adjOutputs.sizes_[1];
     const bool adjOutputRowsOfFloat2 = actualChannelsOut == 2 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 2 == 0
         && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 8 == 0;
-    const bool adjOutputRowsOfFloat4 = actualChannelsOut == 4 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 4 == 0
+    const bool adjOutputRowsOfFloat4 = actualChannelsOut % 4 == 0 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 4 == 0
         && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 16 == 0;
     for (int tileBase = blockIdx.x * WAVES; tileBase < numTiles; tileBase += gridDim.x * WAVES)
     {
@@ -122,25 +122,26 @@ $$ZERO_LDS_GRADIENTS$$
             const bool pv = p < numel;
             validMask |= pv ? (1 << nt) : 0;
             if (adjOutputRowsOfFloat2 || adjOutputRowsOfFloat4) {
-                // two or four channels side by side in memory: one load per point (lane group 0
-                // holds channels 0..3 of its points, everything else is zero)
+                // channels side by side in memory: four per load (a lane holds channels
+                // 16m+4g .. +3 of its points), a row of two channels as one 8-byte load
+                const float* row = adjOutputs.data_ + static_cast<long long>(p) * adjOutputs.strides_[0];
 #pragma unroll
-                for (int m = 0; m < MTL; ++m)
+                for (int m = 0; m < MTL; ++m) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) dyOut[nt][m][i] = static_cast<f16>(0);
-                if (pv && g == 0) {
-                    const float* row = adjOutputs.data_ + static_cast<long long>(p) * adjOutputs.strides_[0];
-                    if (adjOutputRowsOfFloat4) {
-                        const float4 v = *reinterpret_cast<const float4*>(row);
-                        dyOut[nt][0][0] = static_cast<f16>(v.x);
-                        dyOut[nt][0][1] = static_cast<f16>(v.y);
-                        dyOut[nt][0][2] = static_cast<f16>(v.z);
-                        dyOut[nt][0][3] = static_cast<f16>(v.w);
-                    } else {
-                        const float2 v = *reinterpret_cast<const float2*>(row);
-                        dyOut[nt][0][0] = static_cast<f16>(v.x);
-                        dyOut[nt][0][1] = static_cast<f16>(v.y);
+                    const int c = 16 * m + 4 * g;
+                    if (adjOutputRowsOfFloat4 && pv && c < actualChannelsOut) {
+                        const float4 v = *reinterpret_cast<const float4*>(row + c);
+                        dyOut[nt][m][0] = static_cast<f16>(v.x);
+                        dyOut[nt][m][1] = static_cast<f16>(v.y);
+                        dyOut[nt][m][2] = static_cast<f16>(v.z);
+                        dyOut[nt][m][3] = static_cast<f16>(v.w);
                     }
+                }
+                if (!adjOutputRowsOfFloat4 && pv && g == 0) {
+                    const float2 v = *reinterpret_cast<const float2*>(row);
+                    dyOut[nt][0][0] = static_cast<f16>(v.x);
+                    dyOut[nt][0][1] = static_cast<f16>(v.y);
                 }
             } else {
 #pragma unroll
@@ -185,17 +186,20 @@ $$CALL_ENCODINGS$$
 
                 if constexpr (HAS_INPUT_GRADIENTS) {
                     float* adjRow = adjInputs.data_ + static_cast<long long>(index) * adjInputs.strides_[0];
-                    if (!HAS_ENCODING_GRADIENTS && NUM_INPUTS == 4 && adjInputs.strides_[1] == 1 && adjInputs.strides_[0] % 4 == 0
+                    if (!HAS_ENCODING_GRADIENTS && NUM_INPUTS % 4 == 0 && adjInputs.strides_[1] == 1 && adjInputs.strides_[0] % 4 == 0
                         && reinterpret_cast<unsigned long long>(adjInputs.data_) % 16 == 0) {
-                        // the four channels of a row side by side: one load and one store. Kept to
+                        // the channels of a row side by side: four per load and store. Kept to
                         // kernels without a grid scatter: in front of the gradient atomics of a grid
                         // no gain was measurable.
-                        float4 v = *reinterpret_cast<float4*>(adjRow);
-                        v.x += adjEncodingInput[0];
-                        v.y += adjEncodingInput[NUM_INPUTS > 1 ? 1 : 0];
-                        v.z += adjEncodingInput[NUM_INPUTS > 2 ? 2 : 0];
-                        v.w += adjEncodingInput[NUM_INPUTS > 3 ? 3 : 0];
-                        *reinterpret_cast<float4*>(adjRow) = v;
+#pragma unroll
+                        for (int i = 0; i + 3 < NUM_INPUTS; i += 4) {
+                            float4 v = *reinterpret_cast<float4*>(adjRow + i);
+                            v.x += adjEncodingInput[i];
+                            v.y += adjEncodingInput[i + 1];
+                            v.z += adjEncodingInput[i + 2];
+                            v.w += adjEncodingInput[i + 3];
+                            *reinterpret_cast<float4*>(adjRow + i) = v;
+                        }
                     } else {
 #pragma unroll
                         for (int i = 0; i < NUM_INPUTS; ++i)
