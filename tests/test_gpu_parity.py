@@ -745,3 +745,48 @@ def test_inference_sorted_by_grid_slab_gives_the_same_bits_as_the_order_given():
     a = sorted_.net.inference(view, sorted_.params, sorted_.encoding_parameters())
     b = plain.net.inference(view.contiguous(), plain.params, plain.encoding_parameters())
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("n_in,n_out", [(4, 4), (2, 2), (8, 16), (4, 2), (3, 1)])
+def test_rows_moved_as_vectors_and_rows_that_cannot_be(n_in, n_out):
+    """Input, output, dL/dy and input-gradient rows whose channels lie side by side move 8 or 16
+    bytes at a time; rows that start at an address that is not a multiple of that, or whose
+    row stride is not, have to take the scalar path and give the same bits. Both against the
+    oracle, ragged batch."""
+    case = Case(identity_cfg(n_in, [32, n_out], ["relu", "identity"], [True, True]))
+    rng = np.random.default_rng(21)
+    case.set_parameters(random_parameters(case.oracle, rng))
+    N = 64 * 5 + 13
+    X = rng.uniform(-1, 1, (N, n_in)).astype(np.float32)
+    adj = rng.uniform(-1, 1, (N, n_out)).astype(np.float32)
+
+    def shifted(a, pad):
+        """The same rows in memory that starts 4 bytes off and has `pad` more floats per row."""
+        n, c = a.shape
+        flat = torch.zeros(1 + n * (c + pad), device="cuda")
+        view = flat[1:].view(n, c + pad)[:, :c]
+        view.copy_(torch.from_numpy(a))
+        return view
+
+    x0 = torch.from_numpy(X).cuda()
+    a0 = torch.from_numpy(adj).cuda()
+    ref_out = case.oracle.forward(X)
+    results = []
+    for pad in (None, 0, 1):
+        x = x0 if pad is None else shifted(X, pad)
+        a = a0 if pad is None else shifted(adj, pad)
+        assert (x.data_ptr() % 16 == 0) == (pad is None)
+        out = case.net.inference(x, case.params, [])
+        out2, tmp = case.net.forward_raw(x, case.params, [], 3)
+        adj_in = torch.zeros((N, n_in), device="cuda") if pad is None else shifted(np.zeros((N, n_in), np.float32), pad)
+        gnet = torch.zeros((case.net.num_network_parameters(),), device="cuda")
+        case.net.adjoint_raw(x, a, 3, tmp, case.params, [], grad_network=gnet, adj_input=adj_in)
+        torch.cuda.synchronize()
+        results.append((out.cpu().numpy(), out2.cpu().numpy(), adj_in.cpu().numpy().copy(), gnet.cpu().numpy()))
+    assert_close(results[0][0], ref_out, "inference")
+    check_gradients(case, X, adj, 3, dict(adj_x=results[0][2], grads=results[0][3]), kinks=True)
+    for other in results[1:]:
+        for k in range(3):
+            assert np.array_equal(results[0][k], other[k]), k
+        s = float(np.abs(results[0][3]).max())
+        assert_close(other[3] / s, results[0][3] / s, "weight gradients", rel=1e-3, abs_=1e-5)
