@@ -790,3 +790,33 @@ def test_rows_moved_as_vectors_and_rows_that_cannot_be(n_in, n_out):
             assert np.array_equal(results[0][k], other[k]), k
         s = float(np.abs(results[0][3]).max())
         assert_close(other[3] / s, results[0][3] / s, "weight gradients", rel=1e-3, abs_=1e-5)
+
+
+def test_sorted_inference_of_a_two_level_dense_grid_in_several_launches():
+    """Two dense 3-D levels (8 and 17 MB) are swept one after the other, so a long batch is cut
+    into several launches; sorted by slab, every launch takes its stretch of the sorted rows and
+    writes through its stretch of the order. Same bits as the batch evaluated as given, and a
+    sample against the oracle."""
+    grid = {"id": "HashGrid", "start_in": 0, "n_in": 3, "n_levels": 2, "n_features_per_level": 2,
+            "log2_hashmap_size": -1, "min_resolution": 128, "max_resolution": 161, "combination_mode": "concat",
+            "bounding_box_min": [-1.0, 0.0, 2.0], "bounding_box_size": [2.0, 1.0, 0.5], "parameter_precision": "half"}
+    cases = []
+    for mode in (1, 0):
+        cfg = {"num_inputs": 3, "num_outputs": 1, "activation_specification": ["qmlp/builtin-activations.json"],
+               "encodings": [grid], "options": {"sort_points": mode},
+               "network": [{"n_out": 16, "bias": True, "activation": "relu"}, {"n_out": 1, "bias": True, "activation": "identity"}]}
+        case = Case(cfg)
+        rng = np.random.default_rng(31)
+        case.set_parameters(random_parameters(case.oracle, rng))
+        case.set_table(0, rng.uniform(-1, 1, case.oracle.encodings[0][1].n_params).astype(np.float32))
+        cases.append(case)
+    sorted_, plain = cases
+    rng = np.random.default_rng(32)
+    N = (1 << 21) + (1 << 19) + 333
+    X = (rng.uniform(0, 1, (N, 3)) * np.array([2.0, 1.0, 0.5]) + np.array([-1.0, 0.0, 2.0])).astype(np.float32)
+    print("sorted, several launches: %d points" % N, flush=True)
+    a, b = sorted_.gpu_inference(X), plain.gpu_inference(X)
+    assert np.array_equal(a, b) and np.abs(a).max() > 0.05
+    sample = np.arange(0, N, 5003)
+    ref = sorted_.oracle.forward(X[sample])
+    assert_close(a[sample], ref, "sampled oracle check", allowed_fraction=2e-3)
