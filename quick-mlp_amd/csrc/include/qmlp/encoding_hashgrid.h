@@ -74,7 +74,7 @@ public:
     [[nodiscard]] int ldsGradientFloats(int maxBytes, int& levels) const override;
     [[nodiscard]] int numSweptTables() const override { return numLevels_; }
     [[nodiscard]] int gatherRegistersPerPoint() const override;
-    [[nodiscard]] bool pointOrderKey(kernel::PointOrderKey& key) const override;
+    [[nodiscard]] bool pointOrderKey(kernel::PointOrderKey& key, long long numPoints = 0) const override;
     [[nodiscard]] int channelsWrittenTogether() const override { return numFeaturesPerLevel_; }
     void setParameter(const Tensor& tensor, Tensor::Usage usage) override;
     [[nodiscard]] int fillParameterMemory(char* dst, int dstSize) override;

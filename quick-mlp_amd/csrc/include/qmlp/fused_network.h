@@ -124,8 +124,8 @@ private:
         long long capacity = 0;     // points the workspace holds
     };
     PointOrder pointOrder_;
-    /** Batches of at least this many points are sorted when sortPoints < 0. */
-    static constexpr int SORT_POINTS_MIN_BATCH = 1 << 20;
+    /** Smaller batches are never sorted when sortPoints < 0; larger ones if the encoding expects a gain. */
+    static constexpr int SORT_POINTS_MIN_BATCH = 1 << 19;
     /**
      * Sorts the batch by the slab key of the first encoding that offers one.
      * \return false if the batch stays as it is; else sortedInput views the sorted copy and

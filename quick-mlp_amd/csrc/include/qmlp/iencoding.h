@@ -104,10 +104,13 @@ public:
      * gathers are close in memory for points that are close in space (dense grids), fill in how
      * points are assigned to slabs of that table and return true: the fused inference kernel
      * then evaluates the points slab by slab.
+     * \param numPoints size of the batch; >0: only say yes if so many points are also expected
+     *   to gain more from the order than the sort costs. 0: say whether an order exists at all.
      */
-    [[nodiscard]] virtual bool pointOrderKey(kernel::PointOrderKey& key) const
+    [[nodiscard]] virtual bool pointOrderKey(kernel::PointOrderKey& key, long long numPoints = 0) const
     {
         (void)key;
+        (void)numPoints;
         return false;
     }
 

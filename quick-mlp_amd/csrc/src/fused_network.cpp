@@ -1183,7 +1183,7 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     kernel::PointOrderKey key{};
     bool found = false;
     for (const auto& e : encodings_)
-        if (e->pointOrderKey(key)) {
+        if (e->pointOrderKey(key, compileOptions_.sortPoints < 0 ? numel : 0)) {
             found = true;
             break;
         }
