@@ -77,6 +77,10 @@ public:
     [[nodiscard]] bool pointOrderKey(kernel::PointOrderKey& key, long long numPoints = 0) const override;
     [[nodiscard]] int channelsWrittenTogether() const override { return numFeaturesPerLevel_; }
     void setParameter(const Tensor& tensor, Tensor::Usage usage) override;
+    [[nodiscard]] bool hasParameterTensor(Tensor::Usage usage) const override
+    {
+        return usage == Tensor::INFERENCE ? parametersForward_.defined() : parametersGradients_.defined();
+    }
     [[nodiscard]] int fillParameterMemory(char* dst, int dstSize) override;
     void zeroGradients() override;
 

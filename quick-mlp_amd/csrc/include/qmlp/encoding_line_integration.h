@@ -50,6 +50,7 @@ public:
     [[nodiscard]] Tensor::Precision parameterPrecision(Tensor::Usage usage) const override;
     [[nodiscard]] int parameterCount() const override;
     void setParameter(const Tensor& tensor, Tensor::Usage usage) override;
+    [[nodiscard]] bool hasParameterTensor(Tensor::Usage usage) const override { return volume_->hasParameterTensor(usage); }
     [[nodiscard]] int fillParameterMemory(char* dst, int dstSize) override;
     void zeroGradients() override;
 

@@ -287,6 +287,8 @@ private:
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */
+    /** Throws unless every encoding with parameters has a tensor bound for 'usage'. */
+    void checkEncodingParameters(Tensor::Usage usage) const;
     void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 

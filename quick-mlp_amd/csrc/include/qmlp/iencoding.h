@@ -70,6 +70,9 @@ public:
      */
     virtual void setParameter(const Tensor& tensor, Tensor::Usage usage) {}
 
+    /** True iff a tensor is currently bound for this usage (always true without parameters). */
+    [[nodiscard]] virtual bool hasParameterTensor(Tensor::Usage usage) const { return true; }
+
     /**
      * Writes the bytes of the parameter structure (kernel argument) into 'dst' with a
      * capacity of 'dstSize' bytes; returns the number of bytes written.

@@ -1132,6 +1132,19 @@ void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t strea
     CHECK_DIM(output, 2);
     CHECK_SIZE(input, 1, channelsIn());
     CHECK_SIZE(output, 1, channelsOut());
+void FusedNetwork::checkEncodingParameters(Tensor::Usage usage) const
+{
+    for (size_t i = 0; i < encodings_.size(); ++i) {
+        if (!encodings_[i]->hasParameters() || encodings_[i]->hasParameterTensor(usage)) continue;
+        if (usage == Tensor::INFERENCE)
+            throw std::runtime_error(format("Encoding %d has parameters, but no inference tensor is bound to it: call "
+                                            "encoding(%d)->setParameter(tensor, INFERENCE) first", int(i), int(i)));
+        throw std::runtime_error(format("Encoding gradients requested, but encoding %d has no gradient tensor: call "
+                                        "encoding(%d)->setParameter(tensor, GRADIENTS) for every encoding with parameters",
+                                        int(i), int(i)));
+    }
+}
+
     int numel = input.size(0);
     CHECK_SIZE(output, 0, numel);
     CHECK_DTYPE(input, precisionIn());
@@ -1143,6 +1156,7 @@ void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t strea
 }
 
 void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream)
+    checkEncodingParameters(Tensor::INFERENCE);
 {
     const int numel = input.size(0);
     int tmpNumTiles = divUp(numel, TILE_POINTS);
@@ -1315,6 +1329,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
 
     const bool hasInputGradients = adjointFlags & GRADIENTS_INPUT;
     const bool hasNetworkGradients = adjointFlags & GRADIENTS_NETWORK_WEIGHTS;
+    checkEncodingParameters(Tensor::INFERENCE);
     const bool hasEncodingGradients = adjointFlags & GRADIENTS_INPUT_ENCODINGS;
 
     if (hasInputGradients) {
@@ -1336,7 +1351,6 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         CHECK_ERROR(tmpMemoryAdjoint != nullptr, "adjoint() needs temporary memory of adjointMemory() bytes");
         CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemoryAdjoint) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
     }
-    (void)hasEncodingGradients;
 
     compileBackwardKernel(adjointFlags);
     auto& ak = backwardKernel_[adjointFlags].value();
@@ -1382,6 +1396,9 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     if (!hasNetworkGradients) return;
 
     const bool parallel = compileOptions_.parallelWeightUpdate && layers_.size() > 1;
+    checkEncodingParameters(Tensor::INFERENCE);
+    // the kernel adds the gradients of every encoding that has parameters: each needs a tensor to add into
+    if (hasEncodingGradients) checkEncodingParameters(Tensor::GRADIENTS);
     if (parallel) {
         ensureStreams();
         QMLP_HIP_CALL(qmlp_hip_event_record(adjointEvent_, stream));

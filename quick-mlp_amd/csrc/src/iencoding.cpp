@@ -89,6 +89,9 @@ void IEncoding::forward(const Tensor& input, Tensor& output, stream_t stream,
     CHECK_ERROR(output.size(1) >= numOutputChannels());
     CHECK_ERROR(output.strides()[1] == 1, "The output stride along the channels must be 1");
     long long numel = input.size(0);
+    if (hasParameters())
+        CHECK_ERROR((parametersForward.has_value() && parametersForward.value().defined()) || hasParameterTensor(Tensor::INFERENCE),
+                    "The encoding has parameters, but no inference tensor is bound or passed");
     if (numel == 0) return;
 
     if (!forwardKernel_.has_value())
@@ -131,6 +134,13 @@ void IEncoding::adjoint(const Tensor& input, const Tensor& adjOutput, Tensor& ad
     CHECK_ERROR(adjInput.size(1) == input.size(1));
     CHECK_ERROR(adjointMode >= 1 && adjointMode <= ALL_GRADIENTS, "Illegal adjoint mode");
     long long numel = input.size(0);
+    if (hasParameters()) {
+        CHECK_ERROR((parametersForward.has_value() && parametersForward.value().defined()) || hasParameterTensor(Tensor::INFERENCE),
+                    "The encoding has parameters, but no inference tensor is bound or passed");
+        CHECK_ERROR(!(adjointMode & PARAM_GRADIENTS) || (parametersGradients.has_value() && parametersGradients.value().defined())
+                        || hasParameterTensor(Tensor::GRADIENTS),
+                    "Parameter gradients requested, but no gradient tensor is bound or passed");
+    }
     if (numel == 0) return;
 
     if (!adjointKernel_[adjointMode].has_value())

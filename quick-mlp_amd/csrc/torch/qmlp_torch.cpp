@@ -459,7 +459,9 @@ struct NetworkFunction : torch::autograd::Function<NetworkFunction>
             }
             if (flags & QMLP_GRADIENTS_INPUT_ENCODINGS) {
                 for (size_t i = 0; i < encodingParameters.size(); ++i) {
-                    if (!net->encodingHasParameters(static_cast<int64_t>(i)) || !needs[i]) continue;
+                    // the kernel adds the gradients of every encoding with parameters: a frozen one gets a
+                    // zero tensor as well, which is dropped afterwards (bind_network.cpp:277-290)
+                    if (!net->encodingHasParameters(static_cast<int64_t>(i))) continue;
                     int precision = QMLP_FLOAT;
                     QMLP_CHECK(qmlp_encoding_parameter_precision(net->encodingHandle(static_cast<int64_t>(i)), QMLP_GRADIENTS, &precision));
                     adjEncodings[i] = torch::zeros(encodingParameters[i].sizes(), encodingParameters[i].options().dtype(dtypeOf(precision)));
@@ -484,7 +486,8 @@ struct NetworkFunction : torch::autograd::Function<NetworkFunction>
         if (adjNetwork.defined()) adjNetwork = adjNetwork.to(paramDtype);
         torch::autograd::variable_list grads = {torch::Tensor(), torch::Tensor(), adjInput, adjNetwork};
         for (size_t i = 0; i < adjEncodings.size(); ++i)
-            grads.push_back(adjEncodings[i].defined() ? adjEncodings[i].to(encodingParameters[i].scalar_type()) : torch::Tensor());
+            grads.push_back(adjEncodings[i].defined() && needs[i] ? adjEncodings[i].to(encodingParameters[i].scalar_type())
+                                                                   : torch::Tensor());
         return grads;
     }
 };

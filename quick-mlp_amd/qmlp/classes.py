@@ -247,6 +247,8 @@ class Encoding:
         output = _create_output(input, self.num_output_channels())
         check(lib.qmlp_encoding_forward(self._handle, desc(input), desc(output), current_stream(input.device),
                                         desc(parameter_forward)))
+        # the native call binds the table for its own duration and leaves the encoding unbound
+        self._bound_inference = None
         return output
 
     def adjoint(self, input, adj_output):
@@ -269,6 +271,7 @@ class Encoding:
         check(lib.qmlp_encoding_adjoint(self._handle, desc(input), desc(adj_output), desc(adj_input),
                                         current_stream(input.device), desc(parameter_forward), desc(adj_param),
                                         int(flags)))
+        self._bound_inference = None   # as in inference_with_parameter
         return adj_input, adj_param.to(parameter_forward.dtype)
 
     def forward(self, input):
@@ -325,7 +328,9 @@ class _NetworkFunction(torch.autograd.Function):
             if flags & GRADIENTS_INPUT_ENCODINGS:
                 for i, p in enumerate(encoding_parameters):
                     enc = net.encoding(i)
-                    if enc.has_parameters() and ctx.needs_input_grad[4 + i]:
+                    # the kernel adds the gradients of every encoding with parameters: a frozen one
+                    # gets a zero tensor as well, which is dropped below (bind_network.cpp:277-290)
+                    if enc.has_parameters():
                         adj_encodings[i] = torch.zeros(p.shape, dtype=enc.parameter_dtype(True), device=p.device)
                         enc.set_parameter(adj_encodings[i], gradients=True)
             nbytes = net.adjoint_memory(input.shape[0], flags)
@@ -340,7 +345,8 @@ class _NetworkFunction(torch.autograd.Function):
                     net.encoding(i).set_parameter(None, gradients=True)
         if adj_network is not None:
             adj_network = adj_network.to(ctx.param_dtype)
-        adj_encodings = [g.to(p.dtype) if g is not None else None for g, p in zip(adj_encodings, encoding_parameters)]
+        adj_encodings = [g.to(p.dtype) if g is not None and ctx.needs_input_grad[4 + i] else None
+                         for i, (g, p) in enumerate(zip(adj_encodings, encoding_parameters))]
         return (None, None, adj_input, adj_network, *adj_encodings)
 
 

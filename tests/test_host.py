@@ -365,3 +365,71 @@ def test_kernel_cache_key_covers_only_the_headers_a_source_includes(tmp_path):
     with open(kernels / "qmlp" / "kernels" / "common.h", "a") as f:
         f.write("\n// edited\n")
     assert run() == (12, 0)                      # everything includes common.h
+
+
+def _two_grid_cfg():
+    grid = dict(bc.hashgrid3d("float"), n_levels=2, log2_hashmap_size=8, min_resolution=4, max_resolution=16)
+    return {"num_inputs": 3, "num_outputs": 1, "activation_specification": [bc.BUILTIN],
+            "encodings": [grid, dict(grid, n_levels=3)],
+            "network": [{"n_out": 16, "bias": False, "activation": "relu"},
+                        {"n_out": 1, "bias": False, "activation": "identity"}]}
+
+
+def test_unbound_encoding_tensors_are_refused_before_any_launch():
+    """A network call with a grid whose table (or, with encoding gradients, whose gradient
+    tensor) is not bound must raise instead of handing a null pointer to the kernel. The
+    checks come before compilation and launch, so host tensors stand in for device memory."""
+    from qmlp._lib import check, desc, lib
+    net = qmlp.Network(json.dumps(_two_grid_cfg()))
+    n = 64
+    x, y = torch.zeros(n, 3), torch.zeros(n, 1)
+    params = torch.zeros(net.num_network_parameters(), dtype=torch.float16)
+    tables = [torch.zeros(net.encoding(i).num_parameters()) for i in range(2)]
+    tmp = torch.zeros(1 << 20, dtype=torch.uint8)
+    check(lib.qmlp_network_set_parameter(net._handle, desc(params), 0))
+
+    def inference():
+        check(lib.qmlp_network_inference(net._handle, desc(x), desc(y), None))
+
+    def forward():
+        check(lib.qmlp_network_forward(net._handle, desc(x), desc(y), ctypes.c_void_p(tmp.data_ptr()), None))
+
+    def adjoint(flags):
+        check(lib.qmlp_network_adjoint(net._handle, desc(x), desc(y), flags, desc(torch.zeros(n, 3)),
+                                       ctypes.c_void_p(tmp.data_ptr()), ctypes.c_void_p(tmp.data_ptr()), None))
+
+    for call in (inference, forward, lambda: adjoint(1)):
+        with pytest.raises(qmlp.QmlpError, match="Encoding 0 has parameters, but no inference tensor"):
+            call()
+    net.encoding(0).set_parameter(tables[0])
+    with pytest.raises(qmlp.QmlpError, match="Encoding 1 has parameters, but no inference tensor"):
+        inference()
+    net.encoding(1).set_parameter(tables[1])
+    # one grid trainable, one frozen: the kernel adds into both gradient tables
+    net.encoding(0).set_parameter(torch.zeros_like(tables[0]), gradients=True)
+    with pytest.raises(qmlp.QmlpError, match="encoding 1 has no gradient tensor"):
+        adjoint(4)
+    with pytest.raises(qmlp.QmlpError, match="encoding 1 has no gradient tensor"):
+        adjoint(5)
+
+    # standalone encoding: no table bound or passed
+    enc = qmlp.Encoding(json.dumps(_two_grid_cfg()["encodings"][0]))
+    out = torch.zeros(n, enc.num_output_channels())
+    with pytest.raises(qmlp.QmlpError, match="no inference tensor is bound or passed"):
+        check(lib.qmlp_encoding_forward(enc._handle, desc(x), desc(out), None, None))
+    with pytest.raises(qmlp.QmlpError, match="no gradient tensor is bound or passed"):
+        check(lib.qmlp_encoding_adjoint(enc._handle, desc(x), desc(out), desc(torch.zeros(n, 3)), None,
+                                        desc(tables[0]), None, 3))
+
+
+def test_the_python_binding_cache_forgets_a_table_the_standalone_call_unbound():
+    """Encoding.set_parameter skips binding the same memory twice; the standalone
+    *_with_parameter calls leave the native encoding unbound, so they must reset that memory."""
+    enc = qmlp.Encoding(json.dumps(_two_grid_cfg()["encodings"][0]))
+    t = torch.zeros(enc.num_parameters())
+    enc.set_parameter(t)
+    assert enc._bound_inference is not None
+    src = open(os.path.join(ROOT, "quick-mlp_amd", "qmlp", "classes.py")).read()
+    for name in ("inference_with_parameter", "adjoint_with_parameter_and_flags"):
+        body = src.split("def %s(" % name)[1].split("\n    def ")[0]
+        assert "self._bound_inference = None" in body, name

@@ -351,3 +351,72 @@ def test_inference_and_train_step_replay_from_a_hip_graph():
         assert torch.equal(got[2], want[2]), "weight gradients of replay %d" % replay
         assert torch.allclose(got[3], want[3], rtol=1e-4, atol=1e-6), "grid gradients of replay %d" % replay
         assert torch.allclose(got[4], want[4], rtol=1e-5, atol=1e-7), "input gradients of replay %d" % replay
+
+
+def two_grid_cfg():
+    grid = {"id": "HashGrid", "start_in": 0, "n_in": 2, "n_levels": 2, "n_features_per_level": 4,
+            "log2_hashmap_size": 10, "min_resolution": 8, "max_resolution": 64, "combination_mode": "concat",
+            "bounding_box_min": [-1.0, -1.0], "bounding_box_size": [2.0, 2.0]}
+    return json.dumps({"num_inputs": 2, "num_outputs": 3,
+                       "activation_specification": ["qmlp/builtin-activations.json"],
+                       "encodings": [grid, dict(grid, n_levels=2, min_resolution=5, max_resolution=9)],
+                       "network": [{"n_out": 32, "bias": True, "activation": "celu"},
+                                   {"n_out": 3, "bias": False, "activation": "identity"}]})
+
+
+@pytest.mark.parametrize("scriptable", [False, True])
+@pytest.mark.parametrize("frozen", [0, 1])
+def test_two_grids_one_of_them_frozen(scriptable, frozen):
+    """Encoding gradients with one trainable and one frozen grid: the kernel adds the gradients
+    of every grid, so the frozen one gets a throw-away tensor (bind_network.cpp:277-290). The
+    trainable grid's gradient equals the one of the run where both are trainable, the frozen
+    one has none."""
+    cfg = two_grid_cfg()
+    warm_or_gpu(network_cfg=cfg)
+    torch.manual_seed(5)
+    net = FusedNetwork(cfg, weight_dtype=torch.float32, scriptable=scriptable)
+    for p in net.encoding_parameters:
+        p.data.uniform_(-1, 1)
+    x = torch.rand((3000, 2), device="cuda") * 2 - 1
+    target = torch.randn((3000, 3), device="cuda")
+
+    def grads(frozen_index):
+        for i, p in enumerate(net.encoding_parameters):
+            p.requires_grad_(i != frozen_index)
+            p.grad = None
+        net.weights.grad = None
+        torch.nn.functional.mse_loss(net(x), target).backward()
+        return [None if p.grad is None else p.grad.clone() for p in net.encoding_parameters], net.weights.grad.clone()
+
+    both, w_both = grads(-1)
+    got, w_got = grads(frozen)
+    assert got[frozen] is None
+    live = 1 - frozen
+    assert float(both[live].abs().sum()) > 0
+    # float atomics: the order of the additions differs between runs
+    assert torch.allclose(got[live], both[live], rtol=1e-4, atol=1e-6)
+    assert torch.equal(w_got, w_both)
+
+
+def test_network_call_after_a_standalone_call_of_its_encoding():
+    """net.inference -> net.encoding(0) called on its own with the same table -> net.inference:
+    the standalone call leaves the native encoding unbound, the network call has to bind the
+    table again."""
+    cfg = two_grid_cfg()
+    if WARM:
+        e = json.loads(cfg)["encodings"][0]
+        warm_or_gpu(network_cfg=cfg, encoding_cfg=json.dumps(e))
+    warm_or_gpu()
+    net = qmlp.Network(cfg)
+    torch.manual_seed(6)
+    params = torch.randn(net.num_network_parameters(), device="cuda").half() / 4
+    tables = [torch.rand(net.encoding(i).num_parameters(), device="cuda") for i in range(2)]
+    x = torch.rand((777, 2), device="cuda") * 2 - 1
+    first = net.inference(x, params, tables)
+    alone = net.encoding(0).inference_with_parameter(x, tables[0])
+    assert alone.shape == (777, 8)
+    again = net.inference(x, params, tables)
+    assert torch.equal(first, again)
+    gi, gp = net.encoding(0).adjoint_with_parameter(x, tables[0], torch.ones_like(alone))
+    assert gp.shape == tables[0].shape
+    assert torch.equal(first, net.inference(x, params, tables))
