@@ -91,6 +91,19 @@ int qmlp_network_parameter_view(qmlp_network_t network, int layer, int bias, voi
 /* inference(input, output, stream), :229 */
 int qmlp_network_inference(qmlp_network_t network, const qmlp_tensor* input, const qmlp_tensor* output,
                            void* stream);
+/* qmlp_network_inference for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart in the
+ * reference. Same arguments and the same results bit for bit, but no call on its way
+ * allocates or frees: the workspace in which a batch is ordered by grid slab (networks with a
+ * large dense grid; qmlp_network_inference keeps one per network and allocates it on demand)
+ * is a static device buffer of 48 MiB per GPU, and kernels are only used if they are
+ * loaded already. So: run qmlp_network_inference once on a batch of the same size first
+ * (that compiles and loads the kernels and resolves the buffer on this GPU). Errors:
+ * a batch whose order needs more than the buffer (20.5 bytes per point at 4 input channels:
+ * about 2.4 million points), kernels that are not loaded yet. All calls on one GPU share the
+ * buffer, whose contents are not kept between calls: calls that overlap in time race. */
+int qmlp_network_inference_noalloc(qmlp_network_t network, const qmlp_tensor* input, const qmlp_tensor* output,
+                                   void* stream);
 /* forwardMemory(numElements, flags), :240 */
 int qmlp_network_forward_memory(qmlp_network_t network, int num_elements, int adjoint_flags, size_t* bytes);
 /* forward(input, output, tmpMemory, stream), :263 */

@@ -131,7 +131,8 @@ private:
      * \return false if the batch stays as it is; else sortedInput views the sorted copy and
      *   order holds, per row of it, the row of the caller's batch
      */
-    bool sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream);
+    bool sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
+                    bool noAlloc = false);
 
     struct AdjointLayerInfo
     {
@@ -227,6 +228,18 @@ public:
      */
     void inference(const Tensor& input, Tensor& output, stream_t stream);
 
+    /**
+     * inference() for callers that cannot allocate device memory (code under HIP graph
+     * capture, tight serving loops): same results, but nothing on the way allocates.
+     * The workspace that orders a batch by grid slab is the library's static device buffer
+     * of QMLP_STATIC_SCRATCH_BYTES per GPU instead of the network's own: a batch that
+     * needs more is refused. Kernels are only taken if they are loaded already, so
+     * inference() has to have run once on a batch of the same size. All calls on one GPU
+     * share the buffer: calls that overlap in time (other streams, other networks) race.
+     * No counterpart in the reference.
+     */
+    void inferenceNoAlloc(const Tensor& input, Tensor& output, stream_t stream);
+
     /** Bytes of temporary memory forward() needs for 'numElements' points. */
     size_t forwardMemory(int numElements, AdjointModeFlags adjointFlags);
     size_t forwardMemory(const Tensor& input, AdjointModeFlags adjointFlags);
@@ -283,13 +296,13 @@ private:
      * how many of them that launch should take (whole steps of a large shape first; the caller
      * asks again for the rest).
      */
-    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr);
+    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr, bool noAlloc = false);
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */
     /** Throws unless every encoding with parameters has a tensor bound for 'usage'. */
     void checkEncodingParameters(Tensor::Usage usage) const;
-    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream);
+    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false);
     void compileBackwardKernel(int flags, bool compileOnly = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false) const;

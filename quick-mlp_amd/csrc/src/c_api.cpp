@@ -286,6 +286,14 @@ int qmlp_network_inference(qmlp_network_t network, const qmlp_tensor* input, con
     QMLP_API_END
 }
 
+int qmlp_network_inference_noalloc(qmlp_network_t network, const qmlp_tensor* input, const qmlp_tensor* output, void* stream)
+{
+    QMLP_API_BEGIN
+    Tensor out = wrap(output);
+    network->network->inferenceNoAlloc(wrap(input), out, static_cast<stream_t>(stream));
+    QMLP_API_END
+}
+
 int qmlp_network_forward_memory(qmlp_network_t network, int num_elements, int adjoint_flags, size_t* bytes)
 {
     QMLP_API_BEGIN

@@ -1,4 +1,5 @@
 #include <qmlp/fused_network.h>
+#include <qmlp/device_code.h>
 
 #include <qmlp/encoding_identity.h>
 #include <qmlp/qmlp.h>
@@ -940,17 +941,22 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
     slot = std::move(ck);
 }
 
-const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles)
+const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles, bool noAlloc)
 {
     const int s = store ? 1 : 0;
+    // loading a kernel allocates device memory: a call that must not allocate only takes what is loaded
+    auto loaded = [&](int variant) -> const CompiledKernel& {
+        if (noAlloc && !forwardKernels_[s][variant].has_value())
+            throw std::runtime_error("The kernel for a batch of this size is not loaded yet, and loading allocates: run "
+                                     "inference() once on a batch of the same size first");
+        compileForwardKernel(store, variant);
+        return forwardKernels_[s][variant].value();
+    };
     if (launchTiles) *launchTiles = numTiles;
     {
         int blockSize = 0, pointsPerLane = 1;
         forwardShape(store, VARIANT_DEFAULT, blockSize, pointsPerLane);
-        if (pointsPerLane == 1) {   // no gathers, or a pinned shape: one kernel
-            compileForwardKernel(store, VARIANT_DEFAULT);
-            return forwardKernels_[s][VARIANT_DEFAULT].value();
-        }
+        if (pointsPerLane == 1) return loaded(VARIANT_DEFAULT);   // no gathers, or a pinned shape: one kernel
     }
     // Kernels that take more tiles per wave are faster per point, but the time grows in steps
     // of one workgroup per compute unit, whether all compute units have one or not. Measured on
@@ -1000,14 +1006,14 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
             if (launchTiles) *launchTiles = static_cast<int>(steps * sh.stepTiles);
         }
     }
-    compileForwardKernel(store, best);
+    loaded(best);
     if (best == VARIANT_REGISTERS && forwardKernels_[s][best].value().fun.scratchBytes() > MAX_REGISTER_SHAPE_SCRATCH) {
         // the compiler did not get the rows and the gathers into the registers: a kernel that
         // spills this much is slower than the shapes that stage in LDS
         QuickMLP::Instance().getLogger()->debug("the forward kernel with rows in registers spills %d bytes per lane, not used",
                                                 forwardKernels_[s][best].value().fun.scratchBytes());
         registerShapeSpills_[s] = true;
-        return forwardKernelFor(store, numTiles, launchTiles);
+        return forwardKernelFor(store, numTiles, launchTiles, noAlloc);
     }
     return forwardKernels_[s][best].value();
 }
@@ -1126,12 +1132,6 @@ std::vector<char> FusedNetwork::encodingArguments(std::vector<void*>& args, std:
     return {};
 }
 
-void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t stream)
-{
-    CHECK_DIM(input, 2);
-    CHECK_DIM(output, 2);
-    CHECK_SIZE(input, 1, channelsIn());
-    CHECK_SIZE(output, 1, channelsOut());
 void FusedNetwork::checkEncodingParameters(Tensor::Usage usage) const
 {
     for (size_t i = 0; i < encodings_.size(); ++i) {
@@ -1145,18 +1145,41 @@ void FusedNetwork::checkEncodingParameters(Tensor::Usage usage) const
     }
 }
 
+void FusedNetwork::inference(const Tensor& input, Tensor& output, stream_t stream)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(output, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    CHECK_SIZE(output, 1, channelsOut());
     int numel = input.size(0);
     CHECK_SIZE(output, 0, numel);
     CHECK_DTYPE(input, precisionIn());
     CHECK_DTYPE(output, precisionOut());
     CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
+    checkEncodingParameters(Tensor::INFERENCE);
     if (numel == 0) return;
 
     launchForward(false, input, output, nullptr, stream);
 }
 
-void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream)
+void FusedNetwork::inferenceNoAlloc(const Tensor& input, Tensor& output, stream_t stream)
+{
+    CHECK_DIM(input, 2);
+    CHECK_DIM(output, 2);
+    CHECK_SIZE(input, 1, channelsIn());
+    CHECK_SIZE(output, 1, channelsOut());
+    int numel = input.size(0);
+    CHECK_SIZE(output, 0, numel);
+    CHECK_DTYPE(input, precisionIn());
+    CHECK_DTYPE(output, precisionOut());
+    CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
     checkEncodingParameters(Tensor::INFERENCE);
+    if (numel == 0) return;
+
+    launchForward(false, input, output, nullptr, stream, true);
+}
+
+void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc)
 {
     const int numel = input.size(0);
     int tmpNumTiles = divUp(numel, TILE_POINTS);
@@ -1165,12 +1188,12 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     // inference of a network with a large dense grid: rows of the input sorted by grid slab,
     // every row of the result written where its point stands in the caller's batch
     const int* orderAll = nullptr;
-    const bool sorted = !store && sortPoints(input, inputAll, orderAll, stream);
+    const bool sorted = !store && sortPoints(input, inputAll, orderAll, stream, noAlloc);
     const half* networkParams = parametersInference_.dataPtr<half>();
     for (long long start = 0; start < numel;) {
         // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
         int launchTiles = 0;
-        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles);
+        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, noAlloc);
         int count = static_cast<int>(std::min<long long>(
             {static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS, numel - start}));
         auto inputAcc = inputAll;
@@ -1190,7 +1213,8 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     }
 }
 
-bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream)
+bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
+                              bool noAlloc)
 {
     const int numel = input.size(0);
     if (compileOptions_.sortPoints == 0 || (compileOptions_.sortPoints < 0 && numel < SORT_POINTS_MIN_BATCH)) return false;
@@ -1206,6 +1230,9 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     const int maxChannels = channels <= 4 ? 4 : channels <= 8 ? 8 : 16;
 
     auto& po = pointOrder_;
+    if (!po.scatter.has_value() && noAlloc)
+        throw std::runtime_error("The kernels that order the batch are not loaded yet, and loading allocates: run "
+                                 "inference() once on a batch of the same size first");
     if (!po.scatter.has_value()) {
         auto kl = QuickMLP::Instance().kernelLoader();
         const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
@@ -1214,16 +1241,43 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
         po.scatter = kl->getKernel("qmlp::kernel::PointOrderScatter<" + std::to_string(maxChannels) + ">", source, loaderFlags(false)).value();
     }
     constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 8 * BLOCK;   // as in point_order.h
-    if (po.capacity < numel) {
-        // words: sorted inputs, order, one histogram per chunk, totals
-        const long long words = static_cast<long long>(numel) * (channels + 1) + (divUp(numel, CHUNK) + 1ll) * SLABS;
-        if (words > std::numeric_limits<int32_t>::max()) return false;   // beyond one tensor: the batch stays as it is
-        po.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
-        po.capacity = numel;
+    // words: sorted inputs, order, totals, one histogram per chunk
+    const long long words = static_cast<long long>(numel) * (channels + 1) + (divUp(numel, CHUNK) + 1ll) * SLABS;
+    float* sortedData = nullptr;
+    long long capacity = numel;   // rows the workspace is laid out for
+    if (noAlloc) {
+        // the workspace is the library's static device buffer; the kernels get its address
+        // as the same arguments that otherwise point into the network's own workspace
+        void* scratch = nullptr;
+        size_t scratchBytes = 0;
+        std::string error;
+        if (device_code::staticScratch(&scratch, &scratchBytes, error) != 0) throw std::runtime_error(error);
+        if (static_cast<unsigned long long>(words) * sizeof(float) > scratchBytes)
+            throw std::runtime_error(format(
+                "A batch of %d points with %d channels needs %lld bytes to be ordered by grid slab; the call that allocates "
+                "nothing has a static buffer of %lld bytes (at most %lld points of this network): split the batch, or "
+                "call inference()", numel, channels, words * static_cast<long long>(sizeof(float)),
+                static_cast<long long>(scratchBytes),
+                // per point: its row, its index and its share of the histogram of its chunk
+                static_cast<long long>((scratchBytes / sizeof(float) - 2.0 * SLABS) / (channels + 1 + static_cast<double>(SLABS) / CHUNK))));
+        sortedData = static_cast<float*>(scratch);
+    } else {
+        if (po.capacity < numel) {
+            if (words > std::numeric_limits<int32_t>::max()) return false;   // beyond one tensor: the batch stays as it is
+            po.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
+            po.capacity = numel;
+        }
+        sortedData = po.workspace.dataPtr<float>();
+        capacity = po.capacity;
+        // resolves the static buffer of inferenceNoAlloc() on this device while allocating is
+        // still allowed (the first look-up loads the library's own code object)
+        void* scratch = nullptr;
+        size_t scratchBytes = 0;
+        std::string error;
+        (void)device_code::staticScratch(&scratch, &scratchBytes, error);
     }
-    float* sortedData = po.workspace.dataPtr<float>();
-    int* orderData = reinterpret_cast<int*>(sortedData + po.capacity * channels);   // the sorted rows come first: 16-byte aligned
-    int* totals = orderData + po.capacity;
+    int* orderData = reinterpret_cast<int*>(sortedData + capacity * channels);   // the sorted rows come first: 16-byte aligned
+    int* totals = orderData + capacity;
     int* histogram = totals + SLABS;
 
     int count = numel;
@@ -1275,6 +1329,7 @@ void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory,
     CHECK_DTYPE(input, precisionIn());
     CHECK_DTYPE(output, precisionOut());
     CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
+    checkEncodingParameters(Tensor::INFERENCE);
     if (numel == 0) return;
     CHECK_ERROR(tmpMemory != nullptr, "forward() needs temporary memory of forwardMemory() bytes");
     CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemory) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
@@ -1329,7 +1384,6 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
 
     const bool hasInputGradients = adjointFlags & GRADIENTS_INPUT;
     const bool hasNetworkGradients = adjointFlags & GRADIENTS_NETWORK_WEIGHTS;
-    checkEncodingParameters(Tensor::INFERENCE);
     const bool hasEncodingGradients = adjointFlags & GRADIENTS_INPUT_ENCODINGS;
 
     if (hasInputGradients) {
@@ -1343,6 +1397,9 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         CHECK_ERROR(parametersGradients_.defined(),
                     "Network gradients requested, but no gradient tensor was set via setNetworkParameter(..., GRADIENTS)");
     CHECK_ERROR(parametersInference_.defined(), "Inference parameters not defined, call setNetworkParameter(...) first");
+    checkEncodingParameters(Tensor::INFERENCE);
+    // the kernel adds the gradients of every encoding that has parameters: each needs a tensor to add into
+    if (hasEncodingGradients) checkEncodingParameters(Tensor::GRADIENTS);
     if (numel == 0) return;
     CHECK_ERROR(tmpMemoryForward != nullptr, "adjoint() needs the temporary memory written by forward()");
     std::vector<long long> transposedOffsets;
@@ -1396,9 +1453,6 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     if (!hasNetworkGradients) return;
 
     const bool parallel = compileOptions_.parallelWeightUpdate && layers_.size() > 1;
-    checkEncodingParameters(Tensor::INFERENCE);
-    // the kernel adds the gradients of every encoding that has parameters: each needs a tensor to add into
-    if (hasEncodingGradients) checkEncodingParameters(Tensor::GRADIENTS);
     if (parallel) {
         ensureStreams();
         QMLP_HIP_CALL(qmlp_hip_event_record(adjointEvent_, stream));

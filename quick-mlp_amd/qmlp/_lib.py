@@ -71,6 +71,7 @@ _SIGNATURES = {
     "qmlp_network_initialize_inference_parameters": [_vp, ctypes.c_uint32],
     "qmlp_network_parameter_view": [_vp, _ci, _ci, _vp, _ci, _TD],
     "qmlp_network_inference": [_vp, _TD, _TD, _vp],
+    "qmlp_network_inference_noalloc": [_vp, _TD, _TD, _vp],
     "qmlp_network_forward_memory": [_vp, _ci, _ci, _P(ctypes.c_size_t)],
     "qmlp_network_forward": [_vp, _TD, _TD, _vp, _vp],
     "qmlp_network_zero_gradients": [_vp],

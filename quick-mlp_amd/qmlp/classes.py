@@ -483,6 +483,20 @@ class Network:
             check(lib.qmlp_network_inference(self._handle, desc(input), desc(output), current_stream(input.device)))
         return output
 
+    def inference_noalloc(self, input, output, network_parameters, encoding_parameters=()):
+        """inference() into a tensor of the caller through the entry point of the C ABI that
+        allocates no device memory (for code under HIP graph capture and the like): the kernels must
+        have been loaded by an inference() call on a batch of the same size, the parameters are
+        fp16 already, and a batch that is ordered by grid slab has to fit the library's static
+        48 MiB workspace. Calls that overlap on one GPU race on that workspace."""
+        _device_of(input)
+        if network_parameters.dtype != torch.float16:
+            raise RuntimeError("inference_noalloc takes fp16 network parameters (a conversion would allocate)")
+        with self._mutex:
+            self._set_network_parameters(network_parameters, list(encoding_parameters))
+            check(lib.qmlp_network_inference_noalloc(self._handle, desc(input), desc(output), current_stream(input.device)))
+        return output
+
     def forward_raw(self, input, network_parameters, encoding_parameters=(), flags=7):
         """forward() of the C ABI without autograd: returns (output, tmp_forward)."""
         _device_of(input)
