@@ -10,6 +10,9 @@
 
 namespace qmlp { namespace device_code {
 
+/** Fills `bytes` bytes at `ptr` (device memory) with `value` by a kernel on `stream`. Returns 0 or sets `error`. */
+int fillAsync(void* ptr, int value, size_t bytes, void* stream, std::string& error);
+
 /**
  * Address of the current device's copy of the static scratch buffer and its size. The first
  * call on a device resolves the address (which loads the library's code object onto that

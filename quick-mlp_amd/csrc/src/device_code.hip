@@ -1,7 +1,9 @@
 // The only device code that is compiled into the library ahead of time (everything else is
-// generated and compiled at run time through hipRTC): the static device buffer that the entry
-// point which allocates nothing (qmlp_network_inference_noalloc) uses in place of device
-// memory from hipMalloc.
+// generated and compiled at run time through hipRTC):
+//   * a fill kernel that stands in for hipMemsetAsync, so that a caller may capture any call
+//     of this library into a HIP graph without recording a memset node;
+//   * the static device buffer that the entry point which allocates nothing
+//     (qmlp_network_inference_noalloc) uses in place of device memory from hipMalloc.
 #include "qmlp/device_code.h"
 
 #include <hip/hip_runtime.h>
@@ -21,6 +23,23 @@ constexpr int MAX_DEVICES = 64;
 void* g_scratchAddress[MAX_DEVICES] = {};   // per device: where that device holds its copy
 std::mutex g_scratchMutex;
 
+__global__ void __launch_bounds__(256) FillBytesKernel(unsigned char* __restrict__ p, unsigned char value, size_t bytes)
+{
+    const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t numThreads = static_cast<size_t>(gridDim.x) * 256;
+    // bytes up to the first 16-byte boundary, 16-byte stores in the middle, the rest bytewise
+    size_t head = (16 - reinterpret_cast<uintptr_t>(p) % 16) % 16;
+    if (head > bytes) head = bytes;
+    const size_t body = (bytes - head) / 16;
+    const size_t tail = bytes - head - body * 16;
+    if (tid < head) p[tid] = value;
+    if (tid < tail) p[head + body * 16 + tid] = value;
+    const unsigned int w = value * 0x01010101u;
+    const uint4 word = make_uint4(w, w, w, w);
+    uint4* __restrict__ q = reinterpret_cast<uint4*>(p + head);
+    for (size_t i = tid; i < body; i += numThreads) q[i] = word;
+}
+
 std::string describe(hipError_t e, const char* what)
 {
     return std::string(what) + ": " + hipGetErrorName(e) + " (" + hipGetErrorString(e) + ")";
@@ -29,6 +48,21 @@ std::string describe(hipError_t e, const char* what)
 } // namespace
 
 namespace qmlp { namespace device_code {
+
+int fillAsync(void* ptr, int value, size_t bytes, void* stream, std::string& error)
+{
+    if (bytes == 0) return 0;
+    const size_t blocks = (bytes / 16 + 255) / 256 + 1;
+    const unsigned grid = static_cast<unsigned>(blocks < 4096 ? blocks : 4096);
+    hipLaunchKernelGGL(FillBytesKernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<unsigned char*>(ptr), static_cast<unsigned char>(value), bytes);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        error = describe(e, "launch of the fill kernel");
+        return 1;
+    }
+    return 0;
+}
 
 int staticScratch(void** ptr, size_t* bytes, std::string& error)
 {

@@ -1,7 +1,8 @@
 // Implementation of the thin C ABI in include/qmlp_hip.h on top of the HIP runtime,
-// the HIP module API and hipRTC. This is the only translation unit of the library
-// that talks to HIP.
+// the HIP module API and hipRTC. Together with device_code.hip (the fill kernel and the
+// static scratch buffer) these are the only translation units of the library that talk to HIP.
 #include "qmlp_hip.h"
+#include "qmlp/device_code.h"
 
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
@@ -102,8 +103,11 @@ int qmlp_hip_free(void* ptr)
 
 int qmlp_hip_memset_async(void* ptr, int value, size_t bytes, qmlp_hip_stream stream)
 {
-    if (bytes == 0) return 0;
-    return check(hipMemsetAsync(ptr, value, bytes, static_cast<hipStream_t>(stream)), "hipMemsetAsync");
+    // a kernel, not hipMemsetAsync: memset nodes in a captured HIP graph have given wrong
+    // results on replay on MI355X, and every call of the library is meant to be capturable
+    std::string error;
+    if (qmlp::device_code::fillAsync(ptr, value, bytes, stream, error) != 0) return fail(error);
+    return 0;
 }
 
 int qmlp_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, qmlp_hip_stream stream)

@@ -420,3 +420,34 @@ def test_network_call_after_a_standalone_call_of_its_encoding():
     gi, gp = net.encoding(0).adjoint_with_parameter(x, tables[0], torch.ones_like(alone))
     assert gp.shape == tables[0].shape
     assert torch.equal(first, net.inference(x, params, tables))
+
+
+def test_memset_of_the_loader_is_a_fill_kernel_that_handles_any_alignment():
+    """qmlp_hip_memset_async (what Tensor::zero_ and zeroGradients() use) launches a kernel instead
+    of hipMemsetAsync, so that a captured train step records no memset node; ranges that start
+    and end off a 16-byte boundary, inside a larger buffer whose other bytes must stay."""
+    import ctypes
+    warm_or_gpu()
+    lib = qmlp._lib.lib
+    buf = torch.full((70_000,), 0x5a, dtype=torch.uint8, device="cuda")
+    want = buf.clone()
+    stream = qmlp._lib.current_stream(buf.device)
+    for offset, count, value in ((0, 16, 1), (3, 1, 2), (5, 11, 3), (29, 4099, 0), (4500, 65_000, 0xee), (69_999, 1, 7), (100, 0, 9)):
+        assert lib.qmlp_hip_memset_async(ctypes.c_void_p(buf.data_ptr() + offset), value, ctypes.c_size_t(count), stream) == 0
+        want[offset:offset + count] = value
+    torch.cuda.synchronize()
+    assert torch.equal(buf, want)
+    # recorded into a HIP graph it stays a kernel: replays give the same bytes
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = qmlp._lib.current_stream(buf.device)
+            assert lib.qmlp_hip_memset_async(ctypes.c_void_p(buf.data_ptr() + 7), 0, ctypes.c_size_t(33_333), s) == 0
+    want[7:7 + 33_333] = 0
+    for _ in range(3):
+        buf[7:7 + 33_333] = 0x11
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(buf, want)
