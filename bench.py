@@ -29,10 +29,25 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 # HBM bytes one launch moves, from hardware counters (two profiler runs of this script:
 # FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for the
 # 256 MiB device copy of --copy-calibration: x2.000 and x1.000 on MI355X). The summary
-# with the commands is kept under profiles/. Workloads without a counter run report null.
+# with the commands is kept under profiles/. The figures belong to one version of the device
+# code: "kernels" is device_code_hash() at the time of the counter runs, and a workload whose
+# device code has changed since (or that has no counter run) reports traffic null.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2-inference": {"points": 1 << 20, "fetch": 106149.0 * 1024 * 2.0, "write": 8192.0 * 1024 * 1.0},
+    "cfg2-inference": {"points": 1 << 20, "fetch": 106149.0 * 1024 * 2.0, "write": 8192.0 * 1024 * 1.0,
+                       "kernels": "unmeasured"},
 }
+
+
+def device_code_hash(net):
+    """Hash of everything the fused forward kernel of `net` is compiled from: the generated
+    source and the device headers beside it."""
+    import glob
+    import hashlib
+    h = hashlib.sha256(net.generated_source("forward").encode())
+    kernel_dir = os.path.join(ROOT, "quick-mlp_amd", "csrc", "kernels", "qmlp", "kernels")
+    for f in sorted(glob.glob(os.path.join(kernel_dir, "*.h"))):
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
 
 WORKLOADS = {
     "cfg1-inference": (1, False),
@@ -167,13 +182,207 @@ def cpu_baseline(case, train, min_seconds=10.0):
                       % (len(times), n)}
 
 
+# ------------------------------------------------------------------ layer GEMMs alone
+def mlp_cfg(n_in, widths, activation="relu", last="identity"):
+    from qmlp import baseline_configs as bc
+    acts = [activation] * (len(widths) - 1) + [last]
+    return {"num_inputs": n_in, "num_outputs": widths[-1], "activation_specification": [bc.BUILTIN],
+            "encodings": [{"id": "Identity", "start_in": 0, "n_in": n_in}],
+            "network": [{"n_out": w, "bias": False, "activation": a} for w, a in zip(widths, acts)]}
+
+
+def mlp_flops(n_in, widths, padded):
+    up = (lambda v: (v + 15) // 16 * 16) if padded else (lambda v: v)
+    chain = [up(n_in)] + [up(w) for w in widths]
+    return 2 * sum(a * b for a, b in zip(chain[:-1], chain[1:]))
+
+
+def run_mlp(n_in, widths, n, device, steps, warmup, cached_input=False, train=False, seed=0):
+    """The layers of an identity-encoded network on n points. cached_input: every point reads the
+    same input row (a tensor with stride 0 along the batch), so the input comes from cache and
+    the launch is bound by the layers; otherwise the fp32 rows stream from HBM (4*n_in bytes per
+    point, which bounds narrow networks before the matrix cores do). Returns ms per launch."""
+    import numpy as np
+    import torch
+    import qmlp
+    cfg = mlp_cfg(n_in, widths)
+    net = qmlp.Network(json.dumps(cfg))
+    rng = np.random.default_rng(seed)
+    params = torch.from_numpy((rng.uniform(-1, 1, net.num_network_parameters()) / 8).astype(np.float16)).to(device)
+    if cached_input:
+        x = torch.from_numpy(rng.uniform(-1, 1, (1, n_in)).astype(np.float32)).to(device).expand(n, n_in)
+    else:
+        x = torch.from_numpy(rng.uniform(-1, 1, (n, n_in)).astype(np.float32)).to(device)
+    if not train:
+        def step():
+            net.inference(x, params, [])
+    else:
+        adj = torch.from_numpy(rng.uniform(-1, 1, (n, widths[-1])).astype(np.float32)).to(device)
+        grad_net = torch.zeros((net.num_network_parameters(),), dtype=torch.float32, device=device)
+        adj_in = torch.zeros((n, n_in), dtype=torch.float32, device=device)
+
+        def step():
+            # the reference's "forward + backward": gradients for the input and the weights
+            out, tmp = net.forward_raw(x, params, [], 3)
+            net.adjoint_raw(x, adj, 3, tmp, params, [], grad_network=grad_net, adj_input=adj_in)
+    step()
+    torch.cuda.synchronize()
+    elapsed, launch_ms = time_steps(step, steps, warmup)
+    return launch_ms, 1e3 * elapsed / steps
+
+
+LAYER_GEMM_NETWORKS = (("cfg2_mlp", 32, [64, 64, 1]), ("mlp_64x4", 64, [64, 64, 64, 64, 4]))
+REFERENCE_GRID = [(width, [width] * hidden + [4]) for hidden in (2, 4) for width in (16, 32, 64)]
+
+
+def precompile_networks():
+    """Compiles the kernels of the identity-encoded benchmark networks into the kernel cache
+    (no GPU needed); the build step calls this."""
+    import qmlp
+    for n_in, widths in [(n, w) for _, n, w in LAYER_GEMM_NETWORKS] + REFERENCE_GRID:
+        qmlp.Network(json.dumps(mlp_cfg(n_in, widths))).precompile(3)
+
+
+def layer_gemm_report(device, steps, warmup, only="", n=1 << 20):
+    """MFMA fraction of the layer GEMMs of the hash-grid network (32 -> 64 -> 64 -> 1) run on their
+    own on 2^20 points, and of a deeper 64-wide network."""
+    out = {}
+    for name, n_in, widths in LAYER_GEMM_NETWORKS:
+        for cached in (False, True):
+            if only and only != name + ("_cached_input" if cached else ""):
+                continue
+            ms, _ = run_mlp(n_in, widths, n, device, steps, warmup, cached_input=cached)
+            key = name + ("_cached_input" if cached else "")
+            out[key] = {"launch_ms": ms, "points": n,
+                        "frac": mlp_flops(n_in, widths, False) * n / (ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
+                        "frac_padded_flop": mlp_flops(n_in, widths, True) * n / (ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
+                        "input_hbm_bound_ms": None if cached else 4.0 * (n_in + widths[-1]) * n / (HBM_PEAK_GBS * 1e9) * 1e3}
+    return out
+
+
+def reference_grid(device, steps, warmup, only=""):
+    """The benchmark grid of the reference (tests_py/qmlp_tests/profile_network.py:107-190):
+    10^6 points, 2 or 4 hidden layers of 16, 32 or 64 neurons (as many inputs), ReLU, 4 outputs,
+    no bias, identity encoding; inference and forward + backward (input and weight gradients)."""
+    n = 1000 * 1000
+    rows = []
+    for width, widths in REFERENCE_GRID:
+        hidden = len(widths) - 1
+        if not only or only == "%d x %d" % (width, hidden):
+            inf_ms, inf_wall = run_mlp(width, widths, n, device, steps, warmup)
+            trn_ms, trn_wall = run_mlp(width, widths, n, device, max(3, steps // 2), min(warmup, 3), train=True)
+            flop = mlp_flops(width, widths, False)
+            rows.append({"network": "%d x %d" % (width, hidden), "points": n,
+                         "inference_ms": inf_ms, "inference_wall_ms": inf_wall,
+                         "forward_backward_ms": trn_ms, "forward_backward_wall_ms": trn_wall,
+                         "inference_mfma_frac": flop * n / (inf_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,
+                         "inference_hbm_frac": 4.0 * (width + 4) * n / (inf_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                         "forward_backward_mfma_frac": 3 * flop * n / (trn_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS})
+    return rows
+
+
+# ------------------------------------------------------------------ the request rate of random gathers
+GATHER_SOURCE = r"""
+#include <hip/hip_runtime.h>
+// Random 8-byte gathers, one 128-byte line per lane and load, eight loads in flight per lane:
+// what the grid encodings do. The indices are hashed in the kernel, nothing else touches memory.
+__device__ __forceinline__ unsigned mix(unsigned x)
+{
+    x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+    return x;
+}
+extern "C" __global__ void __launch_bounds__(256) GatherCeiling(const unsigned long long* __restrict__ table,
+                                                                unsigned entries, float* __restrict__ out, int iters)
+{
+    const unsigned gid = blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned long long acc = 0;
+    for (int it = 0; it < iters; it += 8) {
+        unsigned e[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) e[k] = mix(gid * 977u + (it + k) * 0x9e3779b9u) % entries;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc += table[e[k]];
+    }
+    if (acc == 0x123456789abcdefull) out[gid] = 1.f;
+}
+"""
+
+
+def gather_ceiling(device, repeats=5):
+    """Lane-loads per second of random 8-byte gathers from a table that stays in the L2 of every
+    die (2 MiB) and from one that does not (64 MiB), through the loader's C ABI (qmlp_hip.h).
+    Every load of a lane is a 128-byte line of its own, as in a hashed grid level."""
+    import ctypes
+    import torch
+    import qmlp
+    lib = qmlp._lib.lib
+    lib.qmlp_hip_last_error.restype = ctypes.c_char_p
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(lib.qmlp_hip_last_error().decode())
+
+    module, fn, lowered = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_char_p()
+    names = (ctypes.c_char_p * 1)(b"GatherCeiling")
+    opts = (ctypes.c_char_p * 6)(b"-O3", b"-I/opt/rocm/include", b"-Xclang", b"-target-feature", b"-Xclang", b"-packed-fp32-ops")
+    ok(lib.qmlp_hip_module_compile(GATHER_SOURCE.encode(), b"gather_ceiling.hip", None, None, 0, names, 1, opts, 6,
+                                   None, ctypes.byref(module), None))
+    ok(lib.qmlp_hip_module_load(module))
+    ok(lib.qmlp_hip_module_lowered_name(module, b"GatherCeiling", ctypes.byref(lowered)))
+    ok(lib.qmlp_hip_module_get_function(module, lowered, ctypes.byref(fn)))
+    props = torch.cuda.get_device_properties(device)
+    cus, clock_hz = props.multi_processor_count, 2.4e9
+    blocks, threads, iters = 2048, 256, 64
+    table = torch.ones((64 << 20) // 8, dtype=torch.int64, device=device)
+    out = torch.zeros(blocks * threads, dtype=torch.float32, device=device)
+    stream = qmlp._lib.current_stream(device)
+    result = {}
+    for name, nbytes in (("l2_hit", 2 << 20), ("l2_miss", 64 << 20)):
+        a_table, a_entries = ctypes.c_void_p(table.data_ptr()), ctypes.c_uint32(nbytes // 8)
+        a_out, a_iters = ctypes.c_void_p(out.data_ptr()), ctypes.c_int(iters)
+        args = (ctypes.c_void_p * 4)(ctypes.addressof(a_table), ctypes.addressof(a_entries), ctypes.addressof(a_out),
+                                     ctypes.addressof(a_iters))
+        ok(lib.qmlp_hip_launch(fn, blocks, threads, 0, stream, args))
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(repeats):
+            ok(lib.qmlp_hip_launch(fn, blocks, threads, 0, stream, args))
+        stop.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop) / repeats
+        loads = float(blocks) * threads * iters
+        result[name] = {"table_bytes": nbytes, "requests_per_s": loads / (ms * 1e-3),
+                        "requests_per_clock_and_cu": loads / (ms * 1e-3) / cus / clock_hz, "launch_ms": ms}
+    ok(lib.qmlp_hip_module_destroy(module))
+    result["compute_units"] = cus
+    result["clock_hz_assumed"] = clock_hz
+    return result
+
+
+def request_ceiling(gather, points, requests_per_point, l2_miss_fraction, launch_ms):
+    """Prices the line requests of a gathering launch with the two measured rates."""
+    hit = points * requests_per_point * (1.0 - l2_miss_fraction) / gather["l2_hit"]["requests_per_s"]
+    miss = points * requests_per_point * l2_miss_fraction / gather["l2_miss"]["requests_per_s"]
+    bound_ms = 1e3 * (hit + miss)
+    return {"requests_per_point": requests_per_point, "l2_miss_fraction": l2_miss_fraction,
+            "l2_hit_requests_per_s": gather["l2_hit"]["requests_per_s"],
+            "l2_miss_requests_per_s": gather["l2_miss"]["requests_per_s"],
+            "bound_ms": bound_ms, "frac_of_bound": bound_ms / launch_ms}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2-inference", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg2-inference",
+                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "all"],
+                    help="layer-gemm: the layers of the hash-grid network on their own; reference-grid: the reference's "
+                         "own benchmark networks; gather-ceiling: request rate of random gathers; all: every workload")
     ap.add_argument("--points", type=int, default=0, help="override the number of points")
+    ap.add_argument("--case", default="", help="layer-gemm / reference-grid: only the case of this name "
+                                               "(e.g. cfg2_mlp_cached_input, '64 x 4')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step measurement")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -200,6 +409,51 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    head = {"metric": "points/sec fused hashgrid+MLP inference & train step; % MFMA/HBM roofline", "unit": "points/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16", "data": "synthetic"}
+    if args.workload == "layer-gemm":
+        report = layer_gemm_report(device, args.steps, args.warmup, args.case, args.points or (1 << 20))
+        ms = next(iter(report.values()))["launch_ms"]
+        print(json.dumps(dict(head, value=(args.points or (1 << 20)) / (ms * 1e-3), ms_per_step=ms,
+                              config={"workload": "layer-gemm", "points": args.points or (1 << 20),
+                                      "case": args.case or "all (value: the first)"},
+                              mfma=dict(peak_tflops=MFMA_FP16_PEAK_TFLOPS, layer_gemm=report))))
+        return
+    if args.workload == "reference-grid":
+        rows = reference_grid(device, args.steps, args.warmup, args.case)
+        print(json.dumps(dict(head, value=rows[-1]["points"] / (rows[-1]["inference_ms"] * 1e-3),
+                              ms_per_step=rows[-1]["inference_ms"],
+                              config={"workload": "reference-grid", "points": rows[-1]["points"],
+                                      "network": rows[-1]["network"] + " (value); all six under networks"},
+                              networks=rows)))
+        return
+    if args.workload == "gather-ceiling":
+        g = gather_ceiling(device)
+        print(json.dumps(dict(head, value=g["l2_hit"]["requests_per_s"], unit="line requests/s",
+                              ms_per_step=g["l2_hit"]["launch_ms"],
+                              config={"workload": "gather-ceiling", "loads": 2048 * 256 * 64}, gather=g)))
+        return
+    if args.workload == "all":
+        g = gather_ceiling(device)
+        summary = {"gather": g, "layer_gemm": layer_gemm_report(device, args.steps, args.warmup),
+                   "reference_grid": reference_grid(device, args.steps, args.warmup), "workloads": {}}
+        for name, (cid, trn) in sorted(WORKLOADS.items()):
+            cc = bc.CONFIGS[cid]
+            cs = build_case(cid, cc["points"], device)
+            el, lms = (run_train if trn else run_inference)(cs, args.steps, args.warmup)
+            bpp = cc["gather_bytes_per_point"] + cc["io_bytes_per_point"]
+            summary["workloads"][name] = {
+                "points": cc["points"], "ms_per_step": 1e3 * el / args.steps, "launch_ms": lms,
+                "points_per_s": args.steps * cc["points"] / el,
+                "hbm_frac": bpp * cc["points"] / (lms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "mfma_frac": cc["flop_per_point"] * cc["points"] / (lms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS}
+            del cs
+        w = summary["workloads"]["cfg2-inference"]
+        print(json.dumps(dict(head, value=w["points_per_s"], ms_per_step=w["ms_per_step"],
+                              config={"workload": "all (value: cfg2-inference)"}, **summary)))
+        return
+
     cfg_id, train = WORKLOADS[args.workload]
     c = bc.CONFIGS[cfg_id]
     n = args.points or c["points"]
@@ -213,7 +467,7 @@ def main():
     flops = c["flop_per_point"] * n / (launch_ms * 1e-3)
     traffic = None
     m = MEASURED_TRAFFIC_BYTES.get(args.workload)
-    if m is not None and m["points"] == n:
+    if m is not None and m["points"] == n and m["kernels"] == device_code_hash(case["net"]):
         # same form as "achieved": bytes of one launch over the launch duration measured now
         traffic = (m["fetch"] + m["write"]) / (launch_ms * 1e-3) / 1e9
     result = {
@@ -233,7 +487,15 @@ def main():
         "mfma": {"achieved_tflops": flops / 1e12, "peak_tflops": MFMA_FP16_PEAK_TFLOPS,
                  "frac": flops / 1e12 / MFMA_FP16_PEAK_TFLOPS, "flop_per_point": c["flop_per_point"]},
         "kernel_cache": dict(zip(("compiled", "disk_hits"), qmlp._lib.kernel_cache_stats())),
+        "device_code": device_code_hash(case["net"]),
     }
+    if not train and cfg_id == 2:
+        # the two north-star fractions of the hash-grid network: its layer GEMMs on their own, and
+        # the launch against the request rate of random gathers measured in this same run (64 line
+        # requests per point: 16 levels x 4 pairs of corners; 3% of them miss the L2, see profiles/)
+        result["mfma"]["layer_gemm"] = layer_gemm_report(device, max(10, args.steps // 2), args.warmup)
+        result["mfma"]["layer_gemm_frac"] = result["mfma"]["layer_gemm"]["cfg2_mlp_cached_input"]["frac"]
+        result["roofline"]["request_ceiling"] = request_ceiling(gather_ceiling(device), n, 64.0, 0.03, launch_ms)
     if not train and cfg_id == 2 and not args.no_train:
         # the train step of the same network at its own batch size
         c3 = bc.CONFIGS[3]

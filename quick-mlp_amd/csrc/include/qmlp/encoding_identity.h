@@ -21,6 +21,8 @@ public:
     [[nodiscard]] int numOutputChannels() const override;
     [[nodiscard]] std::string qualifiedName() const override;
     void fillCode(std::stringstream& code) const override;
+
+    [[nodiscard]] int startChannel() const { return startChannel_; }
 };
 
 QUICKMLP_NAMESPACE_END

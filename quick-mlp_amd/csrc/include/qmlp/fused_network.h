@@ -54,6 +54,11 @@ public:
         // takes 8 tiles at once, and 2^20 points are one sweep over the level tables.
         bool registerStaging = true;
 
+        // If true (default), a network whose only encoding is the identity loads its first
+        // matrix-core operands straight from the input rows; false sends them through the LDS
+        // staging rows like every other encoding (same results bit for bit).
+        bool directInput = true;
+
         // Inference only: evaluate the points slab by slab of a dense grid that exceeds the L2
         // (a counting sort of the batch in front of the fused kernel, see point_order.h; the
         // results are those of the order given). <0 (default): the library decides from the
@@ -300,6 +305,11 @@ private:
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */
+    /** Function attributes of the generated forward / backward kernels. */
+    std::string kernelAttributes() const;
+    /** First input channel of the identity encoding if that is the network's only encoding and
+     *  options.direct_input is on; -1 otherwise. */
+    int directInputStart() const;
     /** Throws unless every encoding with parameters has a tensor bound for 'usage'. */
     void checkEncodingParameters(Tensor::Usage usage) const;
     void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false);

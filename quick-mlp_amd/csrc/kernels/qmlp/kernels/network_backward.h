@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(256) TransposeWeightsKernel(const half* __rest
     }
 }
 
-__global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelBackward(
+__global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkKernelBackward(
     int numel,
     const Tensor2Read<float> inputs,      //shape (numel, Cin)
     const Tensor2Read<float> adjOutputs,  //shape (numel, Cout)

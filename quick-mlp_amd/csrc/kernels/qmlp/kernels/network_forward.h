@@ -44,7 +44,7 @@ __device__ __forceinline__ void bindEncodingRow(PackedRegisterRowsView<T, PPL, C
  *   into forwardTmpMemory for the adjoint pass.
  */
 template <bool STORE>
-__global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForward(
+__global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkKernelInferenceAndForward(
     int numel,
     const Tensor2Read<float> inputs,  //shape (numel, Cin)
     Tensor2RW<float> outputs,         //shape (numel, Cout)
@@ -75,6 +75,12 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     // the wavefronts of the workgroup then walk the tiles and layers in lockstep (workgroup
     // barriers inside the loops), wavefronts without a tile compute on zero rows.
     constexpr bool HAS_STREAMED_LAYERS = $$HAS_STREAMED_LAYERS$$;
+    // >= 0: the only encoding is an identity encoding of the input channels from this one on.
+    // Lanes then load their matrix-core operands (4 consecutive channels of 4 points) straight
+    // from the input rows, and nothing goes through the LDS staging rows.
+    constexpr int DIRECT_INPUT_START = $$DIRECT_INPUT_START$$;
+    constexpr bool DIRECT_INPUT = DIRECT_INPUT_START >= 0;
+    static_assert(!DIRECT_INPUT || PPL == 1, "direct input rows: one tile per wave");
 
     const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
     f16* __restrict__ forwardTmpMemory = reinterpret_cast<f16*>(forwardTmpMemoryH);
@@ -85,6 +91,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) NetworkKernelInferenceAndForwa
     const int lane = threadIdx.x % WAVE_SIZE;
     const int g = lane >> 4, r = lane & 15;
     f16* sStage = sParams + LDS_PARAM_HALVES + wave * (STAGED_TILES * TILE_POINTS * STAGE_STRIDE);
+    (void)sStage;
 
     // stage the weights in operand order, then the biases
 $$STAGE_PARAMETERS$$
@@ -108,7 +115,7 @@ $$STAGE_PARAMETERS$$
         // no NaN enters the matrix cores.
         PackedRegisterRows<f16, REGISTER_STAGING ? PPL : 1, CHANNELS_IN> encodedRegisters = {};   // halves are merged into it
         (void)encodedRegisters;
-        {
+        if constexpr (!DIRECT_INPUT) {
             StaticArray<float, NUM_INPUTS> encodingInput[PPL];
             $$ENCODING_OUTPUT_ROWS$$
             bool valid[PPL];
@@ -150,8 +157,8 @@ $$CALL_ENCODINGS$$
                     for (int c = 0; c < ENCODED_CHANNELS; ++c) encodingOutput[q][c] = static_cast<f16>(0);
                 }
             }
+            waveLdsSync();
         }
-        waveLdsSync();
 
 $$TILE_LOOP_PRAGMA$$
         for (int q = 0; q < PPL; ++q)
@@ -162,6 +169,7 @@ $$TILE_LOOP_PRAGMA$$
         const int tmpTile = tile + tmpTileOffset;
         (void)tmpTile;
         const f16* sTile = sStage + (REGISTER_STAGING ? 0 : q) * (TILE_POINTS * STAGE_STRIDE);
+        (void)sTile;
         if (REGISTER_STAGING) {
             // the lane's row of this tile: registers -> staging row, 8 bytes at a time
             if (q > 0) waveLdsSync();   // the operands of the previous tile have been read
@@ -177,11 +185,57 @@ $$TILE_LOOP_PRAGMA$$
 
         // B operands of the first layer
         f16x4 x0[NT][KT0];
+        if constexpr (DIRECT_INPUT) {
+            const bool rowsOfFloat4 = DIRECT_INPUT_START % 4 == 0 && inputs.strides_[1] == 1 && inputs.strides_[0] % 4 == 0
+                && reinterpret_cast<unsigned long long>(inputs.data_) % 16 == 0;
+            const float* row0 = inputs.data_ + static_cast<long long>(tile * TILE_POINTS + 4 * r) * inputs.strides_[0]
+                + static_cast<long long>(DIRECT_INPUT_START) * inputs.strides_[1];
+            if (rowsOfFloat4 && (tile + 1) * TILE_POINTS <= numel) {
+                // a whole tile of rows whose channels lie side by side: nothing is predicated
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float* row = row0 + static_cast<long long>(nt) * inputs.strides_[0];
 #pragma unroll
-            for (int t = 0; t < KT0; ++t)
-                x0[nt][t] = *reinterpret_cast<const f16x4*>(sTile + Stage::chunkOffset(16 * nt + r, 4 * t + g));
+                    for (int t = 0; t < KT0; ++t) {
+                        const int c = 16 * t + 4 * g;   // first of this lane's four encoded channels
+                        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                        if (16 * t + 15 < ENCODED_CHANNELS) {
+                            v = *reinterpret_cast<const f32x4*>(row + c);
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                if (c + i < ENCODED_CHANNELS) v[i] = row[c + i];
+                        }
+                        x0[nt][t] = toF16(v);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const bool pv = tile * TILE_POINTS + 4 * r + nt < numel;
+                    const float* row = row0 + static_cast<long long>(nt) * inputs.strides_[0];
+#pragma unroll
+                    for (int t = 0; t < KT0; ++t) {
+                        const int c = 16 * t + 4 * g;
+                        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                        if (16 * t + 15 < ENCODED_CHANNELS && rowsOfFloat4) {
+                            if (pv) v = *reinterpret_cast<const f32x4*>(row + c);
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                if (pv && c + i < ENCODED_CHANNELS) v[i] = row[static_cast<long long>(c + i) * inputs.strides_[1]];
+                        }
+                        x0[nt][t] = toF16(v);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int t = 0; t < KT0; ++t)
+                    x0[nt][t] = *reinterpret_cast<const f16x4*>(sTile + Stage::chunkOffset(16 * nt + r, 4 * t + g));
+        }
 
         if (STORE && tileValid) {
             // encoded input, channel-major per tile, for the weight update of layer 0
@@ -251,7 +305,7 @@ $$CALL_NETWORK_LAYERS$$
                 }
         }
         }
-        waveLdsSync();   // the staging rows are overwritten by the next group of tiles
+        if constexpr (!DIRECT_INPUT) waveLdsSync();   // the staging rows are overwritten by the next group of tiles
     }
 }
 

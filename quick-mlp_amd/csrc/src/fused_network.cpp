@@ -75,6 +75,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
             throw configuration_error("points_per_lane must be at most 8, but is %d", compileOptions_.pointsPerLane);
         compileOptions_.registerStaging = options.value("register_staging", compileOptions_.registerStaging);
         compileOptions_.sortPoints = options.value("sort_points", compileOptions_.sortPoints);
+        compileOptions_.directInput = options.value("direct_input", compileOptions_.directInput);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
             options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
@@ -500,8 +501,28 @@ int FusedNetwork::ldsParamHalves(bool adjoint) const
     return ldsLayout(adjoint, w, b);
 }
 
+std::string FusedNetwork::kernelAttributes() const
+{
+    // Two wavefronts per SIMD at least: the register budget is then 256, all of them vector
+    // registers, and the compiler keeps the matrix-core accumulators there (with up to 512 it
+    // puts them into accumulation registers and copies every value out one by one). Layers
+    // wider than 128 need more than 256 registers and keep the larger budget.
+    int widest = 0;
+    for (const auto& l : layers_) widest = std::max(widest, std::max(l.channelsIn, l.channelsOut));
+    return widest <= 128 ? "__attribute__((amdgpu_waves_per_eu(2)))" : "";
+}
+
+int FusedNetwork::directInputStart() const
+{
+    if (!compileOptions_.directInput || encodings_.size() != 1) return -1;
+    const auto* identity = dynamic_cast<const EncodingIdentity*>(encodings_[0].get());
+    return identity ? identity->startChannel() : -1;
+}
+
 int FusedNetwork::stageBytesPerWave(bool adjoint) const
 {
+    // operands straight from the input rows: the forward kernel stages nothing
+    if (!adjoint && directInputStart() >= 0) return 0;
     // the forward kernel rotates the chunks of rows of 32, 64 or 128 halves instead of padding them
     const int c = layers_[0].channelsIn;
     const bool rotated = !adjoint && (c == 32 || c == 64 || c == 128);
@@ -587,6 +608,8 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool r
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
     replaceAll(code, "$$POINTS_PER_LANE$$", std::to_string(pointsPerLane));
     replaceAll(code, "$$REGISTER_STAGING$$", registerStaging ? "true" : "false");
+    replaceAll(code, "$$DIRECT_INPUT_START$$", std::to_string(directInputStart()));
+    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes());
     // rows in registers are indexed by the tile: that loop has to be unrolled
     replaceAll(code, "$$TILE_LOOP_PRAGMA$$", registerStaging ? "#pragma unroll" : "#pragma unroll 1");
     std::vector<int> ldsW, ldsB;
@@ -693,6 +716,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
     std::string code = kl->findFile("qmlp/kernels/network_backward.h").value();
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
+    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes());
     replaceAll(code, "$$HAS_INPUT_GRADIENTS$$", hasInputGradients ? "true" : "false");
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
     replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
@@ -844,6 +868,31 @@ std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFl
         const int blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false, &ppl);
         return forwardSource(blockSize, ppl);
     }
+    if (kind == "shapes") {
+        // which shapes of the forward kernel this network may launch (diagnostics and tests)
+        std::stringstream ss;
+        ss << "[";
+        for (int store = 0; store < 2; ++store) {
+            const char* pass = store ? "forward" : "inference";
+            auto add = [&](const char* name, int variant) {
+                int blockSize = 0, pointsPerLane = 1;
+                forwardShape(store != 0, variant, blockSize, pointsPerLane);
+                if (ss.tellp() > 1) ss << ", ";
+                ss << "{\"pass\": \"" << pass << "\", \"shape\": \"" << name << "\", \"block\": " << blockSize
+                   << ", \"tiles_per_wave\": " << pointsPerLane << "}";
+            };
+            add("default", VARIANT_DEFAULT);
+            int ppl = 1;
+            forwardBlockSize(-1, false, &ppl);
+            if (ppl > 1) add("narrow", VARIANT_NARROW);
+            if (hasLargeVariant(store != 0)) add("large", VARIANT_LARGE);
+            if (registerVariantTiles(store != 0) > 0) add("registers", VARIANT_REGISTERS);
+        }
+        ss << "]";
+        return ss.str();
+    }
+    // the shape with the encoded rows in registers, whether or not the network would get it
+    if (kind == "forward_registers") return forwardSource(2 * DEFAULT_BLOCK_SIZE, std::min(8, 256 / layers_[0].channelsIn), true);
     if (kind == "backward") return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true));
     if (kind == "weight_update") return weightUpdateSource(DEFAULT_BLOCK_SIZE);
     throw std::runtime_error("unknown kernel kind '" + kind + "'");

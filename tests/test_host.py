@@ -433,3 +433,32 @@ def test_the_python_binding_cache_forgets_a_table_the_standalone_call_unbound():
     for name in ("inference_with_parameter", "adjoint_with_parameter_and_flags"):
         body = src.split("def %s(" % name)[1].split("\n    def ")[0]
         assert "self._bound_inference = None" in body, name
+
+
+def test_rows_in_registers_shape_is_not_offered_to_single_table_or_gather_heavy_grids():
+    """The forward shape that keeps the encoded rows of 8 tiles in registers pays through fewer
+    sweeps over the tables of a multi-level grid. A grid with one table has nothing to sweep, and
+    a cell whose gathers need more than 128 registers for 8 points spills by the kilobyte: a
+    dense 4-D grid with 8 features (BASELINE config 5) is both, and its kernel of that shape
+    once ended in a GPU memory fault. Such networks must never be given the shape."""
+    def shapes(cfg):
+        return {(s["pass"], s["shape"]) for s in json.loads(qmlp.Network(json.dumps(cfg)).generated_source("shapes"))}
+
+    assert ("inference", "registers") in shapes(bc.CONFIGS[2]["cfg"])
+    for cfg_id in (1, 4, 5):
+        assert not any(shape == "registers" for _, shape in shapes(bc.CONFIGS[cfg_id]["cfg"])), cfg_id
+    base = bc.CONFIGS[5]["cfg"]
+    for change in ({"n_features_per_level": 2}, {"n_features_per_level": 4, "n_levels": 1},
+                   {"n_levels": 2, "min_resolution": 16, "max_resolution": 32}):      # 2 levels, but 16 corners x 8 features
+        cfg = json.loads(json.dumps(base))
+        cfg["encodings"][0].update(change)
+        got = shapes(cfg)
+        if cfg["encodings"][0]["n_levels"] < 2:
+            assert not any(shape == "registers" for _, shape in got), change
+        else:
+            # 8 points x 16 corners x 8 fp16 features = 512 registers in flight: beyond the limit of 128
+            assert not any(shape == "registers" for _, shape in got), change
+    # and the option switches the shape off for a network that would get it
+    cfg = json.loads(json.dumps(bc.CONFIGS[2]["cfg"]))
+    cfg["options"] = {"register_staging": False}
+    assert not any(shape == "registers" for _, shape in shapes(cfg))
