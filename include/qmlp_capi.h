@@ -160,6 +160,16 @@ int qmlp_encoding_hashgrid_levels(qmlp_encoding_t encoding, int capacity, int* n
  * indices/weights are device arrays of N * levels * 2^dim entries. */
 int qmlp_encoding_hashgrid_corners(qmlp_encoding_t encoding, const qmlp_tensor* input, uint32_t* indices,
                                    float* weights, void* stream);
+/* HashGrid only (test aid, no counterpart in the reference): the same two arrays, written by the
+ * code the fused kernels run. mode 1: the table entries (element offset of feature 0) and weights
+ * that the gathers of the fused forward / inference kernels use, including their paired loads
+ * (needs a bound table, src_cpp/include/qmlp/kernels/encoding_hashgrid.cuh:267-336 is what they
+ * replace); mode 2: the entries and weights the gradient scatter of the fused backward kernel
+ * adds to (encoding_hashgrid.cuh:345-369; nothing is added); mode 0 = qmlp_encoding_hashgrid_corners.
+ * The order of the 2^dim corners of a level is the order the code visits them. input = NULL only
+ * compiles the kernel of that mode into the kernel cache (needs no GPU). */
+int qmlp_encoding_hashgrid_trace(qmlp_encoding_t encoding, const qmlp_tensor* input, int mode, uint32_t* indices,
+                                 float* weights, void* stream);
 
 /* ---- qmlp::Activation (src_cpp/include/qmlp/activation.h:29-150) ---- */
 /* ActivationFactory(loader).getOrInline(key), activation.h:136: a built-in id or an inline

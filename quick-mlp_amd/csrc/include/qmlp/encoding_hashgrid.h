@@ -72,6 +72,7 @@ public:
     [[nodiscard]] Tensor::Precision parameterPrecision(Tensor::Usage usage) const override;
     [[nodiscard]] int parameterCount() const override;
     [[nodiscard]] int ldsGradientFloats(int maxBytes, int& levels) const override;
+    [[nodiscard]] bool gradientSlices(GradientSliceLayout& layout) const override;
     [[nodiscard]] int numSweptTables() const override { return numLevels_; }
     [[nodiscard]] int gatherRegistersPerPoint() const override;
     [[nodiscard]] bool pointOrderKey(kernel::PointOrderKey& key, long long numPoints = 0) const override;
@@ -101,13 +102,17 @@ public:
     /**
      * Test aid: evaluates the device index code. indices / weights are device arrays with
      * N * numLevels() * 2^ndim() entries: table offset of feature 0 and interpolation
-     * weight of every corner.
+     * weight of every corner. mode 0: the index function on its own; 1: the table entries that
+     * the gathers of the fused forward kernels use (needs a bound table); 2: the entries the
+     * gradient scatter of the fused backward kernel adds to (nothing is added).
      */
-    void corners(const Tensor& input, unsigned* indices, float* weights, stream_t stream);
+    void corners(const Tensor& input, unsigned* indices, float* weights, stream_t stream, int mode = 0);
+    /** Compiles the kernel of corners(.., mode); compileOnly: into the kernel cache only, which needs no GPU. */
+    void precompileCorners(int mode, bool compileOnly);
 
 private:
     [[nodiscard]] std::string configName() const;
-    std::optional<KernelFunction> cornersKernel_;
+    std::optional<KernelFunction> cornersKernel_[3];
 };
 
 QUICKMLP_NAMESPACE_END

@@ -68,6 +68,11 @@ public:
         // network on several streams at once would share it.
         int sortPoints = -1;
 
+        // Parameter gradients of grid encodings: summed slice by slice in LDS by a kernel of its own
+        // (kernels/grid_gradient.h) instead of scattered with float atomics by the backward kernel.
+        // <0 (default): for batches of 16 384 points or more; 0: never; >0: always.
+        int sliceGradients = -1;
+
         // Accepted for compatibility; the LDS layouts of this implementation are
         // bank-conflict free for 64 lanes by construction and need no skew.
         bool skewSharedMemory = false;
@@ -156,15 +161,35 @@ private:
         CompiledKernel kernel;
         int numChunks = 1;
     };
+    /** Kernels that sum the parameter gradients of one grid encoding slice by slice (grid_gradient.h). */
+    struct SliceGradientKernel
+    {
+        int encoding = -1;
+        IEncoding::GradientSliceLayout layout;
+        CompiledKernel records;      // GridGradientRecordsKernel
+        CompiledKernel kernel;       // GridGradientSlicesKernel
+        Tensor items;                // device copy of layout.items
+    };
     struct AdjointKernel
     {
         CompiledKernel adjoint;
+        std::vector<SliceGradientKernel> sliceGradients;
         std::vector<WeightUpdateKernel> layers;
         CompiledKernel reduce;
         CompiledKernel transpose;
         int perEntryAdjointMemoryBytes = 0;
     };
-    std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS];
+    // [adjoint flags][grid gradients by slices instead of atomics]
+    std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2];
+    static constexpr int SLICE_GRADIENTS_MIN_BATCH = 1 << 14;
+    /** True if some encoding of the network offers gradient slices (the adjoint memory then has room for the adjoint of the encoded rows). */
+    bool hasSliceGradients() const;
+    /** Bytes per point of adjoint memory for the adjoint of the encoded rows (read by the records kernels); 0 without them. */
+    int sliceGradientBytesPerPoint() const;
+    /** Bytes of bucket cursors and records of all encodings with gradient slices for a batch of numel (padded) points. */
+    size_t sliceGradientWorkspaceBytes(long long numel) const;
+    /** Whether a batch of numel points with these flags takes the slice kernels. */
+    bool useSliceGradients(int numel, int flags) const;
 
     int perEntryForwardMemoryBytes_;
     std::vector<AdjointLayerInfo> backwardInfo_;
@@ -313,10 +338,10 @@ private:
     /** Throws unless every encoding with parameters has a tensor bound for 'usage'. */
     void checkEncodingParameters(Tensor::Usage usage) const;
     void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false);
-    void compileBackwardKernel(int flags, bool compileOnly = false);
+    void compileBackwardKernel(int flags, bool sliceGradients = false, bool compileOnly = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false) const;
-    std::string backwardSource(int flags, int blockSize) const;
+    std::string backwardSource(int flags, int blockSize, bool sliceGradients = false) const;
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const;
     void fillEncodingsAndActivations(std::string& codeTemplate) const;
@@ -352,7 +377,7 @@ private:
         int byteOffset = 0;  // of the region in the kernel's dynamic LDS
     };
     /** One entry per encoding; returns the LDS bytes of the backward kernel including these regions. */
-    int ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding) const;
+    int ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients = false) const;
     std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);
     void ensureStreams();
 };

@@ -120,6 +120,54 @@ public:
     /** Output channels that the device code writes together (the features of a grid entry). */
     [[nodiscard]] virtual int channelsWrittenTogether() const { return 1; }
 
+    /** One work item of GridGradientSlicesKernel (mirrors kernel::GridGradientSlice). */
+    struct GradientSlice
+    {
+        int level;
+        unsigned first;
+        int floats;
+        int slice;
+        int part;
+        int parts;
+        int reserved0;
+        int reserved1;
+    };
+    /** What the host needs to run the kernels of kernels/grid_gradient.h for an encoding. */
+    struct GradientSliceLayout
+    {
+        std::string configType;            // device type of the level table
+        int sliceFloats = 0;               // floats of a full slice (= LDS of the slice kernel / 4)
+        int recordWords = 0;               // 32-bit words of a record
+        int pairs = 0;                     // records per point and level
+        int pointsPerWorkgroup = 0;        // lanes of a workgroup of the records kernel
+        int recordsLdsBytes = 0;           // its dynamic LDS
+        std::vector<int> slicesPerLevel;
+        std::vector<GradientSlice> items;  // one workgroup of the slice kernel each
+        /** Records a bucket of level l holds for a batch of numel points (as in the device code). */
+        long long capacity(int l, long long numel) const { return ((5 * numel * pairs / 4) / slicesPerLevel[l] + 2048) & ~3ll; }
+        long long totalRecords(long long numel) const
+        {
+            long long n = 0;
+            for (size_t l = 0; l < slicesPerLevel.size(); ++l) n += slicesPerLevel[l] * capacity(static_cast<int>(l), numel);
+            return n;
+        }
+        int numBuckets() const
+        {
+            int n = 0;
+            for (int s : slicesPerLevel) n += s;
+            return n;
+        }
+    };
+    /**
+     * Encodings whose parameter gradients can be summed slice by slice in LDS instead of being
+     * scattered with global atomics (see kernels/grid_gradient.h) return true and fill in the layout.
+     */
+    [[nodiscard]] virtual bool gradientSlices(GradientSliceLayout& layout) const
+    {
+        (void)layout;
+        return false;
+    }
+
     [[nodiscard]] virtual int ldsGradientFloats(int maxBytes, int& levels) const
     {
         levels = 0;

@@ -23,6 +23,7 @@
 // input gradient carries the (R-1) chain-rule factor when Cfg::ResolutionFactor.
 
 #include <qmlp/kernels/common.h>
+#include <qmlp/kernels/arrays.h>
 
 QUICKMLP_KERNEL_NAMESPACE_BEGIN
 
@@ -96,6 +97,30 @@ __device__ __forceinline__ void loadPair(const T* __restrict__ p, float (&a)[F],
 __device__ __forceinline__ constexpr bool isPow2(unsigned v) { return v != 0u && (v & (v - 1u)) == 0u; }
 
 } // namespace detail
+
+/** gatherLevel / scatterTile without a record of what they touch (every kernel of the product). */
+struct NoCornerTrace
+{
+    static constexpr bool Enabled = false;
+};
+
+/**
+ * Test aid: gatherLevel and scatterTile write, for every table entry whose value they use (or add
+ * to), its element offset (of feature 0) and the weight it is used with, instead of leaving no
+ * trace. The arrays hold Levels * 2^Dim slots per point; slot = level * 2^Dim + corner in the
+ * order the code visits them.
+ */
+struct CornerTrace
+{
+    static constexpr bool Enabled = true;
+    unsigned* __restrict__ elements;   // slots of the point (gather) or of the whole batch (scatter)
+    float* __restrict__ weights;
+    __device__ __forceinline__ void record(long long slot, unsigned element, float weight) const
+    {
+        elements[slot] = element;
+        weights[slot] = weight;
+    }
+};
 
 /**
  * \tparam Cfg generated struct with
@@ -190,8 +215,10 @@ struct EncodingHashGrid
      * Values and weights are the same as in the corner-by-corner evaluation, only the order
      * of the fp32 additions differs.
      */
+    template <typename Trace = NoCornerTrace>
     __device__ __forceinline__ static void gatherLevel(int l, const float (&pos)[D],
-                                                       const table_t* __restrict__ table, float (&feat)[F])
+                                                       const table_t* __restrict__ table, float (&feat)[F],
+                                                       const Trace& trace = Trace{})
     {
         // no contraction into fused multiply-adds: the kernels of different shapes (tiles per
         // wave) would contract differently, and the same point has to give the same bits
@@ -222,12 +249,17 @@ struct EncodingHashGrid
                     w = w * (hi ? s.f[d] : (1.f - s.f[d]));
                 }
                 float e0[F], e1[F];
-                detail::loadPair<F>(table + (base + idx * static_cast<unsigned>(F)), e0, e1);
+                const unsigned pairElement = base + idx * static_cast<unsigned>(F);   // e0 = this entry, e1 = the next
+                detail::loadPair<F>(table + pairElement, e0, e1);
 #pragma unroll
                 for (int i = 0; i < F; ++i) {
                     const float vL = lSecond ? e1[i] : e0[i];
                     const float vH = hSecond ? e1[i] : e0[i];
                     feat[i] += w * (wzL * vL + wzH * vH);
+                }
+                if constexpr (Trace::Enabled) {
+                    trace.record(l * NC + 2 * c, pairElement + (lSecond ? F : 0), w * wzL);
+                    trace.record(l * NC + 2 * c + 1, pairElement + (hSecond ? F : 0), w * wzH);
                 }
             }
         } else if (hashed && detail::isPow2(Cfg::hashGridSize[l]) && Cfg::hashGridSize[l] >= 2u) {
@@ -246,11 +278,17 @@ struct EncodingHashGrid
                 const unsigned idxL = (s.termL[0] ^ rest) & mask;
                 const unsigned idxH = (s.termH[0] ^ rest) & mask;
                 float e0[F], e1[F];
-                detail::loadPair<F>(table + (base + (idxL & ~1u) * static_cast<unsigned>(F)), e0, e1);
+                const unsigned pairElement = base + (idxL & ~1u) * static_cast<unsigned>(F);   // e0 = this entry, e1 = the next
+                detail::loadPair<F>(table + pairElement, e0, e1);
                 float vH[F];
                 const bool samePair = ((idxL ^ idxH) & ~1u) == 0u;
+                const unsigned upperElement = base + idxH * static_cast<unsigned>(F);
+                if constexpr (Trace::Enabled) {
+                    trace.record(l * NC + 2 * c, pairElement + ((idxL & 1u) ? F : 0), w * wxL);
+                    trace.record(l * NC + 2 * c + 1, samePair ? pairElement + ((idxH & 1u) ? F : 0) : upperElement, w * wxH);
+                }
                 if (!samePair) {
-                    detail::loadFeatures<F>(table + (base + idxH * static_cast<unsigned>(F)), vH);
+                    detail::loadFeatures<F>(table + upperElement, vH);
                 } else {
 #pragma unroll
                     for (int i = 0; i < F; ++i) vH[i] = (idxH & 1u) ? e1[i] : e0[i];
@@ -266,9 +304,11 @@ struct EncodingHashGrid
             for (int c = 0; c < NC; ++c) {
                 const float w = cornerWeight(s, c);
                 float v[F];
-                detail::loadFeatures<F>(table + cornerOffset(l, s, c), v);
+                const unsigned element = cornerOffset(l, s, c);
+                detail::loadFeatures<F>(table + element, v);
 #pragma unroll
                 for (int i = 0; i < F; ++i) feat[i] += w * v[i];
+                if constexpr (Trace::Enabled) trace.record(l * NC + c, element, w);
             }
         }
     }
@@ -459,10 +499,11 @@ struct EncodingHashGrid
      * \param adjOutput callable (point of the tile 0..63, output channel of this encoding) ->
      *    adjoint of that output as float
      */
-    template <int LDS_LEVELS = 0, typename AdjFn>
+    template <int LDS_LEVELS = 0, typename AdjFn, typename Trace = NoCornerTrace>
     __device__ __forceinline__ static void scatterTile(int lane, long long index0, long long numel,
                                                        const Tensor2Read<float>& inputs, const AdjFn& adjOutput,
-                                                       const param_t& params, float* ldsGradients = nullptr)
+                                                       const param_t& params, float* ldsGradients = nullptr,
+                                                       const Trace& trace = Trace{})
     {
         constexpr int G = 2 * F;            // lanes per point
         constexpr int PPR = WAVE_SIZE / G;  // points per round
@@ -514,6 +555,10 @@ struct EncodingHashGrid
                     }
                     if (hashed) idx %= Cfg::hashGridSize[l];
                     const unsigned element = idx * static_cast<unsigned>(F) + static_cast<unsigned>(i);
+                    if constexpr (Trace::Enabled) {
+                        // where this lane would add, instead of adding: one slot per corner, from its feature-0 lane
+                        if (i == 0) trace.record((index * L + l) * NC + 2 * c + k, base + element, w * wk);
+                    } else
                     if (l < LDS_LEVELS)
                         ldsAdd(ldsGradients + (base - static_cast<unsigned>(Cfg::memoryOffset[0]) + element), (w * wk) * adj);
                     else
@@ -521,6 +566,33 @@ struct EncodingHashGrid
                 }
             }
         }
+    }
+
+    /** Test aid: what the gathers of the fused forward kernels (gatherLevel) read for this point:
+     *  element offset and weight per corner, slots as in CornerTrace. */
+    template <typename I>
+    __device__ __forceinline__ static void traceGather(const I& input, const param_t& params,
+                                                       unsigned* __restrict__ idx, float* __restrict__ w)
+    {
+        float pos[D];
+        unitPosition(input, params, pos);
+        const CornerTrace trace{idx, w};
+#pragma unroll
+        for (int l = 0; l < L; ++l) {
+            float feat[F];
+            gatherLevel(l, pos, params.parametersForward, feat, trace);
+            // the values are part of the trace kernel's result so that the loads stay in the program
+            if (feat[0] == 12345.678f) w[l * NC] = 0.f;
+        }
+    }
+
+    /** Test aid: where the gradient scatter of the fused backward kernel (scatterTile) adds for the
+     *  64 points from index0 on (called by a whole wavefront); slots of the whole batch. */
+    __device__ __forceinline__ static void traceScatter(int lane, long long index0, long long numel,
+                                                        const Tensor2Read<float>& inputs, const param_t& params,
+                                                        unsigned* __restrict__ idx, float* __restrict__ w)
+    {
+        scatterTile<0>(lane, index0, numel, inputs, [](int, int) { return 1.f; }, params, nullptr, CornerTrace{idx, w});
     }
 
     /** Writes the element offset and weight of every corner (index checks in tests). */

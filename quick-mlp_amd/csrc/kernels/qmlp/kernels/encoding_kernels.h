@@ -71,4 +71,39 @@ __global__ void EncodingCornersKernel(
     }
 }
 
+// Test aid: the same two arrays, written by the code the fused kernels run. MODE 1: the
+// gathers of the forward pass (one lane per point); MODE 2: the gradient scatter of the
+// backward pass (one wavefront per 64 points), which records where it would add.
+template <int MODE>
+__global__ void __launch_bounds__(256) EncodingTraceKernel(
+    long long numel,
+    const Tensor2Read<float> inputs,  //shape (numel, Cin)
+    unsigned* __restrict__ indices,   //shape (numel, perPoint)
+    float* __restrict__ weights,      //shape (numel, perPoint)
+    int perPoint
+    $$ENCODING_PARAMETERS$$)
+{
+    if constexpr (MODE == 1) {
+        for (long long index = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; index < numel;
+             index += static_cast<long long>(blockDim.x) * gridDim.x)
+        {
+            const StridedArray<const float> encodingInput{inputs.data_ + index * inputs.strides_[0], inputs.strides_[1]};
+            unsigned* cornerIndices = indices + index * perPoint;
+            float* cornerWeights = weights + index * perPoint;
+            (void)encodingInput; (void)cornerIndices; (void)cornerWeights;
+            $$CALL_ENCODINGS_TRACE_GATHER$$
+        }
+    } else {
+        const int lane = threadIdx.x % WAVE_SIZE;
+        const long long wavesPerBlock = blockDim.x / WAVE_SIZE;
+        const long long stride = wavesPerBlock * gridDim.x * TILE_POINTS;
+        (void)lane;
+        for (long long tileBase = (blockIdx.x * wavesPerBlock + threadIdx.x / WAVE_SIZE) * TILE_POINTS; tileBase < numel;
+             tileBase += stride)
+        {
+            $$CALL_ENCODINGS_TRACE_SCATTER$$
+        }
+    }
+}
+
 QUICKMLP_KERNEL_NAMESPACE_END

@@ -1,0 +1,462 @@
+// Parameter gradients of a grid encoding without a global atomic per contribution: the
+// contributions are first written as records into buckets, one bucket per slice of the gradient
+// table, and a workgroup per slice then sums its bucket in LDS and adds the slice to the gradient
+// tensor once.
+//
+// Float atomics on device memory complete at about 21e9 requests per second on the whole
+// device wherever the data lives, and a hashed level offers nothing to combine (a batch of
+// random points touches every entry about once). So the scatter of the fused backward kernel
+// (EncodingHashGrid::scatterTile, 4.5 requests per point and level) bounds a train step. Here
+// the backward kernel only stores the adjoint of the encoded rows. Then
+//   GridGradientRecordsKernel  walks over the points, one per lane, level by level: for every
+//       pair of corners that are neighbours in memory it forms a record (the two elements, their
+//       weights, the adjoint of the level's features), sorts the records of the workgroup by the
+//       slice of the gradient table they belong to (a slice is a run of up to 32 768 floats =
+//       128 KiB of LDS) in LDS, reserves room in the buckets of these slices with one atomic per
+//       slice and workgroup, and copies the sorted records there in runs: all loads and stores
+//       of this kernel are coalesced;
+//   GridGradientSlicesKernel   runs one workgroup per work item (level, slice, part of the
+//       bucket): it streams through its records and adds weight * adjoint to the slice in LDS,
+//       then adds the slice to the gradient tensor with atomics, 16 neighbouring floats per
+//       request (a coarse level has few slices that receive all records of the level; their
+//       buckets are shared out over several work items).
+// The sums in LDS are 64-bit fixed point, added with integer atomics: ds_add_f32 completes one
+// lane every three cycles on this hardware (0.32 lanes per clock and CU measured, whatever the
+// addresses), ds_add_u64 3.5 lanes per clock. The scale is a power of two chosen per launch from the
+// largest adjoint of the batch (which the records kernel finds on its way) and the number of
+// records, such that no sum can overflow: at least 40 bits remain below the largest
+// contribution, and the sums do not depend on the order of the additions. Batches whose
+// adjoints are not finite take the float additions, so that NaN and infinity reach the gradients.
+// Two forms that were measured and dropped: a workgroup per slice that tests every point of
+// the batch against its slice and recomputes the hits (the work of a hit falls to one lane of
+// 64, 890 us for 2^18 points and 16 levels), and the same with the hits queued in LDS first (the
+// queued hits gather their point's coordinates and adjoints at random: bound by line requests).
+// A bucket has room for 1.25 times its share of the records of a uniform batch; a record that
+// finds its bucket full is added to the gradient tensor with atomics by the lane that holds it.
+//
+// Replaces, for batches that are large enough, the atomicAdd of
+// src_cpp/include/qmlp/kernels/encoding_hashgrid.cuh:117-166,345-369 of the reference.
+
+#include <qmlp/kernels/common.h>
+#include <qmlp/kernels/encoding_hashgrid.h>
+
+QUICKMLP_KERNEL_NAMESPACE_BEGIN
+
+/** One work item of GridGradientSlicesKernel: the `floats` elements of the gradient table from
+ *  element `first` on (slice `slice` of level `level`), part `part` of `parts` of its bucket. */
+struct GridGradientSlice
+{
+    int level;
+    unsigned first;
+    int floats;
+    int slice;
+    int part;
+    int parts;       // > 1: other work items hold sums for the same slice, all add it with atomics
+    int reserved0;
+    int reserved1;
+};
+
+template <typename Cfg, int SLICE_FLOATS>
+struct GridGradientLayout
+{
+    typedef EncodingHashGrid<Cfg> Grid;
+    static constexpr int D = Grid::D;
+    static constexpr int F = Grid::F;
+    static constexpr int L = Grid::L;
+    static constexpr int PAIRS = Grid::NC / 2 > 0 ? Grid::NC / 2 : 1;
+    /** A record in 32-bit words: element of the lower and of the upper entry, their weights, F halves of adjoint. */
+    static constexpr int RECORD_WORDS = 4 + (F + 1) / 2;
+
+    __device__ __host__ static constexpr int levelFloats(int l)
+    {
+        return (l + 1 < L ? Cfg::memoryOffset[l + 1] : Cfg::ParameterCount) - Cfg::memoryOffset[l];
+    }
+    __device__ __host__ static constexpr int numSlices(int l) { return (levelFloats(l) + SLICE_FLOATS - 1) / SLICE_FLOATS; }
+    /** Records a bucket of level l holds for a batch of numel points. */
+    __device__ __host__ static constexpr long long capacity(int l, long long numel)
+    {
+        return ((5 * numel * PAIRS / 4) / numSlices(l) + 2048) & ~3ll;
+    }
+    /** Index of the first bucket of level l. */
+    __device__ __host__ static constexpr int firstBucket(int l)
+    {
+        int n = 0;
+        for (int k = 0; k < l; ++k) n += numSlices(k);
+        return n;
+    }
+    /** Offset in records of the first bucket of level l. */
+    __device__ __host__ static constexpr long long levelOffset(int l, long long numel)
+    {
+        long long n = 0;
+        for (int k = 0; k < l; ++k) n += numSlices(k) * capacity(k, numel);
+        return n;
+    }
+};
+
+template <typename Cfg, int ROW_CHANNELS, int CHANNEL_OFFSET, int SLICE_FLOATS, int POINTS>
+struct GridGradientRecords
+{
+    typedef GridGradientLayout<Cfg, SLICE_FLOATS> Layout;
+    typedef EncodingHashGrid<Cfg> Grid;
+    typedef typename Grid::param_t param_t;
+    static constexpr int D = Grid::D;
+    static constexpr int F = Grid::F;
+    static constexpr int PAIRS = Layout::PAIRS;
+    static constexpr int RW = Layout::RECORD_WORDS;
+    static constexpr int MAX_SLICES = 512;
+
+    /** The two table entries of pair c of a point (bit b of c: upper corner in the b-th dimension
+     *  other than the pair's own) and the weight of the pair without its own dimension. */
+    template <int LEVEL>
+    __device__ __forceinline__ static void pairEntries(const typename Grid::LevelSetup& s, int c, unsigned& idxL,
+                                                       unsigned& idxH, float& w)
+    {
+        constexpr bool hashed = Cfg::hashed[LEVEL];
+        constexpr int PD = hashed ? 0 : D - 1;   // the dimension whose two corners are neighbours in memory
+        unsigned rest = 0u;
+        w = 1.f;
+        int bit = 0;
+#pragma unroll
+        for (int d = D - 1; d >= 0; --d) {
+            if (d == PD) continue;
+            const bool hi = (c >> bit) & 1;
+            ++bit;
+            const unsigned t = hi ? s.termH[d] : s.termL[d];
+            rest = hashed ? (rest ^ t) : (rest + t);
+            w = w * (hi ? s.f[d] : (1.f - s.f[d]));
+        }
+        if (hashed) {
+            idxL = (rest ^ s.termL[PD]) % Cfg::hashGridSize[LEVEL];
+            idxH = (rest ^ s.termH[PD]) % Cfg::hashGridSize[LEVEL];
+        } else {
+            idxL = rest + s.termL[PD];
+            idxH = rest + s.termH[PD];
+        }
+    }
+
+    /** Adds a record to the gradient tensor itself (its bucket was full). */
+    __device__ __forceinline__ static void addToTensor(const unsigned (&rec)[RW], float* __restrict__ grad)
+    {
+        const float wL = __builtin_bit_cast(float, rec[2]), wH = __builtin_bit_cast(float, rec[3]);
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            const unsigned short bits = static_cast<unsigned short>(rec[4 + i / 2] >> (16 * (i % 2)));
+            const float adj = static_cast<float>(__builtin_bit_cast(f16, bits));
+            unsafeAtomicAdd(grad + rec[0] + i, wL * adj);
+            unsafeAtomicAdd(grad + rec[1] + i, wH * adj);
+        }
+    }
+
+    template <int LEVEL>
+    __device__ __forceinline__ static void runLevel(int p, bool valid, long long numel, const float (&pos)[D],
+                                                    const f16* __restrict__ adjEncoded, const param_t& params,
+                                                    unsigned* __restrict__ records, int* __restrict__ cursors,
+                                                    unsigned* sStage, unsigned short* sBucketOf, int* sHist,
+                                                    int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits)
+    {
+        constexpr bool hashed = Cfg::hashed[LEVEL];
+        constexpr int PD = hashed ? 0 : D - 1;
+        constexpr unsigned base = static_cast<unsigned>(Cfg::memoryOffset[LEVEL]);
+        constexpr int NS = Layout::numSlices(LEVEL);
+        static_assert(NS <= MAX_SLICES, "the slice of a record is kept in the histogram arrays");
+        const int tid = threadIdx.x;
+        for (int b = tid; b < NS; b += POINTS) sHist[b] = 0;
+        __syncthreads();   // also: the staging area of the previous level has been copied out
+
+        // my records of this level, in registers, and their places among the workgroup's records of the same slice
+        unsigned rec[PAIRS][RW];
+        int bucket[PAIRS], rank[PAIRS];
+        if (valid) {
+            const typename Grid::LevelSetup s = Grid::setupLevel(LEVEL, pos);
+            const f16* adjRow = adjEncoded + static_cast<long long>(p / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
+                + (CHANNEL_OFFSET + (Cfg::Concat ? LEVEL * F : 0)) * TILE_POINTS + (p % TILE_POINTS);
+            unsigned adjWords[(F + 1) / 2];
+#pragma unroll
+            for (int i = 0; i < (F + 1) / 2; ++i) adjWords[i] = 0u;
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                const unsigned bits = __builtin_bit_cast(unsigned short, adjRow[i * TILE_POINTS]);
+                adjWords[i / 2] |= bits << (16 * (i % 2));
+                // largest magnitude seen (as fp16 bits without the sign: ordered like the values, NaN above infinity)
+                maxAdjBits = max(maxAdjBits, bits & 0x7fffu);
+            }
+#pragma unroll
+            for (int c = 0; c < PAIRS; ++c) {
+                unsigned idxL, idxH;
+                float w;
+                pairEntries<LEVEL>(s, c, idxL, idxH, w);
+                rec[c][0] = base + idxL * F;
+                rec[c][1] = base + idxH * F;
+                rec[c][2] = __builtin_bit_cast(unsigned, w * (1.f - s.f[PD]));
+                rec[c][3] = __builtin_bit_cast(unsigned, w * s.f[PD]);
+#pragma unroll
+                for (int i = 0; i < (F + 1) / 2; ++i) rec[c][4 + i] = adjWords[i];
+                bucket[c] = static_cast<int>(idxL * F / SLICE_FLOATS);   // the slice of the lower entry files the record
+                // (a level of one slice needs no sorting: every lane has fixed places)
+                rank[c] = NS == 1 ? tid * PAIRS + c : atomicAdd(sHist + bucket[c], 1);
+            }
+        } else {
+            // lanes beyond the batch: in a level of one slice they fill their fixed places with records that add nothing
+#pragma unroll
+            for (int c = 0; c < PAIRS; ++c) {
+                rec[c][0] = rec[c][1] = base;
+#pragma unroll
+                for (int v = 2; v < RW; ++v) rec[c][v] = 0u;
+                bucket[c] = 0;
+                rank[c] = tid * PAIRS + c;
+            }
+        }
+        if (NS == 1 && tid == 0) sHist[0] = POINTS * PAIRS;
+        __syncthreads();
+
+        // places of the slices in the staging area, and room in their buckets (one atomic per slice)
+        if (tid < 64) {
+            int running = 0;
+            for (int b0 = 0; b0 < NS; b0 += 64) {
+                const int b = b0 + tid;
+                const int n = b < NS ? sHist[b] : 0;
+                int inclusive = n;
+#pragma unroll
+                for (int d = 1; d < 64; d *= 2) {
+                    const int other = __shfl_up(inclusive, d, 64);
+                    if (tid >= d) inclusive += other;
+                }
+                if (b < NS) {
+                    sLocalBase[b] = running + inclusive - n;
+                    sGlobalBase[b] = n > 0 ? static_cast<long long>(atomicAdd(cursors + Layout::firstBucket(LEVEL) + b, n)) : 0;
+                }
+                running += __shfl(inclusive, 63, 64);
+            }
+            if (tid == 0) sLocalBase[NS] = running;
+        }
+        __syncthreads();
+
+        if (valid || NS == 1) {
+#pragma unroll
+            for (int c = 0; c < PAIRS; ++c) {
+                const int at = sLocalBase[bucket[c]] + rank[c];
+#pragma unroll
+                for (int v = 0; v < RW; ++v) sStage[at * RW + v] = rec[c][v];
+                sBucketOf[at] = static_cast<unsigned short>(bucket[c]);
+            }
+        }
+        __syncthreads();
+
+        // sorted by slice: consecutive lanes copy consecutive records of a bucket
+        const int total = sLocalBase[NS];
+        const long long capacity = Layout::capacity(LEVEL, numel);
+        unsigned* levelRecords = records + Layout::levelOffset(LEVEL, numel) * RW;
+        for (int j = tid; j < total; j += POINTS) {
+            const int b = sBucketOf[j];
+            const long long at = sGlobalBase[b] + (j - sLocalBase[b]);
+            unsigned r[RW];
+#pragma unroll
+            for (int v = 0; v < RW; ++v) r[v] = sStage[j * RW + v];
+            if (at < capacity) {
+                unsigned* dst = levelRecords + (static_cast<long long>(b) * capacity + at) * RW;
+#pragma unroll
+                for (int v = 0; v < RW; ++v) dst[v] = r[v];
+            } else {
+                addToTensor(r, params.parametersBackward);
+            }
+        }
+    }
+
+    template <int LEVEL>
+    __device__ __forceinline__ static void runLevels(int p, bool valid, long long numel, const float (&pos)[D],
+                                                     const f16* __restrict__ adjEncoded, const param_t& params,
+                                                     unsigned* __restrict__ records, int* __restrict__ cursors,
+                                                     unsigned* sStage, unsigned short* sBucketOf, int* sHist,
+                                                     int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits)
+    {
+        if constexpr (LEVEL < Cfg::Levels) {
+            runLevel<LEVEL>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf, sHist, sLocalBase,
+                            sGlobalBase, maxAdjBits);
+            runLevels<LEVEL + 1>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf, sHist, sLocalBase,
+                                 sGlobalBase, maxAdjBits);
+        }
+    }
+};
+
+/**
+ * \tparam POINTS points (= lanes) of a workgroup; its records of one level are staged in LDS
+ * records: room for levelOffset(Levels, layoutNumel) records; cursors: one int per bucket, then one word that
+ * receives the largest magnitude among the adjoints (fp16 bits without the sign); all zeroed by the caller.
+ */
+template <typename Cfg, int ROW_CHANNELS, int CHANNEL_OFFSET, int SLICE_FLOATS, int POINTS>
+__global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
+    int numel,
+    int layoutNumel,                          //points the buckets are laid out for (numel rounded up to whole tiles)
+    const Tensor2Read<float> inputs,          //shape (numel, Cin)
+    const half* __restrict__ adjEncodedH,     //adjoint of the encoded rows: (tiles, ROW_CHANNELS, 64)
+    const HashGridParams<typename Cfg::table_t, Cfg::Dim> params,
+    unsigned* __restrict__ records, int* __restrict__ cursors)
+{
+    typedef GridGradientRecords<Cfg, ROW_CHANNELS, CHANNEL_OFFSET, SLICE_FLOATS, POINTS> Impl;
+    constexpr int D = Cfg::Dim;
+    extern __shared__ __align__(16) unsigned char sMemory[];
+    unsigned* sStage = reinterpret_cast<unsigned*>(sMemory);                               // POINTS * PAIRS records
+    long long* sGlobalBase = reinterpret_cast<long long*>(sStage + POINTS * Impl::PAIRS * Impl::RW);
+    int* sHist = reinterpret_cast<int*>(sGlobalBase + Impl::MAX_SLICES);
+    int* sLocalBase = sHist + Impl::MAX_SLICES;
+    unsigned short* sBucketOf = reinterpret_cast<unsigned short*>(sLocalBase + Impl::MAX_SLICES + 1);
+    unsigned maxAdjBits = 0u;
+    for (int chunk = blockIdx.x * POINTS; chunk < numel; chunk += gridDim.x * POINTS) {
+        const int p = chunk + threadIdx.x;
+        const bool valid = p < numel;
+        float pos[D];
+        {
+#pragma clang fp contract(off)
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                const float in = valid ? inputs.data_[static_cast<long long>(p) * inputs.strides_[0]
+                                                      + static_cast<long long>(d + Cfg::Start) * inputs.strides_[1]] : 0.f;
+                pos[d] = (in - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
+            }
+        }
+        Impl::template runLevels<0>(p, valid, layoutNumel, pos, reinterpret_cast<const f16*>(adjEncodedH), params, records, cursors,
+                                    sStage, sBucketOf, sHist, sLocalBase, sGlobalBase, maxAdjBits);
+        __syncthreads();
+    }
+    // the largest adjoint of the workgroup: one LDS word, then one atomic per workgroup
+    if (threadIdx.x == 0) sHist[0] = 0;
+    __syncthreads();
+    if (maxAdjBits != 0u) atomicMax(sHist, static_cast<int>(maxAdjBits));
+    __syncthreads();
+    if (threadIdx.x == 0 && sHist[0] != 0)
+        atomicMax(cursors + GridGradientLayout<Cfg, SLICE_FLOATS>::firstBucket(Cfg::Levels), sHist[0]);
+}
+
+template <typename Cfg, int SLICE_FLOATS>
+struct GridGradientSlices
+{
+    typedef GridGradientLayout<Cfg, SLICE_FLOATS> Layout;
+    typedef EncodingHashGrid<Cfg> Grid;
+    static constexpr int F = Grid::F;
+    static constexpr int RW = Layout::RECORD_WORDS;
+    static constexpr int BLOCK = 1024;
+
+    /** v * 2^scaleExponent as a 64-bit integer, rounded towards minus infinity in the low word (|v * 2^scaleExponent| < 2^62). */
+    __device__ __forceinline__ static long long toFixed(float v, int scaleExponent)
+    {
+        const float x = ldexpf(v, scaleExponent - 32);             // in units of 2^32
+        const float hi = floorf(x);
+        // the low bits of a 24-bit mantissa: exact, in [0, 2^32) (a tiny negative x gives hi = -1 and x - hi = 1 after rounding)
+        const float lo = fminf(ldexpf(x - hi, 32), 4294967040.f);
+        return (static_cast<long long>(static_cast<int>(hi)) << 32) + static_cast<long long>(static_cast<unsigned>(lo));
+    }
+
+    __device__ __forceinline__ static void ldsAddFixed(long long* p, long long v)
+    {
+        typedef __attribute__((address_space(3))) unsigned long long lds_u64;
+        __hip_atomic_fetch_add((lds_u64*)p, static_cast<unsigned long long>(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+
+    /** FIXED: 64-bit fixed-point sums (the slice is SLICE_FLOATS long long); else float sums. */
+    template <int LEVEL, bool FIXED>
+    __device__ __forceinline__ static void sumRecords(long long numel, const unsigned* __restrict__ records,
+                                                      const int* __restrict__ cursors, float* __restrict__ gradients,
+                                                      const GridGradientSlice item, long long* sFixed, float* sFloat,
+                                                      int scaleExponent)
+    {
+        const int tid = threadIdx.x;
+        const long long capacity = Layout::capacity(LEVEL, numel);
+        const long long filled = min(static_cast<long long>(cursors[Layout::firstBucket(LEVEL) + item.slice]), capacity);
+        const long long begin = filled * item.part / item.parts, end = filled * (item.part + 1) / item.parts;
+        const unsigned* bucket = records + (Layout::levelOffset(LEVEL, numel) + static_cast<long long>(item.slice) * capacity) * RW;
+        const unsigned first = item.first, count = static_cast<unsigned>(item.floats);
+        constexpr int UNROLL = 4;
+        for (long long j0 = begin + tid; j0 < end; j0 += UNROLL * BLOCK) {
+            unsigned rec[UNROLL][RW];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const long long j = j0 + u * BLOCK;
+#pragma unroll
+                for (int v = 0; v < RW; ++v) rec[u][v] = j < end ? bucket[j * RW + v] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (j0 + u * BLOCK >= end) continue;
+                const unsigned eL = rec[u][0] - first, eH = rec[u][1] - first;   // unsigned: one compare tells whether it is inside
+                const float wL = __builtin_bit_cast(float, rec[u][2]), wH = __builtin_bit_cast(float, rec[u][3]);
+#pragma unroll
+                for (int i = 0; i < F; ++i) {
+                    const unsigned short bits = static_cast<unsigned short>(rec[u][4 + i / 2] >> (16 * (i % 2)));
+                    const float adj = static_cast<float>(__builtin_bit_cast(f16, bits));
+                    // the lower entry files the record, so it lies in this slice; the upper one may lie in the next
+                    if (eL < count) {
+                        if constexpr (FIXED) ldsAddFixed(sFixed + eL + i, toFixed(wL * adj, scaleExponent));
+                        else Grid::ldsAdd(sFloat + eL + i, wL * adj);
+                    } else {
+                        unsafeAtomicAdd(gradients + rec[u][0] + i, wL * adj);
+                    }
+                    if (eH < count) {
+                        if constexpr (FIXED) ldsAddFixed(sFixed + eH + i, toFixed(wH * adj, scaleExponent));
+                        else Grid::ldsAdd(sFloat + eH + i, wH * adj);
+                    } else {
+                        unsafeAtomicAdd(gradients + rec[u][1] + i, wH * adj);
+                    }
+                }
+            }
+        }
+    }
+
+    template <int LEVEL>
+    __device__ __forceinline__ static void runLevel(long long numel, const unsigned* __restrict__ records,
+                                                    const int* __restrict__ cursors, float* __restrict__ gradients,
+                                                    const GridGradientSlice item, long long* sSlice)
+    {
+        const int tid = threadIdx.x;
+        for (int i = tid; i < item.floats; i += BLOCK) sSlice[i] = 0;
+        __syncthreads();
+        // |adjoint| < 2^maxExponent; a sum has at most 2 * PAIRS * numel terms, each at most that large (weights <= 1)
+        const unsigned maxBits = static_cast<unsigned>(cursors[Layout::firstBucket(Cfg::Levels)]);
+        if (maxBits == 0u) return;   // all adjoints are zero: nothing to add
+        const bool finite = maxBits < 0x7c00u;
+        const int maxExponent = static_cast<int>(maxBits >> 10) - 14;          // fp16: value < 2^(biased exponent - 14), subnormals included
+        const int termsLog2 = 64 - __builtin_clzll(static_cast<unsigned long long>(2 * Layout::PAIRS) * static_cast<unsigned long long>(numel));
+        const int scaleExponent = 61 - maxExponent - termsLog2;
+        float* sFloat = reinterpret_cast<float*>(sSlice);
+        if (finite) sumRecords<LEVEL, true>(numel, records, cursors, gradients, item, sSlice, sFloat, scaleExponent);
+        else sumRecords<LEVEL, false>(numel, records, cursors, gradients, item, sSlice, sFloat, 0);
+        __syncthreads();
+        // Added to the gradient tensor with atomics, 16 neighbouring floats per request: other work items
+        // may hold sums for the same slice (parts > 1), and a record whose upper entry lies in the next
+        // slice is added there with an atomic while that slice's owner is at work.
+        float* __restrict__ grad = gradients + item.first;
+        for (int i = tid; i < item.floats; i += BLOCK) {
+            float v;
+            if (finite) {
+                const long long fixed = sSlice[i];
+                v = static_cast<float>(ldexp(static_cast<double>(fixed), -scaleExponent));
+            } else {
+                v = sFloat[i];
+            }
+            if (v != 0.f) unsafeAtomicAdd(grad + i, v);
+        }
+    }
+
+    template <int LEVEL>
+    __device__ __forceinline__ static void dispatch(long long numel, const unsigned* __restrict__ records,
+                                                    const int* __restrict__ cursors, float* __restrict__ gradients,
+                                                    const GridGradientSlice item, long long* sSlice)
+    {
+        if constexpr (LEVEL < Cfg::Levels) {
+            if (item.level == LEVEL) runLevel<LEVEL>(numel, records, cursors, gradients, item, sSlice);
+            else dispatch<LEVEL + 1>(numel, records, cursors, gradients, item, sSlice);
+        }
+    }
+};
+
+/** One workgroup of 1024 lanes per work item; `items` is indexed by the workgroup; SLICE_FLOATS * 8 bytes of dynamic LDS. */
+template <typename Cfg, int SLICE_FLOATS>
+__global__ void __launch_bounds__(1024) GridGradientSlicesKernel(
+    int numel, const unsigned* __restrict__ records, const int* __restrict__ cursors, float* __restrict__ gradients,
+    const GridGradientSlice* __restrict__ items)
+{
+    extern __shared__ __align__(16) unsigned char sMemory[];
+    GridGradientSlices<Cfg, SLICE_FLOATS>::template dispatch<0>(numel, records, cursors, gradients, items[blockIdx.x],
+                                                                reinterpret_cast<long long*>(sMemory));
+}
+
+QUICKMLP_KERNEL_NAMESPACE_END

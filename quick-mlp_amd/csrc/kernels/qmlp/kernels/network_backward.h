@@ -76,6 +76,12 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     constexpr bool HAS_STREAMED_LAYERS = $$HAS_STREAMED_LAYERS$$;
     // the adjoint of the encoded input is only needed if something sits behind it
     constexpr bool NEEDS_ENCODING_ADJOINT = HAS_INPUT_GRADIENTS || HAS_ENCODING_GRADIENTS;
+    // true: the adjoint of the encoded rows is stored (channel-major per tile, behind the adjoint
+    // pre-activations) for the kernels that sum the parameter gradients of grids slice by slice
+    constexpr bool STORE_ENCODED_ADJOINT = $$STORE_ENCODED_ADJOINT$$;
+    constexpr int OFFSET_ENCODED_ADJOINT = $$OFFSET_ENCODED_ADJOINT$$;   // channels in front of that region
+    // false: nothing in this kernel reads the adjoint of an encoded row point by point
+    constexpr bool NEEDS_STAGED_ADJOINT = $$NEEDS_STAGED_ADJOINT$$;
     (void)ENCODED_CHANNELS; (void)NUM_INPUTS; (void)KT0; (void)STAGE_STRIDE;
 
     const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
@@ -161,7 +167,20 @@ $$ZERO_LDS_GRADIENTS$$
         // layers, last to first
 $$CALL_NETWORK_LAYERS$$
 
-        if constexpr (NEEDS_ENCODING_ADJOINT) {
+        if constexpr (STORE_ENCODED_ADJOINT) {
+            if (tileValid) {
+                f16* adjTile = adjointTmpMemory + (static_cast<long long>(OFFSET_ENCODED_ADJOINT) * numel64
+                                                   + static_cast<long long>(tile) * (CHANNELS_IN * TILE_POINTS));
+#pragma unroll
+                for (int t = 0; t < KT0; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const f16x4 v = {dxIn[0][t][i], dxIn[1][t][i], dxIn[2][t][i], dxIn[3][t][i]};
+                        *reinterpret_cast<f16x4*>(adjTile + (16 * t + 4 * g + i) * TILE_POINTS + 4 * r) = v;
+                    }
+            }
+        }
+        if constexpr (NEEDS_ENCODING_ADJOINT && NEEDS_STAGED_ADJOINT) {
             // adjoint of the encoded input: registers -> one staging row per point
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)

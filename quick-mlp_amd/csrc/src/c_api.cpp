@@ -475,6 +475,17 @@ int qmlp_encoding_hashgrid_corners(qmlp_encoding_t encoding, const qmlp_tensor* 
     QMLP_API_END
 }
 
+int qmlp_encoding_hashgrid_trace(qmlp_encoding_t encoding, const qmlp_tensor* input, int mode, uint32_t* indices,
+                                 float* weights, void* stream)
+{
+    QMLP_API_BEGIN
+    if (input == nullptr)
+        asHashGrid(encoding).precompileCorners(mode, true);
+    else
+        asHashGrid(encoding).corners(wrap(input), indices, weights, static_cast<stream_t>(stream), mode);
+    QMLP_API_END
+}
+
 // ---------------------------------------------------------------- activations
 
 int qmlp_activation_create(const char* key_or_json, qmlp_activation_t* activation)

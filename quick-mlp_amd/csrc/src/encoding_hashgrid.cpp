@@ -1,5 +1,6 @@
 #include <qmlp/encoding_hashgrid.h>
 
+#include <qmlp/fused_network.h>
 #include <qmlp/qmlp.h>
 
 #include <cmath>
@@ -275,6 +276,41 @@ int EncodingHashGrid::ldsGradientFloats(int maxBytes, int& levels) const
         floats = upTo;
     }
     return floats;
+}
+
+bool EncodingHashGrid::gradientSlices(GradientSliceLayout& layout) const
+{
+    if (dimension_ > 4 || numParameters_ >= (1 << 30)) return false;   // up to 8 records per point and level in registers
+    const int lds = FusedNetwork::MaxSharedMemoryBytes();
+    // the slice kernel sums in 64-bit fixed point: 8 bytes of LDS per element
+    const int entries = std::min(16384, lds / 8) / numFeaturesPerLevel_;
+    if (entries < 64) return false;
+    layout = GradientSliceLayout{};
+    layout.sliceFloats = entries * numFeaturesPerLevel_;
+    layout.configType = "qmlp::kernel::" + configName();
+    layout.pairs = std::max(1, (1 << dimension_) / 2);
+    layout.recordWords = 4 + (numFeaturesPerLevel_ + 1) / 2;
+    // the records of a workgroup and level are sorted in LDS: 96 KiB for them, the rest for the book-keeping
+    int points = 1024;
+    while (points > 64 && points * layout.pairs * layout.recordWords * 4 > 96 * 1024) points /= 2;
+    layout.pointsPerWorkgroup = points;
+    layout.recordsLdsBytes = points * layout.pairs * (layout.recordWords * 4 + 2) + 512 * 8 + (2 * 512 + 1) * 4 + 64;
+    if (layout.recordsLdsBytes > lds) return false;
+    // every level gets about this many work items: the bucket of a slice that holds more than its share is split
+    constexpr int ITEMS_PER_LEVEL = 32;
+    for (int l = 0; l < numLevels_; ++l) {
+        const int begin = layers_[l].memoryOffset;
+        const int end = l + 1 < numLevels_ ? layers_[l + 1].memoryOffset : numParameters_;
+        const int count = divUp(end - begin, layout.sliceFloats);
+        if (count > 512) return false;   // the records kernel keeps a histogram of 512 slices
+        layout.slicesPerLevel.push_back(count);
+        const int parts = std::max(1, ITEMS_PER_LEVEL / count);
+        for (int k = 0; k < count; ++k)
+            for (int part = 0; part < parts; ++part)
+                layout.items.push_back({l, static_cast<unsigned>(begin + k * layout.sliceFloats),
+                                        std::min(layout.sliceFloats, end - begin - k * layout.sliceFloats), k, part, parts, 0, 0});
+    }
+    return true;
 }
 
 void EncodingHashGrid::setParameter(const Tensor& tensor, Tensor::Usage usage)

@@ -76,6 +76,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         compileOptions_.registerStaging = options.value("register_staging", compileOptions_.registerStaging);
         compileOptions_.sortPoints = options.value("sort_points", compileOptions_.sortPoints);
         compileOptions_.directInput = options.value("direct_input", compileOptions_.directInput);
+        compileOptions_.sliceGradients = options.value("slice_gradients", compileOptions_.sliceGradients);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
             options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
@@ -685,7 +686,46 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool r
     return code;
 }
 
-int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding) const
+static bool offersSlices(const IEncoding& e, IEncoding::GradientSliceLayout* layout = nullptr)
+{
+    IEncoding::GradientSliceLayout local;
+    return e.hasParameters() && e.gradientSlices(layout ? *layout : local);
+}
+
+bool FusedNetwork::hasSliceGradients() const
+{
+    if (compileOptions_.sliceGradients == 0) return false;
+    for (const auto& e : encodings_)
+        if (offersSlices(*e)) return true;
+    return false;
+}
+
+int FusedNetwork::sliceGradientBytesPerPoint() const
+{
+    // the adjoint of the encoded rows, which the records kernels of the grids read
+    return hasSliceGradients() ? layers_[0].channelsIn * static_cast<int>(sizeof(half)) : 0;
+}
+
+size_t FusedNetwork::sliceGradientWorkspaceBytes(long long numel) const
+{
+    if (!hasSliceGradients()) return 0;
+    size_t bytes = 0;
+    for (const auto& e : encodings_) {
+        IEncoding::GradientSliceLayout layout;
+        if (!offersSlices(*e, &layout)) continue;
+        bytes += roundUp(static_cast<size_t>(layout.numBuckets() + 1) * sizeof(int), size_t(256));   // cursors, largest adjoint
+        bytes += roundUp(static_cast<size_t>(layout.totalRecords(numel)) * layout.recordWords * sizeof(uint32_t), size_t(256));
+    }
+    return bytes;
+}
+
+bool FusedNetwork::useSliceGradients(int numel, int flags) const
+{
+    if (!(flags & GRADIENTS_INPUT_ENCODINGS) || !hasSliceGradients()) return false;
+    return compileOptions_.sliceGradients > 0 || numel >= SLICE_GRADIENTS_MIN_BATCH;
+}
+
+int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients) const
 {
     perEncoding.assign(encodings_.size(), LdsGradients{});
     int bytes = ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (blockSize / WARP_SIZE) * stageBytesPerWave(true);
@@ -695,6 +735,7 @@ int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector
     const int limit = std::min(MaxSharedMemoryBytes(), 96 * 1024);
     for (size_t i = 0; i < encodings_.size(); ++i) {
         if (!encodings_[i]->hasParameters()) continue;
+        if (sliceGradients && offersSlices(*encodings_[i])) continue;   // summed by the slice kernel, not here
         bytes = roundUp(bytes, 16);
         LdsGradients g;
         g.floats = encodings_[i]->ldsGradientFloats(limit - bytes, g.levels);
@@ -706,7 +747,7 @@ int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector
     return bytes;
 }
 
-std::string FusedNetwork::backwardSource(int flags, int blockSize) const
+std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGradients) const
 {
     const bool hasInputGradients = flags & GRADIENTS_INPUT;
     const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
@@ -778,11 +819,18 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
 
     std::stringstream callEncodings, callScatter, zeroLds, flushLds;
     std::vector<LdsGradients> ldsGradients;
-    ldsGradientLayout(flags, blockSize, ldsGradients);
+    ldsGradientLayout(flags, blockSize, ldsGradients, sliceGradients);
     int encodingOffset = 0;
+    bool storeEncodedAdjoint = false, gradientsInKernel = false;
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
-        const bool parameterGradients = hasEncodingGradients && e->hasParameters();
+        bool parameterGradients = hasEncodingGradients && e->hasParameters();
+        if (parameterGradients && sliceGradients && offersSlices(*e)) {
+            // this kernel only stores the adjoint of the encoded rows; a slice kernel sums the gradients
+            parameterGradients = false;
+            storeEncodedAdjoint = true;
+        }
+        gradientsInKernel = gradientsInKernel || parameterGradients;
         const std::string name = e->qualifiedName();
         const LdsGradients& lg = ldsGradients[encodingIdx];
         if (lg.levels > 0) {
@@ -812,6 +860,15 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize) const
         encodingOffset += e->numOutputChannels();
     }
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
+    replaceAll(code, "$$STORE_ENCODED_ADJOINT$$", storeEncodedAdjoint ? "true" : "false");
+    {
+        int adjointChannels = 0;
+        if (hasNetworkGradients)
+            for (const auto& l : layers_) adjointChannels += l.channelsOut;
+        replaceAll(code, "$$OFFSET_ENCODED_ADJOINT$$", std::to_string(adjointChannels));
+    }
+    // the adjoint of the encoded rows goes through the staging rows only if a lane per point still needs it
+    replaceAll(code, "$$NEEDS_STAGED_ADJOINT$$", (hasInputGradients || gradientsInKernel) ? "true" : "false");
     replaceAll(code, "$$CALL_ENCODING_SCATTER$$", callScatter.str());
     replaceAll(code, "$$ZERO_LDS_GRADIENTS$$", zeroLds.str());
     replaceAll(code, "$$FLUSH_LDS_GRADIENTS$$", flushLds.str().empty() ? std::string() : "    __syncthreads();\n" + flushLds.str());
@@ -1067,10 +1124,10 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
     return forwardKernels_[s][best].value();
 }
 
-void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
+void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool compileOnly)
 {
     if (flags <= 0 || flags >= ADJOINT_MODE_MAX_COMBINATIONS) throw std::runtime_error("At least one derivative must be enabled");
-    if (backwardKernel_[flags].has_value() && !compileOnly) return;
+    if (backwardKernel_[flags][sliceGradients ? 1 : 0].has_value() && !compileOnly) return;
     const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
     auto kl = QuickMLP::Instance().kernelLoader();
     auto logger = QuickMLP::Instance().getLogger();
@@ -1079,9 +1136,9 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
     ak.adjoint.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
     {
         std::vector<LdsGradients> ldsGradients;
-        ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients);
+        ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients, sliceGradients);
     }
-    const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize);
+    const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients);
     ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
     {
         std::vector<long long> transposed;
@@ -1100,6 +1157,42 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
     int adjointChannels = 0;
     for (const auto& l : layers_) adjointChannels += l.channelsOut;
     ak.perEntryAdjointMemoryBytes = hasNetworkGradients ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
+    // behind the adjoint pre-activations: the adjoint of the encoded rows for the records kernels
+    if (flags & GRADIENTS_INPUT_ENCODINGS) ak.perEntryAdjointMemoryBytes += sliceGradientBytesPerPoint();
+
+    if (sliceGradients && (flags & GRADIENTS_INPUT_ENCODINGS)) {
+        int channelOffset = 0;
+        for (size_t i = 0; i < encodings_.size(); ++i) {
+            const auto& e = encodings_[i];
+            const int offset = channelOffset;
+            channelOffset += e->numOutputChannels();
+            SliceGradientKernel sk;
+            if (!offersSlices(*e, &sk.layout)) continue;
+            const auto& layout = sk.layout;
+            sk.encoding = static_cast<int>(i);
+            std::stringstream source;
+            e->fillCode(source);
+            source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient.h");
+            sk.records.blockSize = layout.pointsPerWorkgroup;
+            sk.records.sharedMemorySize = layout.recordsLdsBytes;
+            sk.records.fun = kl->getKernel(format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d>", layout.configType.c_str(),
+                                                  layers_[0].channelsIn, offset, layout.sliceFloats, layout.pointsPerWorkgroup),
+                                           source.str(), loaderFlags(compileOnly)).value();
+            sk.kernel.blockSize = 1024;
+            sk.kernel.sharedMemorySize = layout.sliceFloats * static_cast<int>(sizeof(long long));
+            sk.kernel.fun = kl->getKernel(format("qmlp::kernel::GridGradientSlicesKernel<%s, %d>", layout.configType.c_str(), layout.sliceFloats),
+                                          source.str(), loaderFlags(compileOnly)).value();
+            if (!compileOnly) {
+                sk.records.fullGrid = sk.records.fun.fullGridSize(sk.records.blockSize, sk.records.sharedMemorySize);
+                static_assert(sizeof(IEncoding::GradientSlice) == 32, "eight 32-bit words, as in kernels/grid_gradient.h");
+                sk.items = Tensor(Tensor::FLOAT, {static_cast<int32_t>(layout.items.size() * 8)});
+                QMLP_HIP_CALL(qmlp_hip_memcpy_h2d(sk.items.rawPtr(), layout.items.data(), layout.items.size() * sizeof(layout.items[0]), nullptr));
+                logger->debug("gradient slices of encoding %d: %d buckets, %d work items, records kernel with %d points per workgroup (grid %d)",
+                              sk.encoding, layout.numBuckets(), static_cast<int>(layout.items.size()), layout.pointsPerWorkgroup, sk.records.fullGrid);
+            }
+            ak.sliceGradients.push_back(std::move(sk));
+        }
+    }
 
     if (hasNetworkGradients) {
         const int blockSize = weightUpdateBlockSize();
@@ -1124,7 +1217,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool compileOnly)
             }
         }
     }
-    if (!compileOnly) backwardKernel_[flags] = std::move(ak);
+    if (!compileOnly) backwardKernel_[flags][sliceGradients ? 1 : 0] = std::move(ak);
 }
 
 void FusedNetwork::precompile(int adjointFlags)
@@ -1137,7 +1230,11 @@ void FusedNetwork::precompile(int adjointFlags)
         if (hasLargeVariant(store)) compileForwardKernel(store, VARIANT_LARGE, true);
         if (registerVariantTiles(store) > 0) compileForwardKernel(store, VARIANT_REGISTERS, true);
     }
-    if (adjointFlags > 0) compileBackwardKernel(adjointFlags, true);
+    if (adjointFlags > 0) {
+        if (compileOptions_.sliceGradients <= 0 || !hasSliceGradients() || !(adjointFlags & GRADIENTS_INPUT_ENCODINGS))
+            compileBackwardKernel(adjointFlags, false, true);
+        if ((adjointFlags & GRADIENTS_INPUT_ENCODINGS) && hasSliceGradients()) compileBackwardKernel(adjointFlags, true, true);
+    }
     kernel::PointOrderKey key{};
     for (const auto& e : encodings_)
         if (compileOptions_.sortPoints != 0 && e->pointOrderKey(key)) {
@@ -1398,7 +1495,9 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
         throw std::runtime_error("At least one derivative must be enabled");
     int adjointChannels = 0;
     for (const auto& l : layers_) adjointChannels += l.channelsOut;
-    const int perEntry = (adjointFlags & GRADIENTS_NETWORK_WEIGHTS) ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
+    int perEntry = (adjointFlags & GRADIENTS_NETWORK_WEIGHTS) ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
+    // the adjoint of the encoded rows, which the records kernels of the grids read
+    if (adjointFlags & GRADIENTS_INPUT_ENCODINGS) perEntry += sliceGradientBytesPerPoint();
     numElements = roundUp(numElements, WARP_SIZE);
     size_t bytes = static_cast<size_t>(perEntry) * static_cast<size_t>(numElements);
     // behind the adjoint pre-activations: the partial weight gradients of the batch slices
@@ -1407,6 +1506,8 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
     // last: transposed copies of the weights the adjoint kernel cannot keep in LDS
     std::vector<long long> transposed;
     bytes += roundUp(transposedWeightLayout(adjointFlags, transposed) * sizeof(half), size_t(16));
+    // last: bucket cursors and records of the gradient slice kernels
+    if (adjointFlags & GRADIENTS_INPUT_ENCODINGS) bytes = roundUp(bytes, size_t(256)) + sliceGradientWorkspaceBytes(numElements);
     return bytes;
 }
 
@@ -1453,13 +1554,15 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     CHECK_ERROR(tmpMemoryForward != nullptr, "adjoint() needs the temporary memory written by forward()");
     std::vector<long long> transposedOffsets;
     const size_t transposedHalves = transposedWeightLayout(adjointFlags, transposedOffsets);
-    if (hasNetworkGradients || transposedHalves > 0) {
+    if (hasNetworkGradients || transposedHalves > 0 || useSliceGradients(numel, adjointFlags)) {
         CHECK_ERROR(tmpMemoryAdjoint != nullptr, "adjoint() needs temporary memory of adjointMemory() bytes");
         CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemoryAdjoint) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
     }
 
-    compileBackwardKernel(adjointFlags);
-    auto& ak = backwardKernel_[adjointFlags].value();
+    const bool sliceGradients = useSliceGradients(numel, adjointFlags);
+    CHECK_ERROR(!sliceGradients || numel < (1 << 27), "batches of 2^27 points or more: set options.slice_gradients to 0");
+    compileBackwardKernel(adjointFlags, sliceGradients);
+    auto& ak = backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value();
 
     const int numTiles = divUp(numel, TILE_POINTS);
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
@@ -1497,6 +1600,45 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+    }
+
+    // parameter gradients of the grids, slice by slice, from the adjoint of the encoded rows the kernel above stored
+    if (!ak.sliceGradients.empty()) {
+        int adjointChannels = 0;
+        if (hasNetworkGradients)
+            for (const auto& l : layers_) adjointChannels += l.channelsOut;
+        const half* adjEncoded = static_cast<const half*>(tmpMemoryAdjoint) + static_cast<ptrdiff_t>(adjointChannels) * numel64;
+        // the workspace is the last part of the adjoint memory: everything in front of it
+        size_t offset = static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64);
+        if (hasNetworkGradients) offset += static_cast<size_t>(weightUpdateSlices(numTiles)) * numParameters_ * sizeof(float);
+        offset += roundUp(transposedHalves * sizeof(half), size_t(16));
+        char* workspace = static_cast<char*>(tmpMemoryAdjoint) + roundUp(offset, size_t(256));
+        auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+        for (const auto& sk : ak.sliceGradients) {
+            const auto& layout = sk.layout;
+            int* cursors = reinterpret_cast<int*>(workspace);
+            const size_t cursorBytes = roundUp(static_cast<size_t>(layout.numBuckets() + 1) * sizeof(int), size_t(256));
+            uint32_t* records = reinterpret_cast<uint32_t*>(workspace + cursorBytes);
+            workspace += cursorBytes + roundUp(static_cast<size_t>(layout.totalRecords(numel64)) * layout.recordWords * sizeof(uint32_t), size_t(256));
+            QMLP_HIP_CALL(qmlp_hip_memset_async(cursors, 0, cursorBytes, stream));
+            std::vector<char> params(1024);
+            int n = encodings_[sk.encoding]->fillParameterMemory(params.data(), static_cast<int>(params.size()));
+            (void)n;
+            int numelPadded = static_cast<int>(numel64);   // the layout of the buckets is that of adjointMemory()
+            {
+                // the records kernel walks over the real points, but lays its buckets out for the padded batch
+                void* args[] = {&numel, &numelPadded, &inputAcc, &adjEncoded, params.data(), &records, &cursors};
+                sk.records.fun.launch(std::min(divUp(numel, sk.records.blockSize), sk.records.fullGrid), sk.records.blockSize,
+                                      sk.records.sharedMemorySize, stream, args);
+            }
+            const uint32_t* recordsRead = records;
+            const int* cursorsRead = cursors;
+            float* gradients = nullptr;
+            std::memcpy(&gradients, params.data() + sizeof(void*), sizeof(void*));   // HashGridParams: forward table, gradient table, ...
+            const void* items = sk.items.rawPtr();
+            void* args[] = {&numelPadded, &recordsRead, &cursorsRead, &gradients, &items};
+            sk.kernel.fun.launch(static_cast<int>(layout.items.size()), sk.kernel.blockSize, sk.kernel.sharedMemorySize, stream, args);
+        }
     }
 
     if (!hasNetworkGradients) return;
@@ -1546,7 +1688,7 @@ void FusedNetwork::clearCachedKernels()
 {
     for (auto& perStore : forwardKernels_)
         for (auto& k : perStore) k = {};
-    for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i) backwardKernel_[i] = {};
+    for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i) backwardKernel_[i][0] = backwardKernel_[i][1] = {};
     pointOrder_.scan = {};
     pointOrder_.count = {};
     pointOrder_.scatter = {};

@@ -20,7 +20,8 @@ struct ArgPack
 };
 
 std::string standaloneSource(const IEncoding& e, const std::string& callForward, const std::string& callAdjoint,
-                             const std::string& callCorners = "", const std::string& callScatter = "")
+                             const std::string& callCorners = "", const std::string& callScatter = "",
+                             const std::string& callTraceGather = "", const std::string& callTraceScatter = "")
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string codeTemplate = kl->findFile("qmlp/kernels/encoding_kernels.h").value();
@@ -34,6 +35,8 @@ std::string standaloneSource(const IEncoding& e, const std::string& callForward,
     replaceAll(codeTemplate, "$$CALL_ENCODINGS_ADJOINT$$", callAdjoint);
     replaceAll(codeTemplate, "$$CALL_ENCODINGS_CORNERS$$", callCorners);
     replaceAll(codeTemplate, "$$CALL_ENCODINGS_SCATTER$$", callScatter);
+    replaceAll(codeTemplate, "$$CALL_ENCODINGS_TRACE_GATHER$$", callTraceGather);
+    replaceAll(codeTemplate, "$$CALL_ENCODINGS_TRACE_SCATTER$$", callTraceScatter);
     return codeTemplate;
 }
 
@@ -170,29 +173,46 @@ void IEncoding::adjoint(const Tensor& input, const Tensor& adjOutput, Tensor& ad
     if (hasParameters() && parametersGradients.has_value()) setParameter({}, Tensor::GRADIENTS);
 }
 
-void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* weights, stream_t stream)
+void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* weights, stream_t stream, int mode)
 {
     CHECK_DIM(input, 2);
     CHECK_DTYPE(input, Tensor::FLOAT);
     CHECK_ERROR(input.size(1) > maxInputChannel());
+    CHECK_ERROR(mode >= 0 && mode <= 2, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter");
+    CHECK_ERROR(mode != 2 || (numFeaturesPerLevel_ & (numFeaturesPerLevel_ - 1)) == 0 && numFeaturesPerLevel_ <= 32,
+                "the tile-wide gradient scatter exists for 1, 2, 4 .. 32 features per level");
+    CHECK_ERROR(mode == 0 || hasParameterTensor(Tensor::INFERENCE), "the traces read the table: bind one first");
     long long numel = input.size(0);
     if (numel == 0) return;
-    if (!cornersKernel_.has_value()) {
-        std::string call = qualifiedName() + "::corners(encodingInput, cEncoding, cornerIndices, cornerWeights);\n";
-        std::string source = standaloneSource(*this, "", "", call);
-        cornersKernel_ = QuickMLP::Instance().kernelLoader()->getKernel(
-            "qmlp::kernel::EncodingCornersKernel", source, QuickMLP::Instance().getCompileFlags()).value();
-    }
-    auto& fun = cornersKernel_.value();
+    if (!cornersKernel_[mode].has_value()) precompileCorners(mode, false);
+    auto& fun = cornersKernel_[mode].value();
     std::vector<char> paramBytes(4096);
     int n = fillParameterMemory(paramBytes.data(), static_cast<int>(paramBytes.size()));
     (void)n;
     const int block = 256;
+    // modes 0 and 1: a lane per point; mode 2: a wavefront per 64 points
     const int grid = static_cast<int>(std::min<long long>(divUp<long long>(numel, block), fun.fullGridSize(block, 0)));
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     int perPoint = numLevels() * (1 << ndim());
     void* args[] = {&numel, &inputAcc, &indices, &weights, &perPoint, paramBytes.data()};
     fun.launch(grid, block, 0, stream, args);
+}
+
+void EncodingHashGrid::precompileCorners(int mode, bool compileOnly)
+{
+    CHECK_ERROR(mode >= 0 && mode <= 2, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter");
+    {
+        const std::string name = qualifiedName();
+        const std::string source = standaloneSource(
+            *this, "", "", name + "::corners(encodingInput, cEncoding, cornerIndices, cornerWeights);\n", "",
+            name + "::traceGather(encodingInput, cEncoding, cornerIndices, cornerWeights);\n",
+            name + "::traceScatter(lane, tileBase, numel, inputs, cEncoding, indices, weights);\n");
+        const char* kernels[] = {"qmlp::kernel::EncodingCornersKernel", "qmlp::kernel::EncodingTraceKernel<1>",
+                                 "qmlp::kernel::EncodingTraceKernel<2>"};
+        const int flags = QuickMLP::Instance().getCompileFlags() | (compileOnly ? KernelLoader::CompileOnly : 0);
+        auto kernel = QuickMLP::Instance().kernelLoader()->getKernel(kernels[mode], source, flags);
+        if (!compileOnly) cornersKernel_[mode] = kernel.value();
+    }
 }
 
 EncodingFactory::EncodingFactory()

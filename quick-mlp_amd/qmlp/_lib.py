@@ -95,6 +95,7 @@ _SIGNATURES = {
     "qmlp_encoding_adjoint": [_vp, _TD, _TD, _TD, _vp, _TD, _TD, _ci],
     "qmlp_encoding_hashgrid_levels": [_vp, _ci, _pi, _pi, _pi, _pi, _pi],
     "qmlp_encoding_hashgrid_corners": [_vp, _TD, _vp, _vp, _vp],
+    "qmlp_encoding_hashgrid_trace": [_vp, _TD, _ci, _vp, _vp, _vp],
     "qmlp_encoding_precompile": [_vp, _ci],
     "qmlp_activation_create": [ctypes.c_char_p, _P(_vp)],
     "qmlp_activation_destroy": [_vp],

@@ -221,15 +221,20 @@ class Encoding:
         off, res, hs, hashed = arrs
         return [(res[l], bool(hashed[l]), off[l], hs[l]) for l in range(n.value)]
 
-    def hashgrid_corners(self, input):
-        """Device-computed table offsets and weights, shape (N, levels, 2^dim)."""
+    def hashgrid_corners(self, input, mode=0):
+        """Device-computed table offsets and weights, shape (N, levels, 2^dim). mode 0: the index
+        function; 1: what the gathers of the fused forward kernels use (bind a table first);
+        2: what the gradient scatter of the fused backward kernel adds to."""
+        if input is None:      # compile the kernel of this mode into the kernel cache, nothing runs
+            check(lib.qmlp_encoding_hashgrid_trace(self._handle, None, int(mode), None, None, None))
+            return None
         levels = self.hashgrid_levels()
         dim = int(json.loads(self.to_json())["n_in"])
         n = input.shape[0]
-        idx = torch.zeros((n, len(levels), 1 << dim), dtype=torch.int32, device=input.device)
-        w = torch.zeros((n, len(levels), 1 << dim), dtype=torch.float32, device=input.device)
-        check(lib.qmlp_encoding_hashgrid_corners(self._handle, desc(input), idx.data_ptr(), w.data_ptr(),
-                                                 current_stream(input.device)))
+        idx = torch.full((n, len(levels), 1 << dim), -1, dtype=torch.int32, device=input.device)
+        w = torch.full((n, len(levels), 1 << dim), float("nan"), dtype=torch.float32, device=input.device)
+        check(lib.qmlp_encoding_hashgrid_trace(self._handle, desc(input), int(mode), idx.data_ptr(), w.data_ptr(),
+                                               current_stream(input.device)))
         return idx, w
 
     def inference(self, input):

@@ -4,6 +4,7 @@ oracle on the same seeded inputs. Shapes follow the reference's own tests
 tests_py/qmlp_tests/test_network_base.py:87-256). Tolerance of every floating point
 comparison: rel 1e-2 / abs 1e-3 against the fp32 oracle, no entry may exceed it."""
 import json
+import os
 
 import numpy as np
 import pytest
@@ -220,13 +221,40 @@ def _grid_cfg(spec, precision="float", start=0):
     return cfg
 
 
-@pytest.mark.parametrize("spec", GRID_SPECS + [bc.hashgrid3d("float")])
+def _per_point_sets(idx, w):
+    """Per point and level the table entries sorted by index, with the weights of equal entries
+    (corners that coincide at a clamped border, or that collide in a hashed level) added up."""
+    idx = np.asarray(idx).astype(np.int64)
+    order = np.argsort(idx, axis=-1, kind="stable")
+    idx = np.take_along_axis(idx, order, -1)
+    w = np.take_along_axis(np.asarray(w, np.float64), order, -1)
+    # running sum of the weights over runs of equal indices, kept at the last entry of each run
+    same = np.concatenate([np.zeros(idx.shape[:-1] + (1,), bool), idx[..., 1:] == idx[..., :-1]], -1)
+    acc = w.copy()
+    for k in range(1, idx.shape[-1]):
+        acc[..., k] += np.where(same[..., k], acc[..., k - 1], 0.0)
+    last = np.concatenate([idx[..., 1:] != idx[..., :-1], np.ones(idx.shape[:-1] + (1,), bool)], -1)
+    return idx, np.where(last, acc, 0.0)
+
+
+@pytest.mark.parametrize("spec", GRID_SPECS + [bc.hashgrid3d("float"), bc.hashgrid3d("half"), bc.densegrid4d("half")])
 def test_grid_indices_are_bit_exact(spec):
-    require_gpu()
+    """The table entries the device code touches, against the oracle's restatement of the
+    reference's index arithmetic (encoding_hashgrid.cuh:17-60,279-287): the index function on its
+    own (mode 0, corner by corner in the reference's order), and the entries that the code of the
+    fused kernels really uses -- the paired gathers of the forward pass (mode 1: dense pairs
+    along the last coordinate, hashed pairs idx / idx^1) and the lane-group gradient scatter of
+    the backward pass (mode 2) -- as sets per point and level, bit for bit, with their weights."""
     import json
     import qmlp
     cfg = _grid_cfg(spec) if "id" not in spec else spec
     enc = qmlp.Encoding(json.dumps(cfg))
+    f = cfg["n_features_per_level"]
+    modes = [0, 1] + ([2] if f & (f - 1) == 0 and f <= 32 else [])
+    if os.environ.get("QMLP_WARM_CACHE"):
+        for m in modes:
+            enc.hashgrid_corners(None, m)
+    require_gpu()
     g = qo.HashGrid(cfg)
     assert [(r, h, o) for (r, h, o, _) in enc.hashgrid_levels()] == [(r, h, o) for (r, h, o, _) in g.level_table()]
     rng = np.random.default_rng(17)
@@ -236,13 +264,24 @@ def test_grid_indices_are_bit_exact(spec):
     N = 20000
     X = (lo + sz * rng.uniform(-0.05, 1.05, (N, d))).astype(np.float32)   # includes points outside the box
     X[:64] = lo + sz * rng.integers(0, 2, (64, d))                        # and exact box corners
-    table = torch.zeros(enc.num_parameters(), device="cuda")
+    table = torch.zeros(enc.num_parameters(), device="cuda", dtype=enc.parameter_dtype())
     enc.set_parameter(table)
-    idx, w = enc.hashgrid_corners(torch.from_numpy(X).cuda())
+    x = torch.from_numpy(X).cuda()
+    idx, w = enc.hashgrid_corners(x)
     torch.cuda.synchronize()
     ref_idx, ref_w = g.corners(X)
     assert np.array_equal(idx.cpu().numpy().view(np.uint32), ref_idx)
     assert np.allclose(w.cpu().numpy(), ref_w, rtol=1e-5, atol=1e-6)
+    want_idx, want_w = _per_point_sets(ref_idx, ref_w)
+    assert int(want_idx.max()) + f <= enc.num_parameters()
+    for mode in modes[1:]:
+        idx, w = enc.hashgrid_corners(x, mode)
+        torch.cuda.synchronize()
+        got_idx = idx.cpu().numpy().view(np.uint32)
+        assert np.isfinite(w.cpu().numpy()).all(), "mode %d left slots unwritten" % mode
+        got_idx, got_w = _per_point_sets(got_idx, w.cpu().numpy())
+        assert np.array_equal(got_idx, want_idx), "mode %d" % mode
+        assert np.allclose(got_w, want_w, rtol=1e-5, atol=1e-6), "mode %d" % mode
 
 
 @pytest.mark.parametrize("spec", GRID_SPECS)
@@ -366,6 +405,73 @@ def test_network_with_two_grids_against_oracle():
     got = case.gpu_train(X, adj, flags)
     assert_close(got["out"], case.oracle.forward(X), "forward")
     check_gradients(case, X, adj, flags, got)
+
+
+SLICE_GRIDS = [
+    # 3-D, 6 levels, dense and hashed (several slices per level only in the large variants below)
+    (dict(n_in=3, n_levels=6, n_features_per_level=2, log2_hashmap_size=10, min_resolution=4, max_resolution=128), "half"),
+    # hashed levels of 2^16 entries x 2 features = 4 slices each, dense levels of 1, 1 and 3 slices
+    (dict(n_in=3, n_levels=7, n_features_per_level=2, log2_hashmap_size=16, min_resolution=8, max_resolution=300), "float"),
+    # one dense 4-D level of 20^4 x 8 features: 40 slices, pairs along the last coordinate straddle slice borders
+    (dict(n_in=4, n_levels=1, n_features_per_level=8, log2_hashmap_size=-1, min_resolution=20, max_resolution=20), "half"),
+    # dense 2-D levels up to 400^2 cells, 3 features (slices of 10 922 entries), levels summed ("add")
+    (dict(n_in=2, n_levels=4, n_features_per_level=3, log2_hashmap_size=-1, min_resolution=5, max_resolution=400,
+          combination_mode="add"), "float"),
+    (dict(n_in=1, n_levels=3, n_features_per_level=1, log2_hashmap_size=4, min_resolution=2, max_resolution=64), "float"),
+    (dict(n_in=6, n_levels=2, n_features_per_level=1, log2_hashmap_size=12, min_resolution=2, max_resolution=5), "half"),
+]
+
+
+@pytest.mark.parametrize("spec,precision", SLICE_GRIDS)
+def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle(spec, precision):
+    """options.slice_gradients = 1: the backward kernel stores the adjoint of the encoded rows and one
+    workgroup per slice of the gradient table sums the contributions of the whole batch in LDS
+    (kernels/grid_gradient.h); 0: the backward kernel scatters with float atomics. Same entries,
+    same weights, another order of the fp32 additions; both against the fp32 oracle. The grid
+    sits behind an identity encoding (channel offset 2) and reads its coordinates from input
+    channel 1 on; the second call adds onto the gradients of the first."""
+    d = spec["n_in"]
+    grid = _grid_cfg(spec, precision, start=1)
+    n_in = d + 1
+    base = {"num_inputs": n_in, "num_outputs": 2, "activation_specification": ["qmlp/builtin-activations.json"],
+            "encodings": [{"id": "Identity", "start_in": 0, "n_in": 2}, grid],
+            "network": [{"n_out": 32, "bias": True, "activation": "celu"},
+                        {"n_out": 2, "bias": False, "activation": "identity"}]}
+    cases = {}
+    for mode in (0, 1):
+        cfg = json.loads(json.dumps(base))
+        cfg["options"] = {"slice_gradients": mode}
+        cases[mode] = Case(cfg)
+    rng = np.random.default_rng(12)
+    params = random_parameters(cases[0].oracle, rng)
+    table = rng.uniform(-1, 1, cases[0].oracle.encodings[1][1].n_params)
+    for c in cases.values():
+        c.set_parameters(params)
+        c.set_table(1, table)
+    lo = np.array([0.0] + grid["bounding_box_min"], np.float32)
+    sz = np.array([1.0] + grid["bounding_box_size"], np.float32)
+    for N in (3000, 70001):     # one round of every slice workgroup; many rounds and a ragged last tile
+        X = (lo + sz * rng.uniform(-0.05, 1.05, (N, n_in))).astype(np.float32)
+        adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+        for flags in (FLAG_ENC, FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC):
+            got = {mode: c.gpu_train(X, adj, flags) for mode, c in cases.items()}
+            a, b = got[0]["table_grads"][1], got[1]["table_grads"][1]
+            scale = max(1.0, float(np.abs(a).max()))
+            assert np.allclose(a / scale, b / scale, rtol=1e-4, atol=2e-6), "N=%d flags=%d: %g" % (N, flags, np.abs(a - b).max())
+            if flags & FLAG_WEIGHTS:
+                assert np.array_equal(got[0]["grads"], got[1]["grads"])
+                assert np.array_equal(got[0]["adj_x"], got[1]["adj_x"])
+            # (weight and input gradients are those of the other mode bit for bit: checked against the oracle elsewhere)
+            check_gradients(cases[1], X, adj, FLAG_ENC, got[1], what="slices, N=%d flags=%d: " % (N, flags))
+    # gradients are accumulated: a second call onto the same tensor doubles them
+    x, a = torch.from_numpy(X).cuda(), torch.from_numpy(adj).cuda()
+    c = cases[1]
+    out, tmp = c.net.forward_raw(x, c.params, c.encoding_parameters(), FLAG_ENC)
+    _, _, genc = c.net.adjoint_raw(x, a, FLAG_ENC, tmp, c.params, c.encoding_parameters())
+    once = genc[1].clone()
+    c.net.adjoint_raw(x, a, FLAG_ENC, tmp, c.params, c.encoding_parameters(), grad_encodings=genc)
+    torch.cuda.synchronize()
+    assert torch.allclose(genc[1], 2 * once, rtol=1e-4, atol=1e-6)
 
 
 @pytest.mark.parametrize("features,levels", [(16, 2), (32, 1), (1, 6)])

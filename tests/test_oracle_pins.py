@@ -516,6 +516,54 @@ def test_round_mode_one_stays_close_to_fp32():
     assert not np.array_equal(a, b)
 
 
+def test_round_mode_one_rounds_at_every_point_of_the_half_precision_pipeline():
+    """Known answer for the oracle mode that rounds to fp16 where the device does. One point
+    through identity(1) -> 16 sine -> 1 identity with two live hidden units; the numbers are
+    worked out by hand (exact binary fractions, sine / cosine from tables to 16 digits), every value
+    in front of a rounding sits at least 1/8 fp16 ulp away from a tie, and every rounding changes
+    its value, so a rounding that is missing or sits elsewhere changes one of the results below.
+
+      x = 1.0006103515625          -> encoded row   x^ = 1.0009765625      (1 + 0.625 ulp -> 1 + 1 ulp)
+      pre0 = 0.8125  * x^ = 0.81329345703125 -> 0.8134765625 ; pre1 = 0.5625 * x^ = 0.56304931640625 -> 0.56298828125
+      h0 = sin(pre0) = 0.72667986... -> 0.7265625            ; h1 = sin(pre1) = 0.53371566... -> 0.53369140625
+      y  = 0.6875 h0 - 1.4375 h1 = -0.267669677734375 -> -0.267578125
+      g = dL/dy = 0.30010986328125 -> g^ = 0.300048828125
+      dW1 = g^ * (h0, h1) = (0.21800422668457031, 0.16013348102569580)   (fp32 products of fp16 values: exact)
+      dh = (0.6875 g^, -1.4375 g^) = (0.2062835693359375, -0.4313201904296875) -> (0.206298828125, -0.431396484375)
+      dpre0 = cos(pre) * dh = (0.14172239..., -0.36481648...) -> (0.1417236328125, -0.36474609375)
+      dW0 = dpre0 * x^ = (0.14186203479766846, -0.36510229110717773)
+      dx = 0.8125 dpre0[0] + 0.5625 dpre0[1] = -0.09001922607421875 -> -0.09002685546875
+    """
+    net = qo.Network(mlp_cfg(1, [2, 1], ["sine", "identity"], [False, False]))
+    params = np.zeros(net.num_parameters, np.float32)
+    w0, w1 = net.weight(0, params), net.weight(1, params)
+    w0[0, 0], w0[1, 0] = 0.8125, 0.5625
+    w1[0, 0], w1[0, 1] = 0.6875, -1.4375
+    net.set_parameters(params)
+    X = np.array([[1.0006103515625]], np.float32)
+    g = np.array([[0.30010986328125]], np.float32)
+    out, enc, pre = net.forward(X, round_mode=1, store=True)
+    assert enc[0, 0] == np.float32(1.0009765625)
+    assert pre[0][0, 0] == np.float32(0.8134765625) and pre[0][0, 1] == np.float32(0.56298828125)
+    assert pre[1][0, 0] == np.float32(-0.267578125) and out[0, 0] == np.float32(-0.267578125)
+    res = net.backward(X, g, qo.GRAD_INPUT | qo.GRAD_WEIGHTS, round_mode=1, return_dpre=True)
+    assert res["dpre"][1][0, 0] == np.float32(0.300048828125)
+    assert res["dpre"][0][0, 0] == np.float32(0.1417236328125) and res["dpre"][0][0, 1] == np.float32(-0.36474609375)
+    dw0, dw1 = net.weight(0, res["grads"]), net.weight(1, res["grads"])
+    assert dw1[0, 0] == np.float32(0.21800422668457031) and dw1[0, 1] == np.float32(0.16013348102569580)
+    assert dw0[0, 0] == np.float32(0.14186203479766846) and dw0[1, 0] == np.float32(-0.36510229110717773)
+    assert res["adj_x"][0, 0] == np.float32(-0.09002685546875)
+    # everything else of the padded matrices stays zero
+    assert np.count_nonzero(res["grads"]) == 4
+    # the fp32 mode rounds nowhere: the same chain without the arrows
+    out0 = net.forward(X, round_mode=0)
+    assert abs(float(out0[0, 0]) - (-0.26767468)) < 1e-7 and out0[0, 0] != out[0, 0]
+    res0 = net.backward(X, g, qo.GRAD_INPUT | qo.GRAD_WEIGHTS, round_mode=0)
+    assert abs(float(res0["adj_x"][0, 0]) - (-0.09001060)) < 1e-7
+    assert np.allclose(net.weight(1, res0["grads"])[0, :2], [0.21798468, 0.16013654], rtol=0, atol=1e-7)
+    assert np.allclose(net.weight(0, res0["grads"])[:2, 0], [0.14189935, -0.36508220], rtol=0, atol=1e-7)
+
+
 # ------------------------------------------------------------------ line integration
 def line_spec(child, stepsize=0.25, blending="additive", start=0):
     return {"id": "LineIntegration", "start_in": start, "n_in": 3, "volume": child, "stepsize": stepsize,
