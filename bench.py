@@ -64,7 +64,7 @@ def build_case(cfg_id, n_points, device):
     import numpy as np
     import torch
     import qmlp
-    from qmlp import baseline_configs as bc
+    import baseline_configs as bc
     c = bc.CONFIGS[cfg_id]
     rng = np.random.default_rng(bc.PARAMETER_SEED[cfg_id])
     net = qmlp.Network(json.dumps(c["cfg"]))
@@ -122,7 +122,7 @@ def run_inference(case, steps, warmup):
 
 def run_train(case, steps, warmup):
     import torch
-    from qmlp import baseline_configs as bc
+    import baseline_configs as bc
     net, x, params, enc = case["net"], case["x"], case["params"], case["enc_params"]
     cfg_id = case["cfg_id"]
     n = x.shape[0]
@@ -155,7 +155,7 @@ def cpu_baseline(case, train, min_seconds=10.0):
     points) on the same workload, repeated until at least min_seconds of CPU work."""
     import numpy as np
     import qmlp_oracle as qo
-    from qmlp import baseline_configs as bc
+    import baseline_configs as bc
     cfg_id = case["cfg_id"]
     oracle = qo.Network(case["cfg"]["cfg"], bc.ORACLE_ACTIVATIONS)
     oracle.set_parameters(case["params_np"].astype(np.float32))
@@ -184,7 +184,7 @@ def cpu_baseline(case, train, min_seconds=10.0):
 
 # ------------------------------------------------------------------ layer GEMMs alone
 def mlp_cfg(n_in, widths, activation="relu", last="identity"):
-    from qmlp import baseline_configs as bc
+    import baseline_configs as bc
     acts = [activation] * (len(widths) - 1) + [last]
     return {"num_inputs": n_in, "num_outputs": widths[-1], "activation_specification": [bc.BUILTIN],
             "encodings": [{"id": "Identity", "start_in": 0, "n_in": n_in}],
@@ -395,7 +395,7 @@ def main():
 
     import torch
     import qmlp
-    from qmlp import baseline_configs as bc
+    import baseline_configs as bc
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     qmlp.set_log_level("error")

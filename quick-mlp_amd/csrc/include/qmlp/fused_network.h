@@ -331,7 +331,7 @@ private:
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */
     /** Function attributes of the generated forward / backward kernels. */
-    std::string kernelAttributes() const;
+    std::string kernelAttributes(int blockSize) const;
     /** First input channel of the identity encoding if that is the network's only encoding and
      *  options.direct_input is on; -1 otherwise. */
     int directInputStart() const;

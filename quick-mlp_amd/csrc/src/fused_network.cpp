@@ -502,8 +502,10 @@ int FusedNetwork::ldsParamHalves(bool adjoint) const
     return ldsLayout(adjoint, w, b);
 }
 
-std::string FusedNetwork::kernelAttributes() const
+std::string FusedNetwork::kernelAttributes(int blockSize) const
 {
+    // a workgroup of 8 wavefronts has that budget anyway
+    if (blockSize >= 2 * DEFAULT_BLOCK_SIZE) return "";
     // Two wavefronts per SIMD at least: the register budget is then 256, all of them vector
     // registers, and the compiler keeps the matrix-core accumulators there (with up to 512 it
     // puts them into accumulation registers and copies every value out one by one). Layers
@@ -610,7 +612,7 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool r
     replaceAll(code, "$$POINTS_PER_LANE$$", std::to_string(pointsPerLane));
     replaceAll(code, "$$REGISTER_STAGING$$", registerStaging ? "true" : "false");
     replaceAll(code, "$$DIRECT_INPUT_START$$", std::to_string(directInputStart()));
-    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes());
+    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes(blockSize));
     // rows in registers are indexed by the tile: that loop has to be unrolled
     replaceAll(code, "$$TILE_LOOP_PRAGMA$$", registerStaging ? "#pragma unroll" : "#pragma unroll 1");
     std::vector<int> ldsW, ldsB;
@@ -757,7 +759,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     std::string code = kl->findFile("qmlp/kernels/network_backward.h").value();
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
-    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes());
+    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes(blockSize));
     replaceAll(code, "$$HAS_INPUT_GRADIENTS$$", hasInputGradients ? "true" : "false");
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
     replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
@@ -1158,7 +1160,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
     for (const auto& l : layers_) adjointChannels += l.channelsOut;
     ak.perEntryAdjointMemoryBytes = hasNetworkGradients ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
     // behind the adjoint pre-activations: the adjoint of the encoded rows for the records kernels
-    if (flags & GRADIENTS_INPUT_ENCODINGS) ak.perEntryAdjointMemoryBytes += sliceGradientBytesPerPoint();
+    if (sliceGradients && (flags & GRADIENTS_INPUT_ENCODINGS)) ak.perEntryAdjointMemoryBytes += sliceGradientBytesPerPoint();
 
     if (sliceGradients && (flags & GRADIENTS_INPUT_ENCODINGS)) {
         int channelOffset = 0;
@@ -1496,8 +1498,9 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
     int adjointChannels = 0;
     for (const auto& l : layers_) adjointChannels += l.channelsOut;
     int perEntry = (adjointFlags & GRADIENTS_NETWORK_WEIGHTS) ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
-    // the adjoint of the encoded rows, which the records kernels of the grids read
-    if (adjointFlags & GRADIENTS_INPUT_ENCODINGS) perEntry += sliceGradientBytesPerPoint();
+    // batches that take the gradient slice kernels: the adjoint of the encoded rows, which the records kernels read
+    const bool sliceGradients = useSliceGradients(numElements, adjointFlags);
+    if (sliceGradients) perEntry += sliceGradientBytesPerPoint();
     numElements = roundUp(numElements, WARP_SIZE);
     size_t bytes = static_cast<size_t>(perEntry) * static_cast<size_t>(numElements);
     // behind the adjoint pre-activations: the partial weight gradients of the batch slices
@@ -1507,7 +1510,7 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
     std::vector<long long> transposed;
     bytes += roundUp(transposedWeightLayout(adjointFlags, transposed) * sizeof(half), size_t(16));
     // last: bucket cursors and records of the gradient slice kernels
-    if (adjointFlags & GRADIENTS_INPUT_ENCODINGS) bytes = roundUp(bytes, size_t(256)) + sliceGradientWorkspaceBytes(numElements);
+    if (sliceGradients) bytes = roundUp(bytes, size_t(256)) + sliceGradientWorkspaceBytes(numElements);
     return bytes;
 }
 

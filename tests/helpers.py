@@ -9,7 +9,7 @@ import torch
 
 import qmlp
 import qmlp_oracle as qo
-from qmlp import baseline_configs as bc
+import baseline_configs as bc
 
 REL, ABS = 1e-2, 1e-3          # tolerance of the fp16 path against the fp32 oracle
 FLAG_INPUT, FLAG_WEIGHTS, FLAG_ENC = 1, 2, 4

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import qmlp
-from qmlp import baseline_configs as bc
+import baseline_configs as bc
 
 pytestmark = pytest.mark.gpu
 
