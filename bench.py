@@ -360,6 +360,90 @@ def gather_ceiling(device, repeats=5):
     return result
 
 
+LDS_SOURCE = r"""
+#include <hip/hip_runtime.h>
+// Reference patterns for reading the LDS bank-conflict counter: every kernel issues the same number
+// of LDS read instructions per wavefront; only the addresses differ.
+//   0: 16 bytes per lane at consecutive addresses (how the layer weights are read as matrix-core operands)
+//   1:  4 bytes per lane at consecutive addresses (no conflicts by construction)
+//   2:  4 bytes per lane, 128 bytes apart (every lane on the same bank)
+//   3:  8 bytes per lane, rows of 64 bytes rotated as the staging rows of 32 channels are (arrays.h)
+//   4:  8 bytes per lane at consecutive addresses
+template <int KIND>
+__device__ void body(float* out, int iters)
+{
+    __shared__ __attribute__((aligned(16))) float s[16384];
+    for (int i = threadIdx.x; i < 16384; i += blockDim.x) s[i] = 1.f;
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float acc = 0.f;
+    for (int it = 0; it < iters; ++it) {
+        int base = ((it * 4 + wave) & 7) * 2048;
+        asm volatile("" : "+v"(base));                     // keeps the read inside the loop
+        if (KIND == 0) { const float4 v = reinterpret_cast<const float4*>(s)[(base >> 2) + lane]; acc += v.x + v.y + v.z + v.w; }
+        if (KIND == 4) { const float2 v = reinterpret_cast<const float2*>(s)[(base >> 1) + lane]; acc += v.x + v.y; }
+        if (KIND == 1) acc += s[base + lane];
+        if (KIND == 2) acc += s[(base + lane * 32) & 16383];
+        if (KIND == 3) {
+            const int r = lane & 15, g = lane >> 4;          // 16 rows x 4 chunks of 8 bytes, as one operand read
+            const int row = r, chunk = (g + 2 * (row / 4) + (row >> 4)) & 7;
+            const float2 v = *reinterpret_cast<const float2*>(s + base + row * 16 + chunk * 2);
+            acc += v.x + v.y;
+        }
+    }
+    if (acc == 12345.f) out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+extern "C" __global__ void __launch_bounds__(256) LdsRead16Consecutive(float* out, int iters) { body<0>(out, iters); }
+extern "C" __global__ void __launch_bounds__(256) LdsRead4Consecutive(float* out, int iters) { body<1>(out, iters); }
+extern "C" __global__ void __launch_bounds__(256) LdsRead4SameBank(float* out, int iters) { body<2>(out, iters); }
+extern "C" __global__ void __launch_bounds__(256) LdsRead8RotatedRows(float* out, int iters) { body<3>(out, iters); }
+extern "C" __global__ void __launch_bounds__(256) LdsRead8Consecutive(float* out, int iters) { body<4>(out, iters); }
+"""
+
+
+def lds_calibration(device, repeats=3):
+    """Launches the reference LDS read patterns (for a profiler run that collects
+    SQ_LDS_BANK_CONFLICT and SQ_ACTIVE_INST_LDS next to the kernels of the library)."""
+    import ctypes
+    import torch
+    import qmlp
+    lib = qmlp._lib.lib
+    lib.qmlp_hip_last_error.restype = ctypes.c_char_p
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(lib.qmlp_hip_last_error().decode())
+
+    kernels = [b"LdsRead16Consecutive", b"LdsRead4Consecutive", b"LdsRead4SameBank", b"LdsRead8RotatedRows",
+               b"LdsRead8Consecutive"]
+    module = ctypes.c_void_p()
+    names = (ctypes.c_char_p * len(kernels))(*kernels)
+    opts = (ctypes.c_char_p * 6)(b"-O3", b"-I/opt/rocm/include", b"-Xclang", b"-target-feature", b"-Xclang", b"-packed-fp32-ops")
+    ok(lib.qmlp_hip_module_compile(LDS_SOURCE.encode(), b"lds_calibration.hip", None, None, 0, names, len(kernels), opts, 6,
+                                   None, ctypes.byref(module), None))
+    ok(lib.qmlp_hip_module_load(module))
+    out = torch.zeros(1024 * 256, dtype=torch.float32, device=device)
+    stream = qmlp._lib.current_stream(device)
+    result = {}
+    for name in kernels:
+        fn, lowered = ctypes.c_void_p(), ctypes.c_char_p()
+        ok(lib.qmlp_hip_module_lowered_name(module, name, ctypes.byref(lowered)))
+        ok(lib.qmlp_hip_module_get_function(module, lowered, ctypes.byref(fn)))
+        a_out, a_iters = ctypes.c_void_p(out.data_ptr()), ctypes.c_int(4096)
+        args = (ctypes.c_void_p * 2)(ctypes.addressof(a_out), ctypes.addressof(a_iters))
+        ok(lib.qmlp_hip_launch(fn, 1024, 256, 0, stream, args))
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(repeats):
+            ok(lib.qmlp_hip_launch(fn, 1024, 256, 0, stream, args))
+        stop.record()
+        torch.cuda.synchronize()
+        result[name.decode()] = {"launch_ms": start.elapsed_time(stop) / repeats, "lds_reads_per_wave": 4096}
+    ok(lib.qmlp_hip_module_destroy(module))
+    return result
+
+
 def request_ceiling(gather, points, requests_per_point, l2_miss_fraction, launch_ms):
     """Prices the line requests of a gathering launch with the two measured rates."""
     hit = points * requests_per_point * (1.0 - l2_miss_fraction) / gather["l2_hit"]["requests_per_s"]
@@ -377,7 +461,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2-inference",
-                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "all"],
+                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "lds-calibration", "all"],
                     help="layer-gemm: the layers of the hash-grid network on their own; reference-grid: the reference's "
                          "own benchmark networks; gather-ceiling: request rate of random gathers; all: every workload")
     ap.add_argument("--points", type=int, default=0, help="override the number of points")
@@ -433,6 +517,12 @@ def main():
         print(json.dumps(dict(head, value=g["l2_hit"]["requests_per_s"], unit="line requests/s",
                               ms_per_step=g["l2_hit"]["launch_ms"],
                               config={"workload": "gather-ceiling", "loads": 2048 * 256 * 64}, gather=g)))
+        return
+    if args.workload == "lds-calibration":
+        r = lds_calibration(device)
+        print(json.dumps(dict(head, value=1.0 / (r["LdsRead16Consecutive"]["launch_ms"] * 1e-3), unit="launches/s",
+                              ms_per_step=r["LdsRead16Consecutive"]["launch_ms"],
+                              config={"workload": "lds-calibration"}, lds=r)))
         return
     if args.workload == "all":
         g = gather_ceiling(device)

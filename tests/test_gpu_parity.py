@@ -643,10 +643,14 @@ def test_full_size_properties_cfg2():
     s = np.abs(ref).max()
     assert_close(full.cpu().numpy()[sample] / s, ref / s, "sampled oracle check", rel=5e-3, abs_=1e-3,
                  allowed_fraction=1e-3)
-    # and against the fp32 evaluation itself, at the tolerance of the fp16 path (relative to the output scale:
-    # the benchmark's tables of U(+-1e-4) make every output smaller than the absolute part)
-    ref0 = case.oracle.forward(X[sample], round_mode=0)
-    assert_close(full.cpu().numpy()[sample] / s, ref0 / s, "sampled fp32 oracle check", rel=REL, abs_=ABS, allowed_fraction=2e-3)
+    # and against the fp32 evaluation itself, at the tolerance of the fp16 path. With the benchmark's tables
+    # of U(+-1e-4) the encoded features are subnormal in fp16 (spacing 6e-8, several per cent of a value),
+    # so this comparison runs on the same network with tables of U(+-1): same kernels, same indices.
+    big, rng1 = baseline_case(2, table_scale=1.0)
+    out1 = big.net.inference(x, big.params, big.encoding_parameters()).cpu().numpy()[sample]
+    ref0 = big.oracle.forward(X[sample], round_mode=0)
+    s1 = np.abs(ref0).max()
+    assert_close(out1 / s1, ref0 / s1, "sampled fp32 oracle check", rel=REL, abs_=ABS, allowed_fraction=2e-3)
 
 
 def test_full_size_properties_cfg3_train():
