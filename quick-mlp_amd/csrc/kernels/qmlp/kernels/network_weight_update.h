@@ -45,9 +45,7 @@ $$DEFINE_ACTIVATIONS$$
  *         the input and re-applies its activation; the host picks the cheaper split.
  */
 template <int CIN, int COUT, bool BIAS, typename InputActivation, int MO_CHUNK, int KI_CHUNK>
-// (two wavefronts per SIMD at least: with that register budget the compiler keeps the
-// accumulators in vector registers instead of copying them out of accumulation registers)
-__global__ void __launch_bounds__($$BLOCK_SIZE$$) __attribute__((amdgpu_waves_per_eu(2))) WeightUpdateKernel(
+__global__ void __launch_bounds__($$BLOCK_SIZE$$) WeightUpdateKernel(
     int numTiles,                     // 64-point tiles in the batch
     float* __restrict__ partialWeights,  // slice 0 of this layer's (COUT, CIN) row-major partial sums
     float* __restrict__ partialBias,     // slice 0 of this layer's (COUT) partial sums, or nullptr
