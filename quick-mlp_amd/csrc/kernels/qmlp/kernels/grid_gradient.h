@@ -64,8 +64,39 @@ struct GridGradientLayout
     static constexpr int F = Grid::F;
     static constexpr int L = Grid::L;
     static constexpr int PAIRS = Grid::NC / 2 > 0 ? Grid::NC / 2 : 1;
-    /** A record in 32-bit words: element of the lower and of the upper entry, their weights, F halves of adjoint. */
-    static constexpr int RECORD_WORDS = 4 + (F + 1) / 2;
+    /** A record in 32-bit words: the offsets of the lower and of the upper entry within the slice (16 bits
+     *  each), their two weights, F halves of adjoint; one word of padding where that makes it a multiple of
+     *  16 bytes (records of 16 or 32 bytes move as whole vector loads and stores). */
+    static constexpr int RECORD_WORDS_USED = 3 + (F + 1) / 2;
+    static constexpr int RECORD_WORDS = RECORD_WORDS_USED % 4 == 3 ? RECORD_WORDS_USED + 1 : RECORD_WORDS_USED;
+    static_assert(SLICE_FLOATS <= 65536, "offsets within a slice are stored in 16 bits");
+
+    /** Records start at multiples of their size from a 16-byte aligned base (LDS or global memory). */
+    template <typename Pointer>
+    __device__ __forceinline__ static void loadRecord(Pointer src, unsigned (&r)[RECORD_WORDS])
+    {
+        if constexpr (RECORD_WORDS % 4 == 0) {
+#pragma unroll
+            for (int v = 0; v < RECORD_WORDS / 4; ++v) {
+                const uint4 q = reinterpret_cast<const uint4*>(src)[v];
+                r[4 * v] = q.x, r[4 * v + 1] = q.y, r[4 * v + 2] = q.z, r[4 * v + 3] = q.w;
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < RECORD_WORDS; ++v) r[v] = src[v];
+        }
+    }
+    __device__ __forceinline__ static void storeRecord(unsigned* dst, const unsigned (&r)[RECORD_WORDS])
+    {
+        if constexpr (RECORD_WORDS % 4 == 0) {
+#pragma unroll
+            for (int v = 0; v < RECORD_WORDS / 4; ++v)
+                reinterpret_cast<uint4*>(dst)[v] = make_uint4(r[4 * v], r[4 * v + 1], r[4 * v + 2], r[4 * v + 3]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < RECORD_WORDS; ++v) dst[v] = r[v];
+        }
+    }
 
     __device__ __host__ static constexpr int levelFloats(int l)
     {
@@ -134,16 +165,17 @@ struct GridGradientRecords
         }
     }
 
-    /** Adds a record to the gradient tensor itself (its bucket was full). */
+    /** Adds a record to the gradient tensor itself (its bucket was full); grad: element 0 of the record's slice. */
     __device__ __forceinline__ static void addToTensor(const unsigned (&rec)[RW], float* __restrict__ grad)
     {
-        const float wL = __builtin_bit_cast(float, rec[2]), wH = __builtin_bit_cast(float, rec[3]);
+        const float wL = __builtin_bit_cast(float, rec[1]), wH = __builtin_bit_cast(float, rec[2]);
+        const unsigned eL = rec[0] & 0xffffu, eH = rec[0] >> 16;
 #pragma unroll
         for (int i = 0; i < F; ++i) {
-            const unsigned short bits = static_cast<unsigned short>(rec[4 + i / 2] >> (16 * (i % 2)));
+            const unsigned short bits = static_cast<unsigned short>(rec[3 + i / 2] >> (16 * (i % 2)));
             const float adj = static_cast<float>(__builtin_bit_cast(f16, bits));
-            unsafeAtomicAdd(grad + rec[0] + i, wL * adj);
-            unsafeAtomicAdd(grad + rec[1] + i, wH * adj);
+            unsafeAtomicAdd(grad + eL + i, wL * adj);
+            if (wH != 0.f) unsafeAtomicAdd(grad + eH + i, wH * adj);
         }
     }
 
@@ -185,13 +217,30 @@ struct GridGradientRecords
                 unsigned idxL, idxH;
                 float w;
                 pairEntries<LEVEL>(s, c, idxL, idxH, w);
-                rec[c][0] = base + idxL * F;
-                rec[c][1] = base + idxH * F;
-                rec[c][2] = __builtin_bit_cast(unsigned, w * (1.f - s.f[PD]));
-                rec[c][3] = __builtin_bit_cast(unsigned, w * s.f[PD]);
-#pragma unroll
-                for (int i = 0; i < (F + 1) / 2; ++i) rec[c][4 + i] = adjWords[i];
                 bucket[c] = static_cast<int>(idxL * F / SLICE_FLOATS);   // the slice of the lower entry files the record
+                const unsigned sliceStart = static_cast<unsigned>(bucket[c]) * SLICE_FLOATS;
+                const unsigned eL = idxL * F - sliceStart;
+                unsigned eH = idxH * F - sliceStart;                     // wraps if the upper entry lies below the slice
+                float wH = w * s.f[PD];
+                if (eH >= static_cast<unsigned>(SLICE_FLOATS)) {
+                    // the upper entry lies in another slice (an entry next to a slice boundary; in a hashed
+                    // level one pair in thousands): added right here, the record keeps the lower entry only
+#pragma unroll
+                    for (int i = 0; i < F; ++i) {
+                        const unsigned short bits = static_cast<unsigned short>(adjWords[i / 2] >> (16 * (i % 2)));
+                        unsafeAtomicAdd(params.parametersBackward + base + idxH * F + i,
+                                        wH * static_cast<float>(__builtin_bit_cast(f16, bits)));
+                    }
+                    eH = eL;
+                    wH = 0.f;
+                }
+                rec[c][0] = eL | (eH << 16);
+                rec[c][1] = __builtin_bit_cast(unsigned, w * (1.f - s.f[PD]));
+                rec[c][2] = __builtin_bit_cast(unsigned, wH);
+#pragma unroll
+                for (int i = 0; i < (F + 1) / 2; ++i) rec[c][3 + i] = adjWords[i];
+#pragma unroll
+                for (int v = Layout::RECORD_WORDS_USED; v < RW; ++v) rec[c][v] = 0u;
                 // (a level of one slice needs no sorting: every lane has fixed places)
                 rank[c] = NS == 1 ? tid * PAIRS + c : atomicAdd(sHist + bucket[c], 1);
             }
@@ -199,9 +248,8 @@ struct GridGradientRecords
             // lanes beyond the batch: in a level of one slice they fill their fixed places with records that add nothing
 #pragma unroll
             for (int c = 0; c < PAIRS; ++c) {
-                rec[c][0] = rec[c][1] = base;
 #pragma unroll
-                for (int v = 2; v < RW; ++v) rec[c][v] = 0u;
+                for (int v = 0; v < RW; ++v) rec[c][v] = 0u;
                 bucket[c] = 0;
                 rank[c] = tid * PAIRS + c;
             }
@@ -235,8 +283,7 @@ struct GridGradientRecords
 #pragma unroll
             for (int c = 0; c < PAIRS; ++c) {
                 const int at = sLocalBase[bucket[c]] + rank[c];
-#pragma unroll
-                for (int v = 0; v < RW; ++v) sStage[at * RW + v] = rec[c][v];
+                Layout::storeRecord(sStage + at * RW, rec[c]);
                 sBucketOf[at] = static_cast<unsigned short>(bucket[c]);
             }
         }
@@ -250,14 +297,11 @@ struct GridGradientRecords
             const int b = sBucketOf[j];
             const long long at = sGlobalBase[b] + (j - sLocalBase[b]);
             unsigned r[RW];
-#pragma unroll
-            for (int v = 0; v < RW; ++v) r[v] = sStage[j * RW + v];
+            Layout::loadRecord(sStage + j * RW, r);
             if (at < capacity) {
-                unsigned* dst = levelRecords + (static_cast<long long>(b) * capacity + at) * RW;
-#pragma unroll
-                for (int v = 0; v < RW; ++v) dst[v] = r[v];
+                Layout::storeRecord(levelRecords + (static_cast<long long>(b) * capacity + at) * RW, r);
             } else {
-                addToTensor(r, params.parametersBackward);
+                addToTensor(r, params.parametersBackward + base + static_cast<unsigned>(b) * SLICE_FLOATS);
             }
         }
     }
@@ -364,37 +408,41 @@ struct GridGradientSlices
         const long long filled = min(static_cast<long long>(cursors[Layout::firstBucket(LEVEL) + item.slice]), capacity);
         const long long begin = filled * item.part / item.parts, end = filled * (item.part + 1) / item.parts;
         const unsigned* bucket = records + (Layout::levelOffset(LEVEL, numel) + static_cast<long long>(item.slice) * capacity) * RW;
-        const unsigned first = item.first, count = static_cast<unsigned>(item.floats);
         constexpr int UNROLL = 4;
         for (long long j0 = begin + tid; j0 < end; j0 += UNROLL * BLOCK) {
             unsigned rec[UNROLL][RW];
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const long long j = j0 + u * BLOCK;
+                if (j < end) {
+                    Layout::loadRecord(bucket + j * RW, rec[u]);
+                } else {
 #pragma unroll
-                for (int v = 0; v < RW; ++v) rec[u][v] = j < end ? bucket[j * RW + v] : 0u;
+                    for (int v = 0; v < RW; ++v) rec[u][v] = 0u;
+                }
             }
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (j0 + u * BLOCK >= end) continue;
-                const unsigned eL = rec[u][0] - first, eH = rec[u][1] - first;   // unsigned: one compare tells whether it is inside
-                const float wL = __builtin_bit_cast(float, rec[u][2]), wH = __builtin_bit_cast(float, rec[u][3]);
+                const unsigned eL = rec[u][0] & 0xffffu, eH = rec[u][0] >> 16;   // both inside this slice
+                const float wL = __builtin_bit_cast(float, rec[u][1]), wH = __builtin_bit_cast(float, rec[u][2]);
 #pragma unroll
-                for (int i = 0; i < F; ++i) {
-                    const unsigned short bits = static_cast<unsigned short>(rec[u][4 + i / 2] >> (16 * (i % 2)));
+                for (int step = 0; step < F; ++step) {
+                    // Neighbouring lanes take the features in rotated order: an entry starts at a multiple of
+                    // 8 * F bytes, so lanes that all add feature `step` meet on a few LDS banks (measured on a
+                    // dense grid with 8 features: conflicts 90 % of the LDS cycles of this kernel).
+                    const int i = (F & (F - 1)) == 0 ? ((step + tid) & (F - 1)) : ((step + tid % F) % F);
+                    unsigned word = rec[u][3];
+#pragma unroll
+                    for (int w = 1; w < (F + 1) / 2; ++w) word = (i >> 1) == w ? rec[u][3 + w] : word;
+                    const unsigned short bits = static_cast<unsigned short>(word >> (16 * (i & 1)));
                     const float adj = static_cast<float>(__builtin_bit_cast(f16, bits));
-                    // the lower entry files the record, so it lies in this slice; the upper one may lie in the next
-                    if (eL < count) {
-                        if constexpr (FIXED) ldsAddFixed(sFixed + eL + i, toFixed(wL * adj, scaleExponent));
-                        else Grid::ldsAdd(sFloat + eL + i, wL * adj);
+                    if constexpr (FIXED) {
+                        ldsAddFixed(sFixed + eL + i, toFixed(wL * adj, scaleExponent));
+                        ldsAddFixed(sFixed + eH + i, toFixed(wH * adj, scaleExponent));
                     } else {
-                        unsafeAtomicAdd(gradients + rec[u][0] + i, wL * adj);
-                    }
-                    if (eH < count) {
-                        if constexpr (FIXED) ldsAddFixed(sFixed + eH + i, toFixed(wH * adj, scaleExponent));
-                        else Grid::ldsAdd(sFloat + eH + i, wH * adj);
-                    } else {
-                        unsafeAtomicAdd(gradients + rec[u][1] + i, wH * adj);
+                        Grid::ldsAdd(sFloat + eL + i, wL * adj);
+                        Grid::ldsAdd(sFloat + eH + i, wH * adj);
                     }
                 }
             }
@@ -420,9 +468,9 @@ struct GridGradientSlices
         if (finite) sumRecords<LEVEL, true>(numel, records, cursors, gradients, item, sSlice, sFloat, scaleExponent);
         else sumRecords<LEVEL, false>(numel, records, cursors, gradients, item, sSlice, sFloat, 0);
         __syncthreads();
-        // Added to the gradient tensor with atomics, 16 neighbouring floats per request: other work items
-        // may hold sums for the same slice (parts > 1), and a record whose upper entry lies in the next
-        // slice is added there with an atomic while that slice's owner is at work.
+        // Added to the gradient tensor: with atomics (16 neighbouring floats per request) where other work
+        // items hold sums for the same slice (parts > 1), else this workgroup is the only writer of its
+        // slice in this launch (contributions to entries of other slices were added by the records kernel).
         float* __restrict__ grad = gradients + item.first;
         for (int i = tid; i < item.floats; i += BLOCK) {
             float v;
@@ -432,7 +480,10 @@ struct GridGradientSlices
             } else {
                 v = sFloat[i];
             }
-            if (v != 0.f) unsafeAtomicAdd(grad + i, v);
+            if (v != 0.f) {
+                if (item.parts > 1) unsafeAtomicAdd(grad + i, v);
+                else grad[i] += v;
+            }
         }
     }
 

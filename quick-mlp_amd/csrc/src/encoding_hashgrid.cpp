@@ -289,7 +289,9 @@ bool EncodingHashGrid::gradientSlices(GradientSliceLayout& layout) const
     layout.sliceFloats = entries * numFeaturesPerLevel_;
     layout.configType = "qmlp::kernel::" + configName();
     layout.pairs = std::max(1, (1 << dimension_) / 2);
-    layout.recordWords = 4 + (numFeaturesPerLevel_ + 1) / 2;
+    // as GridGradientLayout::RECORD_WORDS: two 16-bit offsets, two weights, the adjoint halves, padded to 16 / 32 bytes
+    const int usedWords = 3 + (numFeaturesPerLevel_ + 1) / 2;
+    layout.recordWords = usedWords % 4 == 3 ? usedWords + 1 : usedWords;
     // the records of a workgroup and level are sorted in LDS: 96 KiB for them, the rest for the book-keeping
     int points = 1024;
     while (points > 64 && points * layout.pairs * layout.recordWords * 4 > 96 * 1024) points /= 2;

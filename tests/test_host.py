@@ -155,7 +155,7 @@ def test_temporary_memory_sizes():
             assert net.adjoint_memory(n, 5) == 0
     # From 2^14 points on the grid gradients are summed slice by slice: the adjoint of the encoded rows
     # (32 halves per point) joins the adjoint pre-activations, and behind everything else come the
-    # bucket cursors and the records (5 words each; per level, slices x (1.25 x share + 2048) of them:
+    # bucket cursors and the records (4 words each; per level, slices x (1.25 x share + 2048) of them:
     # the table of a level holds 8192 .. 1 048 576 floats, a slice 16 384).
     n = 1 << 18
     floats = [8192, 24334, 71874, 221184, 686000] + [1 << 20] * 11
@@ -163,8 +163,8 @@ def test_temporary_memory_sizes():
     records = sum(s * (((5 * n * 4 // 4) // s + 2048) & ~3) for s in slices_per_level)
     cursors = -(-(sum(slices_per_level) + 1) * 4 // 256) * 256
     base = (per_adj + 2 * 32) * n + 512 * n_params * 4
-    assert net.adjoint_memory(n, 7) == -(-base // 256) * 256 + cursors + -(-records * 20 // 256) * 256
-    assert net.adjoint_memory(n, 4) == 2 * 32 * n + cursors + -(-records * 20 // 256) * 256
+    assert net.adjoint_memory(n, 7) == -(-base // 256) * 256 + cursors + -(-records * 16 // 256) * 256
+    assert net.adjoint_memory(n, 4) == 2 * 32 * n + cursors + -(-records * 16 // 256) * 256
     with pytest.raises(qmlp.QmlpError, match="At least one derivative"):
         net.adjoint_memory(10, 0)
 
