@@ -67,6 +67,10 @@ public:
         // the first such call and keeps (grown when a larger batch comes); calls of one
         // network on several streams at once would share it.
         int sortPoints = -1;
+        //true: a training pass (forward with stored intermediates + adjoint) evaluates the batches that
+        //inference would sort in the same sorted order; the sorted rows and the order travel in the
+        //forward memory. false: training passes take the batch as given.
+        bool sortTraining = true;
 
         // Parameter gradients of grid encodings: summed slice by slice in LDS by a kernel of its own
         // (kernels/grid_gradient.h) instead of scattered with float atomics by the backward kernel.
@@ -130,8 +134,9 @@ private:
     struct PointOrder
     {
         std::optional<KernelFunction> count, scan, scatter;
-        Tensor workspace;           // sorted inputs (floats), order (ints), slab totals and per-chunk histograms (ints)
-        long long capacity = 0;     // points the workspace holds
+        std::optional<KernelFunction> gatherRows, scatterAddRows;   // rows of dL/dy into, rows of the input gradients out of the sorted order
+        Tensor workspace;           // slab totals and per-chunk histograms (ints), sorted inputs (floats), order (ints)
+        long long capacityWords = 0;   // 32-bit words the workspace holds
     };
     PointOrder pointOrder_;
     /** Smaller batches are never sorted when sortPoints < 0; larger ones if the encoding expects a gain. */
@@ -142,7 +147,20 @@ private:
      *   order holds, per row of it, the row of the caller's batch
      */
     bool sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
-                    bool noAlloc = false);
+                    bool noAlloc = false, void* destination = nullptr);
+    /** The slab key of the encoding that orders a batch of numel points, if such a batch is ordered at all
+     *  (a function of the specification and numel alone). */
+    bool pointOrderFor(int numel, kernel::PointOrderKey& key) const;
+    /** Does a training pass over numel points run in sorted order? Then the forward memory holds, behind the
+     *  intermediates and 256-byte aligned, the sorted input rows (numel x channelsIn floats) and the order (numel ints). */
+    bool sortsTraining(int numel) const;
+    /** adjointMemory() of a batch that is processed in the order given. */
+    size_t adjointMemoryAsGiven(int numElements, AdjointModeFlags adjointFlags) const;
+    /** Bytes at the end of the adjoint memory of a batch that trains in sorted order (with the gap that aligns them
+     *  behind bytesInFront): the rows of dL/dy and of the input gradients in that order. */
+    size_t sortedAdjointBytes(int numElements, AdjointModeFlags adjointFlags, size_t bytesInFront) const;
+    /** Byte offset of the sorted rows within the forward memory of a batch of numel points. */
+    size_t sortedRowsOffset(int numel) const;
 
     struct AdjointLayerInfo
     {

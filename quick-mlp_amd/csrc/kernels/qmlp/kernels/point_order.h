@@ -199,4 +199,34 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
     }
 }
 
+/**
+ * Rows of a caller's tensor in the sorted order: dst[i, c] = src[order[i], c] (dst dense). One
+ * lane per element, so a wavefront writes consecutive words and reads short runs.
+ */
+__global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderGatherRows(
+    long long elements, int channels, const Tensor2Read<float> src, const int* __restrict__ order, float* __restrict__ dst)
+{
+    for (long long e = static_cast<long long>(blockIdx.x) * POINT_ORDER_BLOCK + threadIdx.x; e < elements;
+         e += static_cast<long long>(gridDim.x) * POINT_ORDER_BLOCK) {
+        const long long row = e / channels;
+        const int c = static_cast<int>(e - row * channels);
+        dst[e] = src.data_[static_cast<long long>(order[row]) * src.strides_[0] + static_cast<long long>(c) * src.strides_[1]];
+    }
+}
+
+/**
+ * Rows that were computed in the sorted order, added to the caller's tensor:
+ * dst[order[i], c] += src[i, c] (src dense; every row of dst is written by one row of src).
+ */
+__global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatterAddRows(
+    long long elements, int channels, const float* __restrict__ src, const int* __restrict__ order, Tensor2RW<float> dst)
+{
+    for (long long e = static_cast<long long>(blockIdx.x) * POINT_ORDER_BLOCK + threadIdx.x; e < elements;
+         e += static_cast<long long>(gridDim.x) * POINT_ORDER_BLOCK) {
+        const long long row = e / channels;
+        const int c = static_cast<int>(e - row * channels);
+        dst.data_[static_cast<long long>(order[row]) * dst.strides_[0] + static_cast<long long>(c) * dst.strides_[1]] += src[e];
+    }
+}
+
 QUICKMLP_KERNEL_NAMESPACE_END

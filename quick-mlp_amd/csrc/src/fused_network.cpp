@@ -75,6 +75,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
             throw configuration_error("points_per_lane must be at most 8, but is %d", compileOptions_.pointsPerLane);
         compileOptions_.registerStaging = options.value("register_staging", compileOptions_.registerStaging);
         compileOptions_.sortPoints = options.value("sort_points", compileOptions_.sortPoints);
+        compileOptions_.sortTraining = options.value("sort_training", compileOptions_.sortTraining);
         compileOptions_.directInput = options.value("direct_input", compileOptions_.directInput);
         compileOptions_.sliceGradients = options.value("slice_gradients", compileOptions_.sliceGradients);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
@@ -1129,7 +1130,8 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
 void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool compileOnly)
 {
     if (flags <= 0 || flags >= ADJOINT_MODE_MAX_COMBINATIONS) throw std::runtime_error("At least one derivative must be enabled");
-    if (backwardKernel_[flags][sliceGradients ? 1 : 0].has_value() && !compileOnly) return;
+    const int variant = sliceGradients ? 1 : 0;
+    if (backwardKernel_[flags][variant].has_value() && !compileOnly) return;
     const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
     auto kl = QuickMLP::Instance().kernelLoader();
     auto logger = QuickMLP::Instance().getLogger();
@@ -1219,7 +1221,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
             }
         }
     }
-    if (!compileOnly) backwardKernel_[flags][sliceGradients ? 1 : 0] = std::move(ak);
+    if (!compileOnly) backwardKernel_[flags][variant] = std::move(ak);
 }
 
 void FusedNetwork::precompile(int adjointFlags)
@@ -1243,7 +1245,8 @@ void FusedNetwork::precompile(int adjointFlags)
             auto kl = QuickMLP::Instance().kernelLoader();
             const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
             const std::string scatter = "PointOrderScatter<" + std::to_string(channelsIn_ <= 4 ? 4 : channelsIn_ <= 8 ? 8 : 16) + ">";
-            for (const std::string& name : {std::string("PointOrderCount"), std::string("PointOrderScan"), scatter})
+            for (const std::string& name : {std::string("PointOrderCount"), std::string("PointOrderScan"), scatter,
+                                            std::string("PointOrderGatherRows"), std::string("PointOrderScatterAddRows")})
                 kl->getKernel("qmlp::kernel::" + name, source, loaderFlags(true));
             break;
         }
@@ -1336,7 +1339,9 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     // inference of a network with a large dense grid: rows of the input sorted by grid slab,
     // every row of the result written where its point stands in the caller's batch
     const int* orderAll = nullptr;
-    const bool sorted = !store && sortPoints(input, inputAll, orderAll, stream, noAlloc);
+    // (a training pass keeps the sorted rows and the order in its forward memory, for the adjoint pass)
+    void* sortedDestination = store && sortsTraining(numel) ? reinterpret_cast<char*>(tmpMemory) + sortedRowsOffset(numel) : nullptr;
+    const bool sorted = (!store || sortedDestination != nullptr) && sortPoints(input, inputAll, orderAll, stream, noAlloc, sortedDestination);
     const half* networkParams = parametersInference_.dataPtr<half>();
     for (long long start = 0; start < numel;) {
         // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
@@ -1361,20 +1366,33 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     }
 }
 
+bool FusedNetwork::pointOrderFor(int numel, kernel::PointOrderKey& key) const
+{
+    if (compileOptions_.sortPoints == 0 || (compileOptions_.sortPoints < 0 && numel < SORT_POINTS_MIN_BATCH)) return false;
+    if (channelsIn() > 16) return false;
+    for (const auto& e : encodings_)
+        if (e->pointOrderKey(key, compileOptions_.sortPoints < 0 ? numel : 0)) return true;
+    return false;
+}
+
+bool FusedNetwork::sortsTraining(int numel) const
+{
+    kernel::PointOrderKey key{};
+    return compileOptions_.sortTraining && pointOrderFor(numel, key);
+}
+
+size_t FusedNetwork::sortedRowsOffset(int numel) const
+{
+    return roundUp(static_cast<size_t>(perEntryForwardMemoryBytes_) * static_cast<size_t>(roundUp(numel, WARP_SIZE)), size_t(256));
+}
+
 bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
-                              bool noAlloc)
+                              bool noAlloc, void* destination)
 {
     const int numel = input.size(0);
-    if (compileOptions_.sortPoints == 0 || (compileOptions_.sortPoints < 0 && numel < SORT_POINTS_MIN_BATCH)) return false;
     kernel::PointOrderKey key{};
-    bool found = false;
-    for (const auto& e : encodings_)
-        if (e->pointOrderKey(key, compileOptions_.sortPoints < 0 ? numel : 0)) {
-            found = true;
-            break;
-        }
+    if (!pointOrderFor(numel, key)) return false;
     const int channels = input.size(1);
-    if (!found || channels > 16) return false;
     const int maxChannels = channels <= 4 ? 4 : channels <= 8 ? 8 : 16;
 
     auto& po = pointOrder_;
@@ -1389,10 +1407,11 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
         po.scatter = kl->getKernel("qmlp::kernel::PointOrderScatter<" + std::to_string(maxChannels) + ">", source, loaderFlags(false)).value();
     }
     constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 8 * BLOCK;   // as in point_order.h
-    // words: sorted inputs, order, totals, one histogram per chunk
-    const long long words = static_cast<long long>(numel) * (channels + 1) + (divUp(numel, CHUNK) + 1ll) * SLABS;
-    float* sortedData = nullptr;
-    long long capacity = numel;   // rows the workspace is laid out for
+    // words: slab totals and one histogram per chunk; then (unless the caller has room for them) sorted inputs and order
+    const long long histogramWords = (divUp(numel, CHUNK) + 1ll) * SLABS;
+    const long long rowWords = static_cast<long long>(numel) * (channels + 1);
+    const long long words = histogramWords + (destination ? 0 : rowWords);
+    int* totals = nullptr;
     if (noAlloc) {
         // the workspace is the library's static device buffer; the kernels get its address
         // as the same arguments that otherwise point into the network's own workspace
@@ -1408,15 +1427,14 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
                 static_cast<long long>(scratchBytes),
                 // per point: its row, its index and its share of the histogram of its chunk
                 static_cast<long long>((scratchBytes / sizeof(float) - 2.0 * SLABS) / (channels + 1 + static_cast<double>(SLABS) / CHUNK))));
-        sortedData = static_cast<float*>(scratch);
+        totals = static_cast<int*>(scratch);
     } else {
-        if (po.capacity < numel) {
+        if (po.capacityWords < words) {
             if (words > std::numeric_limits<int32_t>::max()) return false;   // beyond one tensor: the batch stays as it is
             po.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
-            po.capacity = numel;
+            po.capacityWords = words;
         }
-        sortedData = po.workspace.dataPtr<float>();
-        capacity = po.capacity;
+        totals = reinterpret_cast<int*>(po.workspace.dataPtr<float>());
         // resolves the static buffer of inferenceNoAlloc() on this device while allocating is
         // still allowed (the first look-up loads the library's own code object)
         void* scratch = nullptr;
@@ -1424,9 +1442,10 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
         std::string error;
         (void)device_code::staticScratch(&scratch, &scratchBytes, error);
     }
-    int* orderData = reinterpret_cast<int*>(sortedData + capacity * channels);   // the sorted rows come first: 16-byte aligned
-    int* totals = orderData + capacity;
     int* histogram = totals + SLABS;
+    // the histograms are a multiple of 4 KiB: the sorted rows behind them stay 16-byte aligned
+    float* sortedData = destination ? static_cast<float*>(destination) : reinterpret_cast<float*>(totals + histogramWords);
+    int* orderData = reinterpret_cast<int*>(sortedData + static_cast<long long>(numel) * channels);
 
     int count = numel;
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
@@ -1455,6 +1474,9 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
 size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlags)
 {
     (void)adjointFlags;
+    // a batch that trains in sorted order: its sorted rows and the order, behind the intermediates
+    if (sortsTraining(numElements))
+        return sortedRowsOffset(numElements) + roundUp(static_cast<size_t>(numElements) * (channelsIn() + 1) * sizeof(float), size_t(256));
     numElements = roundUp(numElements, WARP_SIZE);
     return static_cast<size_t>(perEntryForwardMemoryBytes_) * static_cast<size_t>(numElements);
 }
@@ -1493,6 +1515,12 @@ void FusedNetwork::zeroGradients()
 
 size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlags)
 {
+    const size_t bytes = adjointMemoryAsGiven(numElements, adjointFlags);
+    return bytes + sortedAdjointBytes(numElements, adjointFlags, bytes);
+}
+
+size_t FusedNetwork::adjointMemoryAsGiven(int numElements, AdjointModeFlags adjointFlags) const
+{
     if (adjointFlags <= 0 || adjointFlags >= ADJOINT_MODE_MAX_COMBINATIONS)
         throw std::runtime_error("At least one derivative must be enabled");
     int adjointChannels = 0;
@@ -1511,6 +1539,17 @@ size_t FusedNetwork::adjointMemory(int numElements, AdjointModeFlags adjointFlag
     bytes += roundUp(transposedWeightLayout(adjointFlags, transposed) * sizeof(half), size_t(16));
     // last: bucket cursors and records of the gradient slice kernels
     if (sliceGradients) bytes = roundUp(bytes, size_t(256)) + sliceGradientWorkspaceBytes(numElements);
+    return bytes;
+}
+
+size_t FusedNetwork::sortedAdjointBytes(int numElements, AdjointModeFlags adjointFlags, size_t bytesInFront) const
+{
+    // A batch that trains in sorted order: dL/dy gathered into that order, and the input gradients in that order
+    // before they are added to the caller's rows (each dense, 256-byte aligned, behind everything else).
+    if (!sortsTraining(numElements)) return 0;
+    size_t bytes = roundUp(bytesInFront, size_t(256)) - bytesInFront;
+    bytes += roundUp(static_cast<size_t>(numElements) * channelsOut() * sizeof(float), size_t(256));
+    if (adjointFlags & GRADIENTS_INPUT) bytes += roundUp(static_cast<size_t>(numElements) * channelsIn() * sizeof(float), size_t(256));
     return bytes;
 }
 
@@ -1557,18 +1596,63 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     CHECK_ERROR(tmpMemoryForward != nullptr, "adjoint() needs the temporary memory written by forward()");
     std::vector<long long> transposedOffsets;
     const size_t transposedHalves = transposedWeightLayout(adjointFlags, transposedOffsets);
-    if (hasNetworkGradients || transposedHalves > 0 || useSliceGradients(numel, adjointFlags)) {
+    if (hasNetworkGradients || transposedHalves > 0 || useSliceGradients(numel, adjointFlags) || sortsTraining(numel)) {
         CHECK_ERROR(tmpMemoryAdjoint != nullptr, "adjoint() needs temporary memory of adjointMemory() bytes");
         CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemoryAdjoint) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
     }
 
     const bool sliceGradients = useSliceGradients(numel, adjointFlags);
     CHECK_ERROR(!sliceGradients || numel < (1 << 27), "batches of 2^27 points or more: set options.slice_gradients to 0");
+    const bool sortedPoints = sortsTraining(numel);
     compileBackwardKernel(adjointFlags, sliceGradients);
     auto& ak = backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value();
 
     const int numTiles = divUp(numel, TILE_POINTS);
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
+    // a batch that the forward pass evaluated in sorted order: the rows as it sorted them, and for every row its
+    // place in the caller's batch (rows of dL/dy are read, rows of the input gradients written through it)
+    auto sortedInput = input.accessor<kernel::Tensor2Read<float>>();
+    auto sortedAdjOutput = adjOutput.accessor<kernel::Tensor2Read<float>>();
+    kernel::Tensor2RW<float> sortedAdjInput;
+    std::memset(&sortedAdjInput, 0, sizeof(sortedAdjInput));
+    if (hasInputGradients) sortedAdjInput = adjInput.accessor<kernel::Tensor2RW<float>>();
+    const int* pointOrder = nullptr;
+    if (sortedPoints) {
+        const float* rows = reinterpret_cast<const float*>(static_cast<const char*>(tmpMemoryForward) + sortedRowsOffset(numel));
+        sortedInput.data_ = rows;
+        sortedInput.strides_[0] = channelsIn();
+        sortedInput.strides_[1] = 1;
+        pointOrder = reinterpret_cast<const int*>(rows + static_cast<long long>(numel) * channelsIn());
+        // Scattered 8- and 16-byte accesses from inside the adjoint kernel cost a third of its time (cfg5: 577 us
+        // against 389 us on a batch the caller had sorted); two streaming kernels move the rows instead.
+        auto& po = pointOrder_;
+        if (!po.gatherRows.has_value()) {
+            auto kl = QuickMLP::Instance().kernelLoader();
+            const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
+            po.gatherRows = kl->getKernel("qmlp::kernel::PointOrderGatherRows", source, loaderFlags(false)).value();
+            po.scatterAddRows = kl->getKernel("qmlp::kernel::PointOrderScatterAddRows", source, loaderFlags(false)).value();
+        }
+        char* staging = static_cast<char*>(tmpMemoryAdjoint) + roundUp(adjointMemoryAsGiven(numel, adjointFlags), size_t(256));
+        float* adjOutputRows = reinterpret_cast<float*>(staging);
+        staging += roundUp(static_cast<size_t>(numel) * channelsOut() * sizeof(float), size_t(256));
+        {
+            long long elements = static_cast<long long>(numel) * channelsOut();
+            int channels = channelsOut();
+            auto src = adjOutput.accessor<kernel::Tensor2Read<float>>();
+            void* args[] = {&elements, &channels, &src, &pointOrder, &adjOutputRows};
+            po.gatherRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0, stream, args);
+        }
+        sortedAdjOutput.data_ = adjOutputRows;
+        sortedAdjOutput.strides_[0] = channelsOut();
+        sortedAdjOutput.strides_[1] = 1;
+        if (hasInputGradients) {
+            float* adjInputRows = reinterpret_cast<float*>(staging);
+            QMLP_HIP_CALL(qmlp_hip_memset_async(adjInputRows, 0, static_cast<size_t>(numel) * channelsIn() * sizeof(float), stream));
+            sortedAdjInput.data_ = adjInputRows;
+            sortedAdjInput.strides_[0] = channelsIn();
+            sortedAdjInput.strides_[1] = 1;
+        }
+    }
     const half* transposedWeights = nullptr;
     if (transposedHalves > 0) {
         size_t offset = static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64);
@@ -1590,11 +1674,9 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         const auto& ck = ak.adjoint;
         const int waves = ck.blockSize / WARP_SIZE;
         const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
-        auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
-        auto adjOutputAcc = adjOutput.accessor<kernel::Tensor2Read<float>>();
-        kernel::Tensor2RW<float> adjInputAcc;
-        std::memset(&adjInputAcc, 0, sizeof(adjInputAcc));
-        if (hasInputGradients) adjInputAcc = adjInput.accessor<kernel::Tensor2RW<float>>();
+        auto inputAcc = sortedInput;
+        auto adjOutputAcc = sortedAdjOutput;
+        auto adjInputAcc = sortedAdjInput;
         const half* networkParams = parametersInference_.dataPtr<half>();
         const half* forwardTmpMemory = static_cast<const half*>(tmpMemoryForward);
         half* adjointTmpMemory = static_cast<half*>(tmpMemoryAdjoint);
@@ -1603,6 +1685,15 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
+    }
+    if (sortedPoints && hasInputGradients) {
+        long long elements = static_cast<long long>(numel) * channelsIn();
+        int channels = channelsIn();
+        const float* src = sortedAdjInput.data_;
+        auto dst = adjInput.accessor<kernel::Tensor2RW<float>>();
+        void* args[] = {&elements, &channels, &src, &pointOrder, &dst};
+        pointOrder_.scatterAddRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0,
+                                                  stream, args);
     }
 
     // parameter gradients of the grids, slice by slice, from the adjoint of the encoded rows the kernel above stored
@@ -1616,7 +1707,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         if (hasNetworkGradients) offset += static_cast<size_t>(weightUpdateSlices(numTiles)) * numParameters_ * sizeof(float);
         offset += roundUp(transposedHalves * sizeof(half), size_t(16));
         char* workspace = static_cast<char*>(tmpMemoryAdjoint) + roundUp(offset, size_t(256));
-        auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
+        auto inputAcc = sortedInput;
         for (const auto& sk : ak.sliceGradients) {
             const auto& layout = sk.layout;
             int* cursors = reinterpret_cast<int*>(workspace);
@@ -1691,10 +1782,13 @@ void FusedNetwork::clearCachedKernels()
 {
     for (auto& perStore : forwardKernels_)
         for (auto& k : perStore) k = {};
-    for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i) backwardKernel_[i][0] = backwardKernel_[i][1] = {};
+    for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i)
+        for (auto& k : backwardKernel_[i]) k = {};
     pointOrder_.scan = {};
     pointOrder_.count = {};
     pointOrder_.scatter = {};
+    pointOrder_.gatherRows = {};
+    pointOrder_.scatterAddRows = {};
 }
 
 QUICKMLP_NAMESPACE_END

@@ -871,6 +871,51 @@ def test_inference_sorted_by_grid_slab_gives_the_same_bits_as_the_order_given():
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("slices", [0, 1])
+def test_training_sorted_by_grid_slab_matches_the_order_given(slices):
+    """The same network trains its large batches in the sorted order too (``sort_training``): the
+    forward pass leaves the sorted rows and the order in its temporary memory, the adjoint pass
+    reads dL/dy and writes the input gradients through the order. Outputs and input gradients
+    belong to single points and have to agree bit for bit with the pass over the batch as given;
+    weight and grid gradients are sums over the batch in another order. Ragged sizes, two batch
+    sizes in a row on one network, the scatter with atomics and the slice kernels, and a small
+    batch against both oracles."""
+    c = bc.CONFIGS[5]
+    cases = []
+    for sort_training in (True, False):
+        cfg = json.loads(json.dumps(c["cfg"]))
+        cfg.setdefault("options", {}).update({"sort_points": 1, "sort_training": sort_training, "slice_gradients": slices})
+        rng = np.random.default_rng(21)
+        case = Case(cfg, bc.ORACLE_ACTIVATIONS)
+        case.set_parameters(bc.make_parameters(5, rng).astype(np.float32))
+        case.set_table(0, bc.make_table(5, case.oracle.encodings[0][1].n_params, rng, 1.0))
+        cases.append(case)
+    sorted_, plain = cases
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    assert sorted_.net.forward_memory(1000, flags) > plain.net.forward_memory(1000, flags)
+    rng = np.random.default_rng(22)
+    for N in ((1 << 17) + 77, 8193, 63):
+        print("training sorted by slab: %d points" % N, flush=True)
+        X = bc.make_inputs(5, N, rng)
+        X[::13, 0] = -2.0                 # outside the box
+        adj = rng.uniform(-1, 1, (N, 2)).astype(np.float32)
+        a, b = sorted_.gpu_train(X, adj, flags), plain.gpu_train(X, adj, flags)
+        assert np.array_equal(a["out"], b["out"])
+        assert np.array_equal(a["adj_x"], b["adj_x"])
+        s = float(np.abs(b["grads"]).max())
+        assert s > 0
+        assert_close(a["grads"] / s, b["grads"] / s, "weight gradients", rel=1e-3, abs_=1e-4)
+        t = b["table_grads"][0]
+        assert_close(a["table_grads"][0], t, "grid gradients", rel=1e-3, abs_=1e-4 * float(np.abs(t).max()))
+        # input gradients alone (no adjoint memory at all)
+        only = sorted_.gpu_train(X, adj, FLAG_INPUT)
+        assert np.array_equal(only["adj_x"], b["adj_x"])
+    N = 3000
+    X = bc.make_inputs(5, N, rng)
+    adj = (rng.uniform(-1, 1, (N, 2)) / N).astype(np.float32)
+    check_gradients(sorted_, X, adj, flags, sorted_.gpu_train(X, adj, flags), kinks=True)
+
+
 @pytest.mark.parametrize("n_in,n_out", [(4, 4), (2, 2), (8, 16), (4, 2), (3, 1)])
 def test_rows_moved_as_vectors_and_rows_that_cannot_be(n_in, n_out):
     """Input, output, dL/dy and input-gradient rows whose channels lie side by side move 8 or 16
