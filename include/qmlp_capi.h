@@ -124,6 +124,11 @@ int qmlp_network_clear_cached_kernels(qmlp_network_t network);
  * (adjoint_flags <= 0: inference and forward only). No counterpart in the reference,
  * where kernels can only be compiled with a device present. */
 int qmlp_network_precompile(qmlp_network_t network, int adjoint_flags);
+/* Loads the kernels that calls on a batch of `numel` points take (inference; forward and adjoint too if
+ * adjoint_flags > 0) and allocates the workspace that orders such a batch by grid slab, so that the calls
+ * themselves only enqueue kernels (for callers that capture them into a HIP graph). No counterpart in the
+ * reference, whose first call on a network compiles its kernels. */
+int qmlp_network_prepare(qmlp_network_t network, int numel, int adjoint_flags);
 /* The generated device source; kind = "forward" | "backward" | "weight_update". */
 int qmlp_network_generated_source(qmlp_network_t network, const char* kind, int adjoint_flags, char** source);
 

@@ -84,6 +84,12 @@ int qmlp_hip_module_compile(const char* source, const char* source_name,
                             const char* arch,
                             qmlp_hip_module* module, char** log);
 void qmlp_hip_free_string(char* s);
+/* What qmlp_hip_module_compile(..., arch, ...) compiles for and with: "<architecture>;hiprtc <major>.<minor>",
+ * the architecture resolved as there (arch, else the current device, else gfx950) and cut at the first ':'. Part of the key of the
+ * on-disk kernel cache (the reference's ckl::KernelLoader keys its cache on source and flags only,
+ * third-party/cuda-kernel-loader as used in src_cpp/src/qmlp.cpp:23-35). Returns a malloc'ed string
+ * (free with qmlp_hip_free_string) through `target`. */
+int qmlp_hip_compile_target(const char* arch, char** target);
 /* Wraps an existing code object (e.g. from the on-disk kernel cache). */
 int qmlp_hip_module_from_code(const void* code, size_t size, qmlp_hip_module* module);
 int qmlp_hip_module_code(qmlp_hip_module module, const void** code, size_t* size);

@@ -148,6 +148,7 @@ private:
      */
     bool sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
                     bool noAlloc = false, void* destination = nullptr);
+    void loadPointOrderKernels(bool rowMoves);
     /** The slab key of the encoding that orders a batch of numel points, if such a batch is ordered at all
      *  (a function of the specification and numel alone). */
     bool pointOrderFor(int numel, kernel::PointOrderKey& key) const;
@@ -321,6 +322,15 @@ public:
      * (flags < 0: inference and forward only). Fills the kernel disk cache.
      */
     void precompile(int adjointFlags);
+
+    /**
+     * Everything a later call on a batch of numel points would otherwise do on its first use, on the current
+     * device: loads (or compiles) the kernels that inference() takes for a batch of this size and, with
+     * adjointFlags > 0, those of forward() and adjoint(); allocates the workspace that orders such a batch by
+     * grid slab. After it, calls on batches of this size only enqueue kernels (nothing is loaded or
+     * allocated), e.g. under HIP graph capture. No counterpart in the reference.
+     */
+    void prepare(int numel, int adjointFlags);
 
     /** The generated device source of a kernel kind: "inference", "backward", "weight_update". */
     std::string generatedSource(const std::string& kind, int adjointFlags = 0);

@@ -349,6 +349,13 @@ int qmlp_network_precompile(qmlp_network_t network, int adjoint_flags)
     QMLP_API_END
 }
 
+int qmlp_network_prepare(qmlp_network_t network, int numel, int adjoint_flags)
+{
+    QMLP_API_BEGIN
+    network->network->prepare(numel, adjoint_flags);
+    QMLP_API_END
+}
+
 int qmlp_network_generated_source(qmlp_network_t network, const char* kind, int adjoint_flags, char** source)
 {
     QMLP_API_BEGIN

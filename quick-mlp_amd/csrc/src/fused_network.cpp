@@ -1375,6 +1375,54 @@ bool FusedNetwork::pointOrderFor(int numel, kernel::PointOrderKey& key) const
     return false;
 }
 
+void FusedNetwork::loadPointOrderKernels(bool rowMoves)
+{
+    auto& po = pointOrder_;
+    auto kl = QuickMLP::Instance().kernelLoader();
+    const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
+    if (!po.scatter.has_value()) {
+        const int maxChannels = channelsIn_ <= 4 ? 4 : channelsIn_ <= 8 ? 8 : 16;
+        po.scan = kl->getKernel("qmlp::kernel::PointOrderScan", source, loaderFlags(false)).value();
+        po.count = kl->getKernel("qmlp::kernel::PointOrderCount", source, loaderFlags(false)).value();
+        po.scatter = kl->getKernel("qmlp::kernel::PointOrderScatter<" + std::to_string(maxChannels) + ">", source, loaderFlags(false)).value();
+    }
+    if (rowMoves && !po.gatherRows.has_value()) {
+        po.gatherRows = kl->getKernel("qmlp::kernel::PointOrderGatherRows", source, loaderFlags(false)).value();
+        po.scatterAddRows = kl->getKernel("qmlp::kernel::PointOrderScatterAddRows", source, loaderFlags(false)).value();
+    }
+}
+
+void FusedNetwork::prepare(int numel, int adjointFlags)
+{
+    CHECK_ERROR(numel >= 0, "prepare(): the batch size must not be negative");
+    CHECK_ERROR(adjointFlags >= 0 && adjointFlags < ADJOINT_MODE_MAX_COMBINATIONS, "prepare(): unknown adjoint flags ", adjointFlags);
+    if (numel == 0) return;
+    // the forward kernels that launchForward() takes for the pieces of a batch of this size
+    for (int store = 0; store <= (adjointFlags > 0 ? 1 : 0); ++store)
+        for (long long start = 0; start < numel;) {
+            int launchTiles = 0;
+            const auto& ck = forwardKernelFor(store != 0, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles);
+            start += std::min<long long>({static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS,
+                                          numel - start});
+        }
+    // the sort of a batch that is evaluated slab by slab: kernels, workspace, and the static buffer of inferenceNoAlloc()
+    kernel::PointOrderKey key{};
+    if (pointOrderFor(numel, key)) {
+        loadPointOrderKernels(adjointFlags > 0 && sortsTraining(numel));
+        constexpr long long SLABS = 1024, CHUNK = 8 * 1024;   // as in sortPoints()
+        const long long words = (divUp<long long>(numel, CHUNK) + 1) * SLABS + static_cast<long long>(numel) * (channelsIn_ + 1);
+        if (pointOrder_.capacityWords < words && words <= std::numeric_limits<int32_t>::max()) {
+            pointOrder_.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
+            pointOrder_.capacityWords = words;
+        }
+        void* scratch = nullptr;
+        size_t scratchBytes = 0;
+        std::string error;
+        (void)device_code::staticScratch(&scratch, &scratchBytes, error);
+    }
+    if (adjointFlags > 0) compileBackwardKernel(adjointFlags, useSliceGradients(numel, adjointFlags));
+}
+
 bool FusedNetwork::sortsTraining(int numel) const
 {
     kernel::PointOrderKey key{};
@@ -1399,13 +1447,8 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     if (!po.scatter.has_value() && noAlloc)
         throw std::runtime_error("The kernels that order the batch are not loaded yet, and loading allocates: run "
                                  "inference() once on a batch of the same size first");
-    if (!po.scatter.has_value()) {
-        auto kl = QuickMLP::Instance().kernelLoader();
-        const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
-        po.scan = kl->getKernel("qmlp::kernel::PointOrderScan", source, loaderFlags(false)).value();
-        po.count = kl->getKernel("qmlp::kernel::PointOrderCount", source, loaderFlags(false)).value();
-        po.scatter = kl->getKernel("qmlp::kernel::PointOrderScatter<" + std::to_string(maxChannels) + ">", source, loaderFlags(false)).value();
-    }
+    loadPointOrderKernels(false);
+    (void)maxChannels;
     constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 8 * BLOCK;   // as in point_order.h
     // words: slab totals and one histogram per chunk; then (unless the caller has room for them) sorted inputs and order
     const long long histogramWords = (divUp(numel, CHUNK) + 1ll) * SLABS;
@@ -1626,12 +1669,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         // Scattered 8- and 16-byte accesses from inside the adjoint kernel cost a third of its time (cfg5: 577 us
         // against 389 us on a batch the caller had sorted); two streaming kernels move the rows instead.
         auto& po = pointOrder_;
-        if (!po.gatherRows.has_value()) {
-            auto kl = QuickMLP::Instance().kernelLoader();
-            const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
-            po.gatherRows = kl->getKernel("qmlp::kernel::PointOrderGatherRows", source, loaderFlags(false)).value();
-            po.scatterAddRows = kl->getKernel("qmlp::kernel::PointOrderScatterAddRows", source, loaderFlags(false)).value();
-        }
+        loadPointOrderKernels(true);
         char* staging = static_cast<char*>(tmpMemoryAdjoint) + roundUp(adjointMemoryAsGiven(numel, adjointFlags), size_t(256));
         float* adjOutputRows = reinterpret_cast<float*>(staging);
         staging += roundUp(static_cast<size_t>(numel) * channelsOut() * sizeof(float), size_t(256));

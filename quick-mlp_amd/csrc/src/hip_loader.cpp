@@ -192,6 +192,38 @@ int qmlp_hip_event_elapsed_ms(qmlp_hip_event start, qmlp_hip_event stop, float* 
                  "hipEventElapsedTime");
 }
 
+static std::string resolveArchitecture(const char* arch)
+{
+    if (arch && *arch) return arch;
+    std::string archName;
+    int count = 0;
+    qmlp_hip_device_count(&count);
+    if (count > 0) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
+            archName = p.gcnArchName;
+    }
+    if (archName.empty()) archName = "gfx950";
+    return archName;
+}
+
+int qmlp_hip_compile_target(const char* arch, char** target)
+{
+    if (!target) return fail("qmlp_hip_compile_target: target is NULL");
+    int major = 0, minor = 0;
+    if (int rc = checkRtc(hiprtcVersion(&major, &minor), "hiprtcVersion")) return rc;
+    // the processor without its feature suffixes (":sramecc+:xnack-"): a code object compiled for the plain
+    // name runs with any of them, and a cache filled on a machine without a GPU has to be found on one with
+    std::string processor = resolveArchitecture(arch);
+    processor = processor.substr(0, processor.find(':'));
+    const std::string text = processor + ";hiprtc " + std::to_string(major) + "." + std::to_string(minor);
+    *target = static_cast<char*>(std::malloc(text.size() + 1));
+    if (!*target) return fail("qmlp_hip_compile_target: out of memory");
+    std::memcpy(*target, text.c_str(), text.size() + 1);
+    return 0;
+}
+
 int qmlp_hip_module_compile(const char* source, const char* source_name,
                             const char* const* header_names, const char* const* headers,
                             int num_headers,
@@ -203,20 +235,7 @@ int qmlp_hip_module_compile(const char* source, const char* source_name,
     *module = nullptr;
     if (log) *log = nullptr;
 
-    std::string archName;
-    if (arch && *arch) {
-        archName = arch;
-    } else {
-        int count = 0;
-        qmlp_hip_device_count(&count);
-        if (count > 0) {
-            int dev = 0;
-            hipDeviceProp_t p;
-            if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
-                archName = p.gcnArchName;
-        }
-        if (archName.empty()) archName = "gfx950";
-    }
+    const std::string archName = resolveArchitecture(arch);
 
     hiprtcProgram prog;
     if (int rc = checkRtc(hiprtcCreateProgram(&prog, source, source_name ? source_name : "qmlp_kernel.hip",

@@ -235,6 +235,16 @@ std::string KernelLoader::cacheKey(const std::string& kernelName, const std::str
 {
     std::string all = includedHeadersDigest(source);
     all += '\0';
+    // what the code object is compiled for and with: a cache directory may outlive a ROCm update or be
+    // carried to a machine with another GPU
+    {
+        char* target = nullptr;
+        if (qmlp_hip_compile_target(std::getenv("QMLP_OFFLOAD_ARCH"), &target) == 0 && target) {
+            all += target;
+            qmlp_hip_free_string(target);
+        }
+    }
+    all += '\0';
     all += kernelName;
     all += '\0';
     for (const auto& o : options) {

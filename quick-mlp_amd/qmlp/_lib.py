@@ -79,6 +79,7 @@ _SIGNATURES = {
     "qmlp_network_adjoint": [_vp, _TD, _TD, _ci, _TD, _vp, _vp, _vp],
     "qmlp_network_clear_cached_kernels": [_vp],
     "qmlp_network_precompile": [_vp, _ci],
+    "qmlp_network_prepare": [_vp, _ci, _ci],
     "qmlp_network_generated_source": [_vp, ctypes.c_char_p, _ci, _pstr],
     "qmlp_encoding_create": [ctypes.c_char_p, _P(_vp)],
     "qmlp_encoding_destroy": [_vp],

@@ -463,6 +463,11 @@ class Network:
     def precompile(self, adjoint_flags=7):
         check(lib.qmlp_network_precompile(self._handle, int(adjoint_flags)))
 
+    def prepare(self, num_elements, adjoint_flags=0):
+        """Loads the kernels and allocates the workspace that calls on a batch of this size need,
+        so that those calls only enqueue kernels (e.g. under graph capture)."""
+        check(lib.qmlp_network_prepare(self._handle, int(num_elements), int(adjoint_flags)))
+
     def generated_source(self, kind, adjoint_flags=0):
         return _lib.get_string(lib.qmlp_network_generated_source, self._handle, kind.encode(), int(adjoint_flags))
 

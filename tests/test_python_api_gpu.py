@@ -353,6 +353,63 @@ def test_inference_and_train_step_replay_from_a_hip_graph():
         assert torch.allclose(got[4], want[4], rtol=1e-5, atol=1e-7), "input gradients of replay %d" % replay
 
 
+def test_a_prepared_network_is_captured_without_an_eager_call_first():
+    """``prepare(n, flags)`` loads the kernels of a batch of that size and allocates the workspace that
+    orders it by grid slab. A capture right after it, without any eager call before, records inference
+    and a train step of a network whose batches are sorted (dense grid beyond the L2, ``sort_points``
+    1): loading a kernel or allocating inside the capture would fail it."""
+    import baseline_configs as bc
+    cfg = json.loads(json.dumps(bc.CONFIGS[5]["cfg"]))
+    cfg.setdefault("options", {})["sort_points"] = 1
+    cfg = json.dumps(cfg)
+    warm_or_gpu(network_cfg=cfg)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    N, flags = 20000, 7
+
+    def make():
+        net = qmlp.Network(cfg)
+        return net, net.encoding(0)
+
+    net, enc = make()
+    params = ((torch.rand(net.num_network_parameters(), device="cuda", generator=g) - 0.5) * 0.5).half()
+    table = (torch.rand(enc.num_parameters(), device="cuda", generator=g) - 0.5).to(enc.parameter_dtype())
+    tables = [table, None]
+    x = torch.rand((N, 4), device="cuda", generator=g)
+    adj = torch.rand((N, 2), device="cuda", generator=g)
+    grad_net = torch.zeros(net.num_network_parameters(), device="cuda")
+    grad_table = torch.zeros(enc.num_parameters(), device="cuda")
+    adj_x = torch.zeros_like(x)
+
+    def step(n):
+        out, tmp = n.forward_raw(x, params, tables, flags)
+        n.adjoint_raw(x, adj, flags, tmp, params, tables, grad_network=grad_net,
+                      grad_encodings=[grad_table, None], adj_input=adj_x)
+        return out, n.inference(x, params, tables)
+
+    net.prepare(N, flags)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("prepared network: capture", flush=True)
+    with torch.cuda.graph(graph):
+        out_g, inf_g = step(net)
+    print("prepared network: replay", flush=True)
+    graph.replay()
+    torch.cuda.synchronize()
+    got = [t.clone() for t in (out_g, inf_g, grad_net, grad_table, adj_x)]
+    # a second network object, eager
+    other, _ = make()
+    for t in (grad_net, grad_table, adj_x):
+        t.zero_()
+    out, inf = step(other)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0], out) and torch.equal(got[1], inf)
+    assert torch.equal(got[2], grad_net)
+    assert torch.allclose(got[3], grad_table, rtol=1e-4, atol=1e-6)
+    assert torch.equal(got[4], adj_x)
+    with pytest.raises(qmlp.QmlpError):
+        net.prepare(-1, 0)
+
+
 def two_grid_cfg():
     grid = {"id": "HashGrid", "start_in": 0, "n_in": 2, "n_levels": 2, "n_features_per_level": 4,
             "log2_hashmap_size": 10, "min_resolution": 8, "max_resolution": 64, "combination_mode": "concat",
