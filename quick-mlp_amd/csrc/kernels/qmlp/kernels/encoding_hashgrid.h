@@ -78,6 +78,29 @@ __device__ __forceinline__ void loadFeatures(const T* __restrict__ p, float (&v)
     }
 }
 
+/** The F values of a table entry as they are loaded (the widest aligned vectors), converted to float only when
+ *  asked for: nothing touches the loaded registers in between, so the loads may stay in flight. */
+template <int F, typename T>
+struct HeldFeatures
+{
+    static constexpr int MAXV = 16 / static_cast<int>(sizeof(T));
+    static constexpr int V = (F % 8 == 0 && MAXV >= 8) ? 8 : (F % 4 == 0 && MAXV >= 4) ? 4 : (F % 2 == 0) ? 2 : 1;
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    vec_t part[F / V];
+    __device__ __forceinline__ void load(const T* __restrict__ p)
+    {
+#pragma unroll
+        for (int i = 0; i < F / V; ++i) part[i] = *reinterpret_cast<const vec_t*>(p + i * V);
+    }
+    __device__ __forceinline__ void toFloat(float (&v)[F]) const
+    {
+#pragma unroll
+        for (int i = 0; i < F / V; ++i)
+#pragma unroll
+            for (int j = 0; j < V; ++j) v[i * V + j] = static_cast<float>(part[i][j]);
+    }
+};
+
 /** Loads two consecutive table entries (2*F values) with one wide load; the address is
  *  only guaranteed to be aligned to one entry. */
 template <int F, typename T>

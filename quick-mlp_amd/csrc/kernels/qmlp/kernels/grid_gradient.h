@@ -179,12 +179,13 @@ struct GridGradientRecords
         }
     }
 
-    template <int LEVEL>
+    template <int LEVEL, bool INPUT_GRADIENTS>
     __device__ __forceinline__ static void runLevel(int p, bool valid, long long numel, const float (&pos)[D],
                                                     const f16* __restrict__ adjEncoded, const param_t& params,
                                                     unsigned* __restrict__ records, int* __restrict__ cursors,
                                                     unsigned* sStage, unsigned short* sBucketOf, int* sHist,
-                                                    int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits)
+                                                    int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits,
+                                                    float (&adjPos)[D])
     {
         constexpr bool hashed = Cfg::hashed[LEVEL];
         constexpr int PD = hashed ? 0 : D - 1;
@@ -198,8 +199,10 @@ struct GridGradientRecords
         // my records of this level, in registers, and their places among the workgroup's records of the same slice
         unsigned rec[PAIRS][RW];
         int bucket[PAIRS], rank[PAIRS];
+        const typename Grid::LevelSetup s = Grid::setupLevel(LEVEL, pos);
+        detail::HeldFeatures<F, typename Cfg::table_t> held[Grid::NC];
+        (void)held;
         if (valid) {
-            const typename Grid::LevelSetup s = Grid::setupLevel(LEVEL, pos);
             const f16* adjRow = adjEncoded + static_cast<long long>(p / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
                 + (CHANNEL_OFFSET + (Cfg::Concat ? LEVEL * F : 0)) * TILE_POINTS + (p % TILE_POINTS);
             unsigned adjWords[(F + 1) / 2];
@@ -211,6 +214,14 @@ struct GridGradientRecords
                 adjWords[i / 2] |= bits << (16 * (i % 2));
                 // largest magnitude seen (as fp16 bits without the sign: ordered like the values, NaN above infinity)
                 maxAdjBits = max(maxAdjBits, bits & 0x7fffu);
+            }
+            if constexpr (INPUT_GRADIENTS) {
+                // the entries of all corners, for this grid's share of dL/dinput: loaded here and, where they take
+                // few registers, used at the end of the level, so that the sort of the records in between hides
+                // their latency (a dense 4-D grid with 8 features would hold 64 registers: 304 against 282 us)
+#pragma unroll
+                for (int c = 0; c < Grid::NC; ++c) held[c].load(params.parametersForward + Grid::cornerOffset(LEVEL, s, c));
+                if constexpr (!DEFER_ENTRIES) positionGradient<LEVEL>(p, s, held, adjEncoded, adjPos);
             }
 #pragma unroll
             for (int c = 0; c < PAIRS; ++c) {
@@ -304,20 +315,66 @@ struct GridGradientRecords
                 addToTensor(r, params.parametersBackward + base + static_cast<unsigned>(b) * SLICE_FLOATS);
             }
         }
+
+        if constexpr (INPUT_GRADIENTS && DEFER_ENTRIES) {
+            if (valid) positionGradient<LEVEL>(p, s, held, adjEncoded, adjPos);
+        }
     }
 
+    /** Registers worth holding across the sort of a level's records: 64 bytes of table entries per lane. */
+    static constexpr bool DEFER_ENTRIES = Grid::NC * F * static_cast<int>(sizeof(typename Cfg::table_t)) <= 64;
+
+    /**
+     * This level's share of the gradient with respect to the position, operation by operation as
+     * EncodingHashGrid::adjoint computes it (same corner order, same products), so both give the same bits.
+     */
     template <int LEVEL>
+    __device__ __forceinline__ static void positionGradient(int p, const typename Grid::LevelSetup& s,
+                                                            const detail::HeldFeatures<F, typename Cfg::table_t> (&held)[Grid::NC],
+                                                            const f16* __restrict__ adjEncoded, float (&adjPos)[D])
+    {
+        const f16* adjRow = adjEncoded + static_cast<long long>(p / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
+            + (CHANNEL_OFFSET + (Cfg::Concat ? LEVEL * F : 0)) * TILE_POINTS + (p % TILE_POINTS);
+        float adjFeat[F];
+#pragma unroll
+        for (int i = 0; i < F; ++i) adjFeat[i] = static_cast<float>(adjRow[i * TILE_POINTS]);
+        float lvl[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) lvl[d] = 0.f;
+#pragma unroll
+        for (int c = 0; c < Grid::NC; ++c) {
+            float v[F];
+            held[c].toFloat(v);
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < F; ++i) dot += adjFeat[i] * v[i];
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                float prod = 1.f;
+#pragma unroll
+                for (int e = D - 1; e >= 0; --e)
+                    if (e != d) prod *= ((c >> e) & 1) ? s.f[e] : (1.f - s.f[e]);
+                lvl[d] += (((c >> d) & 1) ? prod : -prod) * dot;
+            }
+        }
+        const float scale = Cfg::ResolutionFactor ? static_cast<float>(Cfg::resolution[LEVEL] - 1) : 1.f;
+#pragma unroll
+        for (int d = 0; d < D; ++d) adjPos[d] += scale * lvl[d];
+    }
+
+    template <int LEVEL, bool INPUT_GRADIENTS>
     __device__ __forceinline__ static void runLevels(int p, bool valid, long long numel, const float (&pos)[D],
                                                      const f16* __restrict__ adjEncoded, const param_t& params,
                                                      unsigned* __restrict__ records, int* __restrict__ cursors,
                                                      unsigned* sStage, unsigned short* sBucketOf, int* sHist,
-                                                     int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits)
+                                                     int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits,
+                                                     float (&adjPos)[D])
     {
         if constexpr (LEVEL < Cfg::Levels) {
-            runLevel<LEVEL>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf, sHist, sLocalBase,
-                            sGlobalBase, maxAdjBits);
-            runLevels<LEVEL + 1>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf, sHist, sLocalBase,
-                                 sGlobalBase, maxAdjBits);
+            runLevel<LEVEL, INPUT_GRADIENTS>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf, sHist,
+                                             sLocalBase, sGlobalBase, maxAdjBits, adjPos);
+            runLevels<LEVEL + 1, INPUT_GRADIENTS>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf,
+                                                  sHist, sLocalBase, sGlobalBase, maxAdjBits, adjPos);
         }
     }
 };
@@ -327,14 +384,15 @@ struct GridGradientRecords
  * records: room for levelOffset(Levels, layoutNumel) records; cursors: one int per bucket, then one word that
  * receives the largest magnitude among the adjoints (fp16 bits without the sign); all zeroed by the caller.
  */
-template <typename Cfg, int ROW_CHANNELS, int CHANNEL_OFFSET, int SLICE_FLOATS, int POINTS>
+template <typename Cfg, int ROW_CHANNELS, int CHANNEL_OFFSET, int SLICE_FLOATS, int POINTS, bool INPUT_GRADIENTS>
 __global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
     int numel,
     int layoutNumel,                          //points the buckets are laid out for (numel rounded up to whole tiles)
     const Tensor2Read<float> inputs,          //shape (numel, Cin)
     const half* __restrict__ adjEncodedH,     //adjoint of the encoded rows: (tiles, ROW_CHANNELS, 64)
     const HashGridParams<typename Cfg::table_t, Cfg::Dim> params,
-    unsigned* __restrict__ records, int* __restrict__ cursors)
+    unsigned* __restrict__ records, int* __restrict__ cursors,
+    Tensor2RW<float> adjInputs)               //INPUT_GRADIENTS: shape (numel, Cin), this grid's share of dL/dinput is added
 {
     typedef GridGradientRecords<Cfg, ROW_CHANNELS, CHANNEL_OFFSET, SLICE_FLOATS, POINTS> Impl;
     constexpr int D = Cfg::Dim;
@@ -358,8 +416,21 @@ __global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
                 pos[d] = (in - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
             }
         }
-        Impl::template runLevels<0>(p, valid, layoutNumel, pos, reinterpret_cast<const f16*>(adjEncodedH), params, records, cursors,
-                                    sStage, sBucketOf, sHist, sLocalBase, sGlobalBase, maxAdjBits);
+        float adjPos[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) adjPos[d] = 0.f;
+        Impl::template runLevels<0, INPUT_GRADIENTS>(p, valid, layoutNumel, pos, reinterpret_cast<const f16*>(adjEncodedH), params,
+                                                     records, cursors, sStage, sBucketOf, sHist, sLocalBase, sGlobalBase, maxAdjBits,
+                                                     adjPos);
+        if constexpr (INPUT_GRADIENTS) {
+            // every point belongs to one lane of one workgroup: a plain read-modify-write
+            if (valid) {
+#pragma unroll
+                for (int d = 0; d < D; ++d)
+                    adjInputs.data_[static_cast<long long>(p) * adjInputs.strides_[0]
+                                    + static_cast<long long>(d + Cfg::Start) * adjInputs.strides_[1]] += adjPos[d] * params.boundingBoxInvSize[d];
+            }
+        }
         __syncthreads();
     }
     // the largest adjoint of the workgroup: one LDS word, then one atomic per workgroup

@@ -75,7 +75,7 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     // barriers inside the loop), wavefronts without a tile work on zeros.
     constexpr bool HAS_STREAMED_LAYERS = $$HAS_STREAMED_LAYERS$$;
     // the adjoint of the encoded input is only needed if something sits behind it
-    constexpr bool NEEDS_ENCODING_ADJOINT = HAS_INPUT_GRADIENTS || HAS_ENCODING_GRADIENTS;
+    constexpr bool NEEDS_ENCODING_ADJOINT = $$NEEDS_ENCODING_ADJOINT$$;
     // true: the adjoint of the encoded rows is stored (channel-major per tile, behind the adjoint
     // pre-activations) for the kernels that sum the parameter gradients of grids slice by slice
     constexpr bool STORE_ENCODED_ADJOINT = $$STORE_ENCODED_ADJOINT$$;

@@ -761,7 +761,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
     replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes(blockSize));
-    replaceAll(code, "$$HAS_INPUT_GRADIENTS$$", hasInputGradients ? "true" : "false");
+    // (set below: input gradients that the kernels of the gradient slices compute are none of this kernel's)
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
     replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
     std::vector<int> ldsW, ldsB;
@@ -824,16 +824,21 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     std::vector<LdsGradients> ldsGradients;
     ldsGradientLayout(flags, blockSize, ldsGradients, sliceGradients);
     int encodingOffset = 0;
-    bool storeEncodedAdjoint = false, gradientsInKernel = false;
+    bool storeEncodedAdjoint = false, gradientsInKernel = false, inputGradientsInKernel = false;
     for (size_t encodingIdx = 0; encodingIdx < encodings_.size(); ++encodingIdx) {
         const auto& e = encodings_[encodingIdx];
         bool parameterGradients = hasEncodingGradients && e->hasParameters();
+        bool inputGradients = hasInputGradients;
         if (parameterGradients && sliceGradients && offersSlices(*e)) {
-            // this kernel only stores the adjoint of the encoded rows; a slice kernel sums the gradients
+            // This kernel only stores the adjoint of the encoded rows; the records kernel of the gradient slices,
+            // which walks the levels of every point anyway, also gathers for this grid's share of dL/dinput
+            // (at 16 wavefronts per compute unit instead of the 8 this kernel's registers leave).
             parameterGradients = false;
+            inputGradients = false;
             storeEncodedAdjoint = true;
         }
         gradientsInKernel = gradientsInKernel || parameterGradients;
+        inputGradientsInKernel = inputGradientsInKernel || inputGradients;
         const std::string name = e->qualifiedName();
         const LdsGradients& lg = ldsGradients[encodingIdx];
         if (lg.levels > 0) {
@@ -848,7 +853,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
             parameterGradients ? "!" + name + "::HasTileScatter" : std::string("false");
         callEncodings << "                {\n                    auto adjEncodingOutputK = adjEncodingOutput + "
                       << encodingOffset << ";\n                    " << name << "::template adjoint<"
-                      << (hasInputGradients ? "true" : "false") << ", " << perPointParameterGradients
+                      << (inputGradients ? "true" : "false") << ", " << perPointParameterGradients
                       << ">(encodingInput, adjEncodingOutputK, adjEncodingInput";
         if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
         callEncodings << ");\n                }\n";
@@ -871,7 +876,10 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
         replaceAll(code, "$$OFFSET_ENCODED_ADJOINT$$", std::to_string(adjointChannels));
     }
     // the adjoint of the encoded rows goes through the staging rows only if a lane per point still needs it
-    replaceAll(code, "$$NEEDS_STAGED_ADJOINT$$", (hasInputGradients || gradientsInKernel) ? "true" : "false");
+    replaceAll(code, "$$NEEDS_STAGED_ADJOINT$$", (inputGradientsInKernel || gradientsInKernel) ? "true" : "false");
+    replaceAll(code, "$$HAS_INPUT_GRADIENTS$$", inputGradientsInKernel ? "true" : "false");
+    // layer 0 still has to produce the adjoint of the encoded rows for the kernels behind this one
+    replaceAll(code, "$$NEEDS_ENCODING_ADJOINT$$", (hasInputGradients || hasEncodingGradients) ? "true" : "false");
     replaceAll(code, "$$CALL_ENCODING_SCATTER$$", callScatter.str());
     replaceAll(code, "$$ZERO_LDS_GRADIENTS$$", zeroLds.str());
     replaceAll(code, "$$FLUSH_LDS_GRADIENTS$$", flushLds.str().empty() ? std::string() : "    __syncthreads();\n" + flushLds.str());
@@ -1179,8 +1187,9 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
             source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient.h");
             sk.records.blockSize = layout.pointsPerWorkgroup;
             sk.records.sharedMemorySize = layout.recordsLdsBytes;
-            sk.records.fun = kl->getKernel(format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d>", layout.configType.c_str(),
-                                                  layers_[0].channelsIn, offset, layout.sliceFloats, layout.pointsPerWorkgroup),
+            sk.records.fun = kl->getKernel(format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d, %s>", layout.configType.c_str(),
+                                                  layers_[0].channelsIn, offset, layout.sliceFloats, layout.pointsPerWorkgroup,
+                                                  (flags & GRADIENTS_INPUT) ? "true" : "false"),
                                            source.str(), loaderFlags(compileOnly)).value();
             sk.kernel.blockSize = 1024;
             sk.kernel.sharedMemorySize = layout.sliceFloats * static_cast<int>(sizeof(long long));
@@ -1724,16 +1733,6 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
     }
-    if (sortedPoints && hasInputGradients) {
-        long long elements = static_cast<long long>(numel) * channelsIn();
-        int channels = channelsIn();
-        const float* src = sortedAdjInput.data_;
-        auto dst = adjInput.accessor<kernel::Tensor2RW<float>>();
-        void* args[] = {&elements, &channels, &src, &pointOrder, &dst};
-        pointOrder_.scatterAddRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0,
-                                                  stream, args);
-    }
-
     // parameter gradients of the grids, slice by slice, from the adjoint of the encoded rows the kernel above stored
     if (!ak.sliceGradients.empty()) {
         int adjointChannels = 0;
@@ -1759,7 +1758,8 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
             int numelPadded = static_cast<int>(numel64);   // the layout of the buckets is that of adjointMemory()
             {
                 // the records kernel walks over the real points, but lays its buckets out for the padded batch
-                void* args[] = {&numel, &numelPadded, &inputAcc, &adjEncoded, params.data(), &records, &cursors};
+                auto adjInputAcc = sortedAdjInput;   // this grid's share of dL/dinput (zeros in it if none is asked for: unused)
+                void* args[] = {&numel, &numelPadded, &inputAcc, &adjEncoded, params.data(), &records, &cursors, &adjInputAcc};
                 sk.records.fun.launch(std::min(divUp(numel, sk.records.blockSize), sk.records.fullGrid), sk.records.blockSize,
                                       sk.records.sharedMemorySize, stream, args);
             }
@@ -1771,6 +1771,17 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
             void* args[] = {&numelPadded, &recordsRead, &cursorsRead, &gradients, &items};
             sk.kernel.fun.launch(static_cast<int>(layout.items.size()), sk.kernel.blockSize, sk.kernel.sharedMemorySize, stream, args);
         }
+    }
+
+    // the input gradients of a batch that trained in sorted order: back to the caller's rows
+    if (sortedPoints && hasInputGradients) {
+        long long elements = static_cast<long long>(numel) * channelsIn();
+        int channels = channelsIn();
+        const float* src = sortedAdjInput.data_;
+        auto dst = adjInput.accessor<kernel::Tensor2RW<float>>();
+        void* args[] = {&elements, &channels, &src, &pointOrder, &dst};
+        pointOrder_.scatterAddRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0,
+                                                  stream, args);
     }
 
     if (!hasNetworkGradients) return;
