@@ -283,7 +283,15 @@ bool EncodingHashGrid::gradientSlices(GradientSliceLayout& layout) const
     if (dimension_ > 4 || numParameters_ >= (1 << 30)) return false;   // up to 8 records per point and level in registers
     const int lds = FusedNetwork::MaxSharedMemoryBytes();
     // the slice kernel sums in 64-bit fixed point: 8 bytes of LDS per element
-    const int entries = std::min(16384, lds / 8) / numFeaturesPerLevel_;
+    // Slices of 8192 sums (64 KiB, two workgroups of the slice kernel per compute unit: one streams records while the
+    // other zeroes or writes back; a train step of a 16-level hash grid 0.557 -> 0.533 ms) where no level then has
+    // more than 512 of them, else of 16384.
+    int largestLevel = 0;
+    for (int l = 0; l < numLevels_; ++l)
+        largestLevel = std::max(largestLevel, (l + 1 < numLevels_ ? layers_[l + 1].memoryOffset : numParameters_) - layers_[l].memoryOffset);
+    const int smallSlice = 8192 / numFeaturesPerLevel_ * numFeaturesPerLevel_;
+    const int sliceSums = smallSlice > 0 && divUp(largestLevel, smallSlice) <= 512 ? 8192 : 16384;
+    const int entries = std::min(sliceSums, lds / 8) / numFeaturesPerLevel_;
     if (entries < 64) return false;
     layout = GradientSliceLayout{};
     layout.sliceFloats = entries * numFeaturesPerLevel_;

@@ -179,10 +179,10 @@ def test_temporary_memory_sizes():
     # From 2^14 points on the grid gradients are summed slice by slice: the adjoint of the encoded rows
     # (32 halves per point) joins the adjoint pre-activations, and behind everything else come the
     # bucket cursors and the records (4 words each; per level, slices x (1.25 x share + 2048) of them:
-    # the table of a level holds 8192 .. 1 048 576 floats, a slice 16 384).
+    # the table of a level holds 8192 .. 1 048 576 floats, a slice 8192).
     n = 1 << 18
     floats = [8192, 24334, 71874, 221184, 686000] + [1 << 20] * 11
-    slices_per_level = [-(-f // 16384) for f in floats]
+    slices_per_level = [-(-f // 8192) for f in floats]
     records = sum(s * (((5 * n * 4 // 4) // s + 2048) & ~3) for s in slices_per_level)
     cursors = -(-(sum(slices_per_level) + 1) * 4 // 256) * 256
     base = (per_adj + 2 * 32) * n + 512 * n_params * 4
