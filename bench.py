@@ -33,20 +33,29 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 # code: "kernels" is device_code_hash() at the time of the counter runs, and a workload whose
 # device code has changed since (or that has no counter run) reports traffic null.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2-inference": {"points": 1 << 20, "fetch": 105175.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
-                       "kernels": "8c8d5322b473cfff"},
+    "cfg2-inference": {"points": 1 << 20, "fetch": 105164.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
+                       "kernels": "c1b1148b11172c9a"},
 }
 
 
 def device_code_hash(net):
     """Hash of everything the fused forward kernel of `net` is compiled from: the generated
-    source and the device headers beside it."""
-    import glob
+    source and the device headers it includes, directly or through other headers."""
     import hashlib
-    h = hashlib.sha256(net.generated_source("forward").encode())
-    kernel_dir = os.path.join(ROOT, "quick-mlp_amd", "csrc", "kernels", "qmlp", "kernels")
-    for f in sorted(glob.glob(os.path.join(kernel_dir, "*.h"))):
-        h.update(open(f, "rb").read())
+    import re
+    source = net.generated_source("forward")
+    kernel_dir = os.path.join(ROOT, "quick-mlp_amd", "csrc", "kernels")
+    seen, todo = {}, [source]
+    while todo:
+        text = todo.pop()
+        for name in re.findall(r'#include\s*[<"]([^>"]+)[>"]', text):
+            path = os.path.join(kernel_dir, name)
+            if name not in seen and os.path.isfile(path):
+                seen[name] = open(path, "rb").read()
+                todo.append(seen[name].decode())
+    h = hashlib.sha256(source.encode())
+    for name in sorted(seen):
+        h.update(name.encode() + b"\0" + seen[name] + b"\0")
     return h.hexdigest()[:16]
 
 WORKLOADS = {
