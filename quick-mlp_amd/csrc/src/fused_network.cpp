@@ -1450,14 +1450,12 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     kernel::PointOrderKey key{};
     if (!pointOrderFor(numel, key)) return false;
     const int channels = input.size(1);
-    const int maxChannels = channels <= 4 ? 4 : channels <= 8 ? 8 : 16;
 
     auto& po = pointOrder_;
     if (!po.scatter.has_value() && noAlloc)
         throw std::runtime_error("The kernels that order the batch are not loaded yet, and loading allocates: run "
                                  "inference() once on a batch of the same size first");
     loadPointOrderKernels(false);
-    (void)maxChannels;
     constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 8 * BLOCK;   // as in point_order.h
     // words: slab totals and one histogram per chunk; then (unless the caller has room for them) sorted inputs and order
     const long long histogramWords = (divUp(numel, CHUNK) + 1ll) * SLABS;
