@@ -450,8 +450,12 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
         c.set_table(1, table)
     lo = np.array([0.0] + grid["bounding_box_min"], np.float32)
     sz = np.array([1.0] + grid["bounding_box_size"], np.float32)
-    for N in (3000, 70001):     # one round of every slice workgroup; many rounds and a ragged last tile
-        X = (lo + sz * rng.uniform(-0.05, 1.05, (N, n_in))).astype(np.float32)
+    # one round of every slice workgroup; many rounds and a ragged last tile; all points in one small
+    # region (the records of a level then fall into one or two buckets, which overflow: the rest is added
+    # to the gradient tensor by the records kernel itself)
+    for N, clustered in ((3000, False), (70001, False), (70001, True)):
+        u = rng.uniform(-0.05, 1.05, (N, n_in)) if not clustered else 0.37 + 2e-3 * rng.uniform(0, 1, (N, n_in))
+        X = (lo + sz * u).astype(np.float32)
         adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
         for flags in (FLAG_ENC, FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC):
             got = {mode: c.gpu_train(X, adj, flags) for mode, c in cases.items()}
