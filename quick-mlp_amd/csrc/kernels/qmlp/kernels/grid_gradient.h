@@ -9,23 +9,26 @@
 // (EncodingHashGrid::scatterTile, 4.5 requests per point and level) bounds a train step. Here
 // the backward kernel only stores the adjoint of the encoded rows. Then
 //   GridGradientRecordsKernel  walks over the points, one per lane, level by level: for every
-//       pair of corners that are neighbours in memory it forms a record (the two elements, their
-//       weights, the adjoint of the level's features), sorts the records of the workgroup by the
-//       slice of the gradient table they belong to (a slice is a run of up to 32 768 floats =
-//       128 KiB of LDS) in LDS, reserves room in the buckets of these slices with one atomic per
-//       slice and workgroup, and copies the sorted records there in runs: all loads and stores
-//       of this kernel are coalesced;
+//       pair of corners that are neighbours in memory it forms a record (the offsets of the two
+//       entries within their slice, their weights, the adjoint of the level's features), sorts the
+//       records of the workgroup by the slice of the gradient table they belong to (a slice is a
+//       run of 8192 or 16 384 floats, whose 64-bit sums take 64 or 128 KiB of LDS) in LDS, reserves
+//       room in the buckets of these slices with one atomic per slice and workgroup, and copies the
+//       sorted records there in runs: all stores of the records are coalesced. An upper entry that
+//       lies in another slice than the lower one is added to the gradient tensor right away. With
+//       INPUT_GRADIENTS the kernel also gathers the entries of all corners and adds the grid's
+//       share of the gradient with respect to the input (what EncodingHashGrid::adjoint computes,
+//       operation by operation);
 //   GridGradientSlicesKernel   runs one workgroup per work item (level, slice, part of the
 //       bucket): it streams through its records and adds weight * adjoint to the slice in LDS,
-//       then adds the slice to the gradient tensor with atomics, 16 neighbouring floats per
-//       request (a coarse level has few slices that receive all records of the level; their
-//       buckets are shared out over several work items).
+//       then adds the slice to the gradient tensor (with atomics only for a coarse level, whose
+//       few slices receive all records of the level and are shared out over several work items).
 // The sums in LDS are 64-bit fixed point, added with integer atomics: ds_add_f32 completes one
 // lane every three cycles on this hardware (0.32 lanes per clock and CU measured, whatever the
 // addresses), ds_add_u64 3.5 lanes per clock. The scale is a power of two chosen per launch from the
 // largest adjoint of the batch (which the records kernel finds on its way) and the number of
-// records, such that no sum can overflow: at least 40 bits remain below the largest
-// contribution, and the sums do not depend on the order of the additions. Batches whose
+// records, such that no sum can overflow: at least 37 bits remain below the largest possible
+// contribution at 2^24 records, and the sums do not depend on the order of the additions. Batches whose
 // adjoints are not finite take the float additions, so that NaN and infinity reach the gradients.
 // Two forms that were measured and dropped: a workgroup per slice that tests every point of
 // the batch against its slice and recomputes the hits (the work of a hit falls to one lane of
