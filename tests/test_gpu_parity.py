@@ -681,6 +681,21 @@ def test_full_size_properties_cfg3_train():
     ref0 = case.oracle.backward(X[sample], adj[sample], FLAG_INPUT, round_mode=0)
     assert_close(a["adj_x"][sample] / s, ref0["adj_x"] / s, "sampled input gradients vs fp32", rel=REL, abs_=ABS,
                  allowed_fraction=2e-2)
+    # At this size the grid gradients are summed by slices and the input gradients come from the records
+    # kernel; the same network with the scatter inside the backward kernel (one atomic per contribution):
+    # outputs, input and weight gradients bit for bit, grid gradients up to the order of the fp32 additions.
+    cfg = json.loads(json.dumps(bc.CONFIGS[3]["cfg"]))
+    cfg.setdefault("options", {})["slice_gradients"] = 0
+    scatter = Case(cfg, bc.ORACLE_ACTIVATIONS)
+    scatter.set_parameters(case.params_np)
+    scatter.set_table(0, case.tables_np[0])
+    c = scatter.gpu_train(X, adj, flags)
+    assert np.array_equal(c["out"], a["out"])
+    assert np.array_equal(c["adj_x"], a["adj_x"])
+    assert np.array_equal(c["grads"], a["grads"])
+    tc = c["table_grads"][0]
+    assert_close(ta, tc, "grid gradients by slices against the atomic scatter", rel=1e-3, abs_=1e-5 * float(np.abs(tc).max()))
+    assert float(np.abs(tc).max()) > 0
 
 
 @pytest.mark.parametrize("cfg_id,N", [(4, 1 << 20), (5, 1 << 21)])
