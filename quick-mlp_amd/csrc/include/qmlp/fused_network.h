@@ -200,7 +200,11 @@ private:
     };
     // [adjoint flags][grid gradients by slices instead of atomics]
     std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2];
-    static constexpr int SLICE_GRADIENTS_MIN_BATCH = 1 << 14;
+    // Below this the two slice kernels cost more than the atomics they save (their work items zero and write
+    // back whole slices whatever the batch): a train step of a 16-level hash grid at 2^14 / 2^15 / 2^16 / 2^17
+    // points 0.18 / 0.24 / 0.37 / 0.63 ms with atomics, 0.28 / 0.28 / 0.29 / 0.34 ms by slices; a dense 4-D grid
+    // crosses over at the same size.
+    static constexpr int SLICE_GRADIENTS_MIN_BATCH = 1 << 16;
     /** True if some encoding of the network offers gradient slices (the adjoint memory then has room for the adjoint of the encoded rows). */
     bool hasSliceGradients() const;
     /** Bytes per point of adjoint memory for the adjoint of the encoded rows (read by the records kernels); 0 without them. */

@@ -172,11 +172,11 @@ def test_temporary_memory_sizes():
         assert net.adjoint_memory(n, 2) == per_adj * padded + slices * n_params * 4
         assert net.adjoint_memory(n, 3) == per_adj * padded + slices * n_params * 4
         assert net.adjoint_memory(n, 1) == 0
-        if n < (1 << 14):
+        if n < (1 << 16):
             # small batches scatter their grid gradients with atomics and need nothing for it
             assert net.adjoint_memory(n, 7) == per_adj * padded + slices * n_params * 4
             assert net.adjoint_memory(n, 5) == 0
-    # From 2^14 points on the grid gradients are summed slice by slice: the adjoint of the encoded rows
+    # From 2^16 points on the grid gradients are summed slice by slice: the adjoint of the encoded rows
     # (32 halves per point) joins the adjoint pre-activations, and behind everything else come the
     # bucket cursors and the records (4 words each; per level, slices x (1.25 x share + 2048) of them:
     # the table of a level holds 8192 .. 1 048 576 floats, a slice 8192).
