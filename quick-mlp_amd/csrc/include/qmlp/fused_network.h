@@ -185,7 +185,12 @@ private:
     {
         int encoding = -1;
         IEncoding::GradientSliceLayout layout;
-        CompiledKernel records;      // GridGradientRecordsKernel
+        // GridGradientRecordsKernel with layout.pointsPerWorkgroup >> i lanes per workgroup (down to 128), compiled
+        // when a batch first asks for it: a batch of fewer points than the largest workgroups of all compute units
+        // hold goes to smaller ones
+        std::vector<std::optional<CompiledKernel>> records;
+        std::string recordsSource;
+        int channelOffset = 0;
         CompiledKernel kernel;       // GridGradientSlicesKernel
         Tensor items;                // device copy of layout.items
     };
@@ -371,6 +376,9 @@ private:
     void checkEncodingParameters(Tensor::Usage usage) const;
     void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false);
     void compileBackwardKernel(int flags, bool sliceGradients = false, bool compileOnly = false);
+    /** The records kernel of a batch of numel points (compiled on first use; compileOnly: all of them into the cache). */
+    const CompiledKernel& recordsKernelFor(SliceGradientKernel& sk, int flags, int numel);
+    void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly);
 
     std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false) const;
     std::string backwardSource(int flags, int blockSize, bool sliceGradients = false) const;

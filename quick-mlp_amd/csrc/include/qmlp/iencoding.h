@@ -139,8 +139,10 @@ public:
         int sliceFloats = 0;               // floats of a full slice (= LDS of the slice kernel / 4)
         int recordWords = 0;               // 32-bit words of a record
         int pairs = 0;                     // records per point and level
-        int pointsPerWorkgroup = 0;        // lanes of a workgroup of the records kernel
-        int recordsLdsBytes = 0;           // its dynamic LDS
+        int pointsPerWorkgroup = 0;        // most lanes of a workgroup of the records kernel (a power of two)
+        /** Dynamic LDS of the records kernel with this many lanes: its records of one level with the slice of each
+         *  (16 bits), and per slice of the level (at most 512) room in the bucket, count and place among the records. */
+        int recordsLdsBytes(int points) const { return points * pairs * (recordWords * 4 + 2) + 512 * 8 + (2 * 512 + 1) * 4 + 64; }
         std::vector<int> slicesPerLevel;
         std::vector<GradientSlice> items;  // one workgroup of the slice kernel each
         /** Records a bucket of level l holds for a batch of numel points (as in the device code). */

@@ -304,8 +304,7 @@ bool EncodingHashGrid::gradientSlices(GradientSliceLayout& layout) const
     int points = 1024;
     while (points > 64 && points * layout.pairs * layout.recordWords * 4 > 96 * 1024) points /= 2;
     layout.pointsPerWorkgroup = points;
-    layout.recordsLdsBytes = points * layout.pairs * (layout.recordWords * 4 + 2) + 512 * 8 + (2 * 512 + 1) * 4 + 64;
-    if (layout.recordsLdsBytes > lds) return false;
+    if (layout.recordsLdsBytes(points) > lds) return false;
     // every level gets about this many work items: the bucket of a slice that holds more than its share is split
     constexpr int ITEMS_PER_LEVEL = 32;
     for (int l = 0; l < numLevels_; ++l) {

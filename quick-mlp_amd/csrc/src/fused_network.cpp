@@ -1185,23 +1185,22 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
             std::stringstream source;
             e->fillCode(source);
             source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient.h");
-            sk.records.blockSize = layout.pointsPerWorkgroup;
-            sk.records.sharedMemorySize = layout.recordsLdsBytes;
-            sk.records.fun = kl->getKernel(format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d, %s>", layout.configType.c_str(),
-                                                  layers_[0].channelsIn, offset, layout.sliceFloats, layout.pointsPerWorkgroup,
-                                                  (flags & GRADIENTS_INPUT) ? "true" : "false"),
-                                           source.str(), loaderFlags(compileOnly)).value();
+            sk.recordsSource = source.str();
+            sk.channelOffset = offset;
+            for (int points = layout.pointsPerWorkgroup; points >= std::min(128, layout.pointsPerWorkgroup); points /= 2)
+                sk.records.emplace_back();
+            if (compileOnly)
+                for (size_t v = 0; v < sk.records.size(); ++v) compileRecordsKernel(sk, flags, v, true);
             sk.kernel.blockSize = 1024;
             sk.kernel.sharedMemorySize = layout.sliceFloats * static_cast<int>(sizeof(long long));
             sk.kernel.fun = kl->getKernel(format("qmlp::kernel::GridGradientSlicesKernel<%s, %d>", layout.configType.c_str(), layout.sliceFloats),
                                           source.str(), loaderFlags(compileOnly)).value();
             if (!compileOnly) {
-                sk.records.fullGrid = sk.records.fun.fullGridSize(sk.records.blockSize, sk.records.sharedMemorySize);
                 static_assert(sizeof(IEncoding::GradientSlice) == 32, "eight 32-bit words, as in kernels/grid_gradient.h");
                 sk.items = Tensor(Tensor::FLOAT, {static_cast<int32_t>(layout.items.size() * 8)});
                 QMLP_HIP_CALL(qmlp_hip_memcpy_h2d(sk.items.rawPtr(), layout.items.data(), layout.items.size() * sizeof(layout.items[0]), nullptr));
-                logger->debug("gradient slices of encoding %d: %d buckets, %d work items, records kernel with %d points per workgroup (grid %d)",
-                              sk.encoding, layout.numBuckets(), static_cast<int>(layout.items.size()), layout.pointsPerWorkgroup, sk.records.fullGrid);
+                logger->debug("gradient slices of encoding %d: %d buckets, %d work items", sk.encoding, layout.numBuckets(),
+                              static_cast<int>(layout.items.size()));
             }
             ak.sliceGradients.push_back(std::move(sk));
         }
@@ -1231,6 +1230,37 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
         }
     }
     if (!compileOnly) backwardKernel_[flags][variant] = std::move(ak);
+}
+
+void FusedNetwork::compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly)
+{
+    const auto& layout = sk.layout;
+    const int points = layout.pointsPerWorkgroup >> variant;
+    CompiledKernel ck;
+    ck.blockSize = points;
+    ck.sharedMemorySize = layout.recordsLdsBytes(points);
+    ck.fun = QuickMLP::Instance().kernelLoader()->getKernel(
+        format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d, %s>", layout.configType.c_str(), layers_[0].channelsIn,
+               sk.channelOffset, layout.sliceFloats, points, (flags & GRADIENTS_INPUT) ? "true" : "false"),
+        sk.recordsSource, loaderFlags(compileOnly)).value();
+    if (compileOnly) return;
+    ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
+    QuickMLP::Instance().getLogger()->debug("records kernel of encoding %d with %d points per workgroup: %d VGPRs, full grid %d",
+                                            sk.encoding, points, ck.fun.numVgprs(), ck.fullGrid);
+    sk.records[variant] = std::move(ck);
+}
+
+const FusedNetwork::CompiledKernel& FusedNetwork::recordsKernelFor(SliceGradientKernel& sk, int flags, int numel)
+{
+    // The table entries that a workgroup gathers for the input gradients and the records it writes pass through
+    // one compute unit's memory pipeline: a batch that fills fewer workgroups than there are compute units leaves
+    // the rest of the chip idle. Measured on a 16-level hash grid (train step, ms; 1024 / 512 / 256 / 128 points):
+    // 2^17 points 0.414 / 0.302 / 0.319 / 0.371, 2^16 points 0.290 / 0.233 / 0.215 / 0.244.
+    const int computeUnits = KernelFunction::computeUnits();
+    size_t variant = 0;
+    while (variant + 1 < sk.records.size() && divUp(numel, sk.layout.pointsPerWorkgroup >> variant) < computeUnits) ++variant;
+    if (!sk.records[variant].has_value()) compileRecordsKernel(sk, flags, variant, false);
+    return sk.records[variant].value();
 }
 
 void FusedNetwork::precompile(int adjointFlags)
@@ -1429,7 +1459,12 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
         std::string error;
         (void)device_code::staticScratch(&scratch, &scratchBytes, error);
     }
-    if (adjointFlags > 0) compileBackwardKernel(adjointFlags, useSliceGradients(numel, adjointFlags));
+    if (adjointFlags > 0) {
+        const bool sliceGradients = useSliceGradients(numel, adjointFlags);
+        compileBackwardKernel(adjointFlags, sliceGradients);
+        for (auto& sk : backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value().sliceGradients)
+            (void)recordsKernelFor(sk, adjointFlags, numel);
+    }
 }
 
 bool FusedNetwork::sortsTraining(int numel) const
@@ -1743,7 +1778,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         offset += roundUp(transposedHalves * sizeof(half), size_t(16));
         char* workspace = static_cast<char*>(tmpMemoryAdjoint) + roundUp(offset, size_t(256));
         auto inputAcc = sortedInput;
-        for (const auto& sk : ak.sliceGradients) {
+        for (auto& sk : ak.sliceGradients) {
             const auto& layout = sk.layout;
             int* cursors = reinterpret_cast<int*>(workspace);
             const size_t cursorBytes = roundUp(static_cast<size_t>(layout.numBuckets() + 1) * sizeof(int), size_t(256));
@@ -1758,8 +1793,8 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
                 // the records kernel walks over the real points, but lays its buckets out for the padded batch
                 auto adjInputAcc = sortedAdjInput;   // this grid's share of dL/dinput (zeros in it if none is asked for: unused)
                 void* args[] = {&numel, &numelPadded, &inputAcc, &adjEncoded, params.data(), &records, &cursors, &adjInputAcc};
-                sk.records.fun.launch(std::min(divUp(numel, sk.records.blockSize), sk.records.fullGrid), sk.records.blockSize,
-                                      sk.records.sharedMemorySize, stream, args);
+                const CompiledKernel& rk = recordsKernelFor(sk, adjointFlags, numel);
+                rk.fun.launch(std::min(divUp(numel, rk.blockSize), rk.fullGrid), rk.blockSize, rk.sharedMemorySize, stream, args);
             }
             const uint32_t* recordsRead = records;
             const int* cursorsRead = cursors;

@@ -452,8 +452,11 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
     sz = np.array([1.0] + grid["bounding_box_size"], np.float32)
     # one round of every slice workgroup; many rounds and a ragged last tile; all points in one small
     # region (the records of a level then fall into one or two buckets, which overflow: the rest is added
-    # to the gradient tensor by the records kernel itself)
-    for N, clustered in ((3000, False), (70001, False), (70001, True)):
+    # to the gradient tensor by the records kernel itself). The records kernel runs with fewer points per
+    # workgroup for batches that would not give every compute unit a workgroup of the largest size: of the sizes
+    # 1024 / 512 / 256 / 128 these batches take the last, the third and (140001 points) the second.
+    sizes = [(3000, False), (70001, False), (70001, True)] + ([(140001, False)] if d == 3 else [])
+    for N, clustered in sizes:
         u = rng.uniform(-0.05, 1.05, (N, n_in)) if not clustered else 0.37 + 2e-3 * rng.uniform(0, 1, (N, n_in))
         X = (lo + sz * u).astype(np.float32)
         adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
