@@ -74,8 +74,14 @@ public:
 
         // Parameter gradients of grid encodings: summed slice by slice in LDS by a kernel of its own
         // (kernels/grid_gradient.h) instead of scattered with float atomics by the backward kernel.
-        // <0 (default): for batches of 16 384 points or more; 0: never; >0: always.
+        // <0 (default): for batches of SLICE_GRADIENTS_MIN_BATCH points or more; 0: never; >0: always.
         int sliceGradients = -1;
+
+        // Gradients of the layer weights: summed inside the backward kernel, which holds the adjoint
+        // pre-activations in registers (Layer::weightGradient), instead of by one kernel per layer that reads
+        // them back from memory. <0 (default): the layers with the fewest gradient tiles, up to 16 tiles (64
+        // registers of a wavefront), in networks whose weights all stay in LDS; 0: never; >0: up to 32 tiles.
+        int fusedWeightUpdate = -1;
 
         // Accepted for compatibility; the LDS layouts of this implementation are
         // bank-conflict free for 64 lanes by construction and need no skew.
@@ -202,6 +208,8 @@ private:
         CompiledKernel reduce;
         CompiledKernel transpose;
         int perEntryAdjointMemoryBytes = 0;
+        std::vector<bool> fusedLayers;    // layers whose weight gradients the adjoint kernel sums (no kernel in 'layers')
+        bool fusedWeightUpdate = false;   // any of them
     };
     // [adjoint flags][grid gradients by slices instead of atomics]
     std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2];
@@ -389,6 +397,12 @@ private:
     int weightUpdateBlockSize() const;
     // number of batch slices whose partial weight gradients are kept in the adjoint memory
     int weightUpdateSlices(int numTiles) const;
+    /** Layers whose weight gradients the backward kernel sums itself (options.fused_weight_update). */
+    std::vector<bool> fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients) const;
+    /** LDS halves per wavefront of the backward kernel for the tile that Layer::weightGradient transposes. */
+    int fusedWeightUpdateTransposeHalves() const;
+    /** Channels of adjoint pre-activations that the backward kernel stores per point for the weight-update kernels. */
+    int storedAdjointChannels(int adjointFlags, bool sliceGradients) const;
     // Where a kernel finds the weights of a layer. RESIDENT: in LDS for the whole kernel.
     // STREAMED: staged into a shared LDS buffer by the whole workgroup right before the layer
     // runs, for every group of tiles (networks whose weights exceed the LDS). GLOBAL: gathered

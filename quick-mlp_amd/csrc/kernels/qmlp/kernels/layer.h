@@ -30,6 +30,20 @@ __device__ __forceinline__ f32x4 mfma32(f16x8 a, f16x8 b, f32x4 c)
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+template <int A>
+__device__ __forceinline__ void zeroTiles(f32x4 (&acc)[A])
+{
+#pragma unroll
+    for (int a = 0; a < A; ++a) acc[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+template <int A, int B>
+__device__ __forceinline__ void zeroTiles(f32x4 (&acc)[A][B])
+{
+#pragma unroll
+    for (int a = 0; a < A; ++a) zeroTiles(acc[a]);
+}
+
 /**
  * \tparam CIN padded input channels (multiple of 16)
  * \tparam COUT padded output channels (multiple of 16)
@@ -222,10 +236,11 @@ struct Layer
      *           out: adjoint of the pre-activation, zeroed for points outside the batch
      * \param dx adjoint of the layer input (only written if COMPUTE_DX)
      * \param preTile pre-activations stored by forward<true>
-     * \param dpreTile [STORE_DPRE] receives the pre-activation adjoints, same layout
+     * \param dpreTile [STORE_DPRE] receives the pre-activation adjoints, same layout with DPRE_STRIDE halves
+     *        between the channels (T_STRIDE: the LDS tile that weightGradient reads)
      * \param validMask bit nt set iff point 4r+nt of this lane is inside the batch
      */
-    template <bool STORE_DPRE, bool COMPUTE_DX, bool GLOBAL_W = false, bool GUARDED = false>
+    template <bool STORE_DPRE, bool COMPUTE_DX, bool GLOBAL_W = false, bool GUARDED = false, int DPRE_STRIDE = TILE_POINTS>
     __device__ __forceinline__ static void adjoint(const f16* __restrict__ wT, f16x4 (&dy)[NT][MT],
                                                    f16x4 (&dx)[NT][KT], const f16* __restrict__ preTile,
                                                    f16* __restrict__ dpreTile, int validMask, int lane)
@@ -244,7 +259,7 @@ struct Layer
                     dy[nt][m][i] = d[nt];
                 }
                 if (STORE_DPRE && (!GUARDED || dpreTile != nullptr))
-                    *reinterpret_cast<f16x4*>(dpreTile + (16 * m + 4 * g + i) * TILE_POINTS + 4 * r) = d;
+                    *reinterpret_cast<f16x4*>(dpreTile + (16 * m + 4 * g + i) * DPRE_STRIDE + 4 * r) = d;
             }
         }
         if constexpr (COMPUTE_DX) {
@@ -265,6 +280,102 @@ struct Layer
                 }
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) dx[nt][mi] = toF16(acc[nt]);
+            }
+        }
+    }
+
+    // halves between the channel rows of the tile that weightGradient transposes in LDS: 64 points and 16 bytes,
+    // so that the sixteen rows a 16-byte operand read touches start in different banks
+    static constexpr int T_STRIDE = TILE_POINTS + 8;
+    static constexpr int T_HALVES = COUT * T_STRIDE;
+
+    /**
+     * Adds this tile's share to the gradients of the layer's weights and bias: dW (COUT x CIN) += dpre^T * in and
+     * db += dpre^T * 1 on the matrix cores, the 64 points of the tile as contraction index (two k-blocks of 32).
+     * The A operand needs 8 consecutive points of one channel per lane, the registers hold 4 channels of 4 points:
+     * adjoint<true, .., T_STRIDE> has written the adjoint pre-activations into rows of 64 points per channel in
+     * this wavefront's LDS tile. The B
+     * operand is read from the channel-major tile the forward kernel stored, the activation of the previous layer
+     * applied again (as WeightUpdateKernel does, which this replaces for networks whose gradient tiles fit into
+     * the registers of a wavefront; replaces network_weight_update_block.cuh:356-494 of the reference).
+     * \param sTile T_HALVES halves of LDS of this wavefront: the adjoint pre-activations (zero for points outside the batch)
+     * \param inTile (CIN, 64) halves: the stored input of the layer before InputActivation
+     */
+    template <typename InputActivation>
+    __device__ __forceinline__ static void weightGradient(const f16* sTile, const f16* __restrict__ inTile,
+                                                          f32x4 (&accW)[MT][KT], f32x4 (&accB)[MT], int lane)
+    {
+        const int g = lane >> 4, r = lane & 15;
+        waveLdsSync();
+        const f16x8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
+#pragma unroll
+        for (int kb = 0; kb < TILE_POINTS / 32; ++kb) {
+            f16x8 b[KT];
+#pragma unroll
+            for (int k = 0; k < KT; ++k) {
+                const int channel = 16 * k + r;
+                const f16x8 raw = *reinterpret_cast<const f16x8*>(inTile + channel * TILE_POINTS + 32 * kb + 8 * g);
+                b[k] = activationForwardChannel<InputActivation>(raw, channel);
+            }
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const f16x8 a = *reinterpret_cast<const f16x8*>(sTile + (16 * m + r) * T_STRIDE + 32 * kb + 8 * g);
+#pragma unroll
+                for (int k = 0; k < KT; ++k) accW[m][k] = mfma32(a, b[k], accW[m][k]);
+                if constexpr (BIAS) accB[m] = mfma32(a, ones, accB[m]);
+            }
+        }
+        waveLdsSync();   // the next layer writes its rows over these
+    }
+
+    /**
+     * After the last tile: the gradient tiles of the wavefronts of a workgroup are added up in LDS, one wavefront
+     * after the other (so that the sum rounds the same way in every run), and stored as this workgroup's partial sums,
+     * (COUT, CIN) row-major and COUT bias sums, into slice blockIdx.x of numSlices slices that lie sliceStride floats
+     * apart; the slices beyond the grid are zeroed, each by one workgroup. All threads of the workgroup call this;
+     * sAcc: (MT * KT + MT) * 256 floats.
+     */
+    template <int WAVES>
+    __device__ __forceinline__ static void storeWeightGradient(const f32x4 (&accW)[MT][KT], const f32x4 (&accB)[MT], float* sAcc,
+                                                               float* __restrict__ partialWeights, float* __restrict__ partialBias,
+                                                               int numSlices, int sliceStride, int wave, int lane)
+    {
+        const int g = lane >> 4, r = lane & 15;
+        constexpr int TILES = MT * KT + (BIAS ? MT : 0);
+        __syncthreads();   // whatever used this LDS before is done
+        for (int i = threadIdx.x; i < TILES * 256; i += blockDim.x) sAcc[i] = 0.f;
+        __syncthreads();
+        for (int w = 0; w < WAVES; ++w) {
+            if (wave == w) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+#pragma unroll
+                    for (int k = 0; k < KT; ++k)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sAcc[(m * KT + k) * 256 + (4 * g + i) * 16 + r] += accW[m][k][i];
+                    if constexpr (BIAS) {
+                        if (r == 0) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) sAcc[(MT * KT + m) * 256 + 4 * g + i] += accB[m][i];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        for (int e = threadIdx.x; e < MT * KT * 256; e += blockDim.x) {
+            const int t = e >> 8, within = e & 255;
+            const int m = t / KT, k = t - m * KT;
+            partialWeights[(16 * m + (within >> 4)) * CIN + 16 * k + (within & 15)] = sAcc[e];
+        }
+        if constexpr (BIAS) {
+            for (int e = threadIdx.x; e < COUT; e += blockDim.x) partialBias[e] = sAcc[(MT * KT + (e >> 4)) * 256 + (e & 15)];
+        }
+        for (int slice = blockIdx.x + gridDim.x; slice < numSlices; slice += gridDim.x) {
+            const long long offset = static_cast<long long>(slice - static_cast<int>(blockIdx.x)) * sliceStride;
+            for (int e = threadIdx.x; e < COUT * CIN; e += blockDim.x) partialWeights[offset + e] = 0.f;
+            if constexpr (BIAS) {
+                for (int e = threadIdx.x; e < COUT; e += blockDim.x) partialBias[offset + e] = 0.f;
             }
         }
     }

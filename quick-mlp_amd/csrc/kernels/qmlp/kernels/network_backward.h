@@ -5,7 +5,10 @@
 // of the matrix cores, each layer (last to first) applies the activation adjoint on
 // the stored pre-activations and contracts with the transposed weights
 // (dX = W^T dpre, the same MFMA path as the forward pass with the weight tiles
-// staged transposed), optionally storing dpre for the weight update. The adjoint of
+// staged transposed). For the weight gradients dpre is either stored for the weight-update
+// kernels or, where the gradient tiles of all layers fit into the registers of a wavefront,
+// contracted with the layer input right here (Layer::weightGradient), the workgroup storing
+// its partial sums after its last tile. The adjoint of
 // the encoded input finally goes through the LDS staging rows to one lane per point,
 // which accumulates input gradients and scatter-adds grid gradients with hardware
 // fp32 atomics.
@@ -25,6 +28,11 @@ QUICKMLP_KERNEL_NAMESPACE_BEGIN
 namespace activations
 {
 $$DEFINE_ACTIVATIONS$$
+    // stands for "no activation": the stored input of the first layer is its input
+    struct passthrough_
+    {
+        static __device__ __forceinline__ half forward(half x) { return x; }
+    };
 }
 
 /**
@@ -55,7 +63,9 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     const half* __restrict__ networkParametersH,
     const half* __restrict__ forwardTmpMemoryH,  //written by the forward kernel
     half* __restrict__ adjointTmpMemoryH,        //receives dpre if weight gradients are requested
-    const half* __restrict__ transposedWeightsH  //W^T of the layers whose weights do not stay in LDS, or nullptr
+    const half* __restrict__ transposedWeightsH, //W^T of the layers whose weights do not stay in LDS, or nullptr
+    float* __restrict__ partialGradients,        //FUSED_WEIGHT_UPDATE: partialSlices x the layout of the parameters; workgroup b
+    int partialSlices                            //stores the sums of its tiles into slice b (and zeroes slices b + k * gridDim.x)
     $$ENCODING_PARAMETERS$$)
 {
     constexpr int NUM_INPUTS = $$NUM_INPUTS$$;
@@ -82,6 +92,12 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     constexpr int OFFSET_ENCODED_ADJOINT = $$OFFSET_ENCODED_ADJOINT$$;   // channels in front of that region
     // false: nothing in this kernel reads the adjoint of an encoded row point by point
     constexpr bool NEEDS_STAGED_ADJOINT = $$NEEDS_STAGED_ADJOINT$$;
+    // true: the weight gradients are summed in this kernel and dpre is not stored
+    constexpr bool FUSED_WEIGHT_UPDATE = $$FUSED_WEIGHT_UPDATE$$;
+    constexpr bool STORE_DPRE = HAS_NETWORK_GRADIENTS;   // of the layers that have a weight-update kernel
+    (void)FUSED_WEIGHT_UPDATE;
+    constexpr int NUM_PARAMETERS = $$NUM_PARAMETERS$$;
+    (void)STORE_DPRE; (void)NUM_PARAMETERS;
     (void)ENCODED_CHANNELS; (void)NUM_INPUTS; (void)KT0; (void)STAGE_STRIDE;
 
     const f16* __restrict__ networkParameters = reinterpret_cast<const f16*>(networkParametersH);
@@ -97,9 +113,14 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     const int g = lane >> 4, r = lane & 15;
     f16* sStage = sParams + LDS_PARAM_HALVES + wave * (TILE_POINTS * STAGE_STRIDE);
     (void)sStage;
+    // FUSED_WEIGHT_UPDATE: this wavefront's tile of adjoint pre-activations, a row of 64 points per channel
+    f16* sTranspose = reinterpret_cast<f16*>(sMemory + $$OFFSET_TRANSPOSE$$) + wave * $$TRANSPOSE_HALVES$$;
+    (void)sTranspose;
 
     // stage the transposed weights in operand order
 $$STAGE_PARAMETERS$$
+    // FUSED_WEIGHT_UPDATE: the gradient tiles of this wavefront, summed over its tiles of the batch
+$$DECLARE_WEIGHT_GRADIENTS$$
     // gradients of coarse grid levels are summed in LDS first (zeroed here, added to the
     // gradient tensor once per workgroup after the loop over the tiles)
 $$ZERO_LDS_GRADIENTS$$
@@ -233,6 +254,7 @@ $$CALL_ENCODING_SCATTER$$
         }
     }
 $$FLUSH_LDS_GRADIENTS$$
+$$STORE_WEIGHT_GRADIENTS$$
 }
 
 QUICKMLP_KERNEL_NAMESPACE_END

@@ -78,6 +78,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         compileOptions_.sortTraining = options.value("sort_training", compileOptions_.sortTraining);
         compileOptions_.directInput = options.value("direct_input", compileOptions_.directInput);
         compileOptions_.sliceGradients = options.value("slice_gradients", compileOptions_.sliceGradients);
+        compileOptions_.fusedWeightUpdate = options.value("fused_weight_update", compileOptions_.fusedWeightUpdate);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
             options.value("parallel_weight_update", compileOptions_.parallelWeightUpdate);
@@ -591,10 +592,73 @@ int FusedNetwork::weightUpdateBlockSize() const
     return blockSize;
 }
 
+static bool offersSlices(const IEncoding& e, IEncoding::GradientSliceLayout* layout = nullptr)
+{
+    IEncoding::GradientSliceLayout local;
+    return e.hasParameters() && e.gradientSlices(layout ? *layout : local);
+}
+
 int FusedNetwork::weightUpdateSlices(int numTiles) const
 {
     const int waves = weightUpdateBlockSize() / WARP_SIZE;
     return std::max(1, std::min(divUp(numTiles, waves), MAX_WEIGHT_UPDATE_SLICES));
+}
+
+std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients) const
+{
+    std::vector<bool> fused(layers_.size(), false);
+    if (compileOptions_.fusedWeightUpdate == 0 || !(adjointFlags & GRADIENTS_NETWORK_WEIGHTS)) return fused;
+    // a backward kernel that gathers from or scatters into the tables of an encoding itself has no registers to spare
+    // (32 -> 64 -> 64 -> 16 behind a hash grid: 320 bytes of scratch per lane without any gradient tile)
+    for (const auto& e : encodings_) {
+        if (!e->hasParameters() || !(adjointFlags & (GRADIENTS_INPUT | GRADIENTS_INPUT_ENCODINGS))) continue;
+        if (!(sliceGradients && (adjointFlags & GRADIENTS_INPUT_ENCODINGS) && offersSlices(*e))) return fused;
+    }
+    for (int p : weightPlacement(true))
+        if (p != WEIGHTS_RESIDENT) return fused;
+    // a workgroup of 8 wavefronts leaves 128 registers to each: none to spare
+    const int blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
+    if (blockSize != DEFAULT_BLOCK_SIZE) return fused;
+    // room for the transposed tiles beside the weights and staging rows (32 KiB are kept for the gradients of a coarse grid level)
+    const int lds = ldsParamHalves(true) * static_cast<int>(sizeof(half))
+        + (blockSize / WARP_SIZE) * (stageBytesPerWave(true) + fusedWeightUpdateTransposeHalves() * static_cast<int>(sizeof(half)));
+    if (lds + 32 * 1024 > MaxSharedMemoryBytes()) return fused;
+    // Four accumulator registers per gradient tile and lane, for as long as the kernel runs: the layers with the
+    // fewest tiles first, up to 16 tiles (all 28 tiles of a 32 -> 64 -> 64 -> 16 network: 1 KB of scratch per lane
+    // and a backward kernel of 116 instead of 31 us; the weight-update kernels it replaced took 62 us).
+    const int budget = compileOptions_.fusedWeightUpdate > 0 ? 32 : 16;
+    std::vector<std::pair<int, int>> byTiles;
+    for (size_t i = 0; i < layers_.size(); ++i) {
+        const int mt = layers_[i].channelsOut / MATRIX_SIZE, kt = layers_[i].channelsIn / MATRIX_SIZE;
+        byTiles.push_back({mt * kt + (layers_[i].useBias ? mt : 0), static_cast<int>(i)});
+    }
+    std::sort(byTiles.begin(), byTiles.end());
+    int tiles = 0;
+    for (const auto& [count, layer] : byTiles) {
+        if (tiles + count > budget) break;
+        tiles += count;
+        fused[layer] = true;
+    }
+    return fused;
+}
+
+int FusedNetwork::fusedWeightUpdateTransposeHalves() const
+{
+    int widest = 0;
+    for (const auto& l : layers_) widest = std::max(widest, l.channelsOut);
+    return widest * (TILE_POINTS + 8);   // Layer::T_HALVES
+}
+
+int FusedNetwork::storedAdjointChannels(int adjointFlags, bool sliceGradients) const
+{
+    if (!(adjointFlags & GRADIENTS_NETWORK_WEIGHTS)) return 0;
+    // (the regions of the layers keep their places while any of them is stored)
+    bool allFused = true;
+    for (bool f : fusedWeightUpdateLayers(adjointFlags, sliceGradients)) allFused = allFused && f;
+    if (allFused) return 0;
+    int channels = 0;
+    for (const auto& l : layers_) channels += l.channelsOut;
+    return channels;
 }
 
 static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
@@ -687,12 +751,6 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool r
     callLayers << "        auto& xOut = x" << layers_.size() << ";\n";
     replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
     return code;
-}
-
-static bool offersSlices(const IEncoding& e, IEncoding::GradientSliceLayout* layout = nullptr)
-{
-    IEncoding::GradientSliceLayout local;
-    return e.hasParameters() && e.gradientSlices(layout ? *layout : local);
 }
 
 bool FusedNetwork::hasSliceGradients() const
@@ -790,13 +848,17 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
 
     std::vector<long long> transposed;
     transposedWeightLayout(flags, transposed);
-    std::stringstream callLayers;
+    std::stringstream callLayers, declareGradients, storeGradients;
+    const std::vector<bool> fusedLayers = fusedWeightUpdateLayers(flags, sliceGradients);
+    bool anyFused = false;
+    for (bool f : fusedLayers) anyFused = anyFused || f;
     const int L = static_cast<int>(layers_.size());
     bool anyStreamed = false;
     for (int i = L - 1; i >= 0; --i) {
         const auto& l = layers_[i];
         const std::string dy = (i == L - 1) ? std::string("dyOut") : "dx" + std::to_string(i + 1);
         const bool needsWeights = i > 0 || needsEncodingAdjoint;
+        const bool fused = fusedLayers[i];
         callLayers << "        f16x4 dx" << i << "[NT][Layer" << i << "::KT];\n";
         std::string weights = "sParams + " + std::to_string(ldsW[i]);
         if (placement[i] == WEIGHTS_GLOBAL)
@@ -807,14 +869,38 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
                        << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + " << ldsW[i]
                        << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
         }
-        callLayers << "        Layer" << i << "::template adjoint<HAS_NETWORK_GRADIENTS, "
+        callLayers << "        Layer" << i << "::template adjoint<" << (fused ? "true" : "STORE_DPRE") << ", "
                    << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (placement[i] == WEIGHTS_GLOBAL ? ", true" : ", false")
-                   << ", HAS_STREAMED_LAYERS>(" << weights << ", " << dy
+                   << ", HAS_STREAMED_LAYERS" << (fused ? ", Layer" + std::to_string(i) + "::T_STRIDE" : std::string()) << ">(" << weights << ", " << dy
                    << ", dx" << i << ",\n            forwardTmpMemory + (" << backwardInfo_[i].offsetPre
                    << "ll * numel64 + static_cast<long long>(tileRead) * (" << l.channelsOut << " * TILE_POINTS)),\n"
-                   << "            (HAS_NETWORK_GRADIENTS && tileValid) ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut
-                   << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut
-                   << " * TILE_POINTS)) : nullptr,\n            validMask, lane);\n";
+                   << "            ";
+        if (fused) callLayers << "sTranspose";
+        else callLayers << "(STORE_DPRE && tileValid) ? adjointTmpMemory + (" << backwardInfo_[i].offsetAdjOut
+                        << "ll * numel64 + static_cast<long long>(tile) * (" << l.channelsOut << " * TILE_POINTS)) : nullptr";
+        callLayers << ",\n            validMask, lane);\n";
+        if (fused) {
+            // the LDS tile now holds the adjoint of the pre-activations, zero outside the batch
+            const std::string inputActivation = i > 0 ? "activations::" + activationTypeName(i - 1) : std::string("activations::passthrough_");
+            callLayers << "        Layer" << i << "::template weightGradient<" << inputActivation << ">(sTranspose,\n"
+                       << "            forwardTmpMemory + (" << backwardInfo_[i].offsetIn << "ll * numel64 + static_cast<long long>(tileRead) * ("
+                       << l.channelsIn << " * TILE_POINTS)), accW" << i << ", accB" << i << ", lane);\n";
+            declareGradients << "    f32x4 accW" << i << "[Layer" << i << "::MT][Layer" << i << "::KT], accB" << i << "[Layer" << i << "::MT];\n"
+                             << "    zeroTiles(accW" << i << ");\n    zeroTiles(accB" << i << ");\n";
+            storeGradients << "    Layer" << i << "::template storeWeightGradient<WAVES>(accW" << i << ", accB" << i
+                           << ", reinterpret_cast<float*>(sMemory),\n        partialGradients + (static_cast<long long>(blockIdx.x) * NUM_PARAMETERS + "
+                           << l.weightsStart << "), partialGradients + (static_cast<long long>(blockIdx.x) * NUM_PARAMETERS + "
+                           << (l.useBias ? l.biasStart : 0) << "), partialSlices, NUM_PARAMETERS, wave, lane);\n";
+        }
+    }
+    replaceAll(code, "$$FUSED_WEIGHT_UPDATE$$", anyFused ? "true" : "false");
+    replaceAll(code, "$$NUM_PARAMETERS$$", std::to_string(numParameters_));
+    replaceAll(code, "$$DECLARE_WEIGHT_GRADIENTS$$", declareGradients.str());
+    replaceAll(code, "$$STORE_WEIGHT_GRADIENTS$$", storeGradients.str());
+    {
+        std::vector<LdsGradients> unused;
+        replaceAll(code, "$$OFFSET_TRANSPOSE$$", std::to_string(roundUp(ldsGradientLayout(flags, blockSize, unused, sliceGradients), 16)));
+        replaceAll(code, "$$TRANSPOSE_HALVES$$", std::to_string(anyFused ? fusedWeightUpdateTransposeHalves() : 0));
     }
     callLayers << "        auto& dxIn = dx0;\n        (void)dxIn;\n";
     replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
@@ -870,10 +956,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
     replaceAll(code, "$$STORE_ENCODED_ADJOINT$$", storeEncodedAdjoint ? "true" : "false");
     {
-        int adjointChannels = 0;
-        if (hasNetworkGradients)
-            for (const auto& l : layers_) adjointChannels += l.channelsOut;
-        replaceAll(code, "$$OFFSET_ENCODED_ADJOINT$$", std::to_string(adjointChannels));
+        replaceAll(code, "$$OFFSET_ENCODED_ADJOINT$$", std::to_string(storedAdjointChannels(flags, sliceGradients)));
     }
     // the adjoint of the encoded rows goes through the staging rows only if a lane per point still needs it
     replaceAll(code, "$$NEEDS_STAGED_ADJOINT$$", (inputGradientsInKernel || gradientsInKernel) ? "true" : "false");
@@ -1150,6 +1233,22 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
         std::vector<LdsGradients> ldsGradients;
         ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients, sliceGradients);
     }
+    ak.fusedLayers = fusedWeightUpdateLayers(flags, sliceGradients);
+    ak.fusedWeightUpdate = false;
+    for (bool f : ak.fusedLayers) ak.fusedWeightUpdate = ak.fusedWeightUpdate || f;
+    if (ak.fusedWeightUpdate) {
+        // behind everything else: a tile per wavefront for Layer::weightGradient; after the last tile the gradient
+        // tiles of one layer at a time are summed over the wavefronts from the start of the LDS
+        int widestTiles = 0;
+        for (size_t i = 0; i < layers_.size(); ++i) {
+            const auto& l = layers_[i];
+            const int mt = l.channelsOut / MATRIX_SIZE, kt = l.channelsIn / MATRIX_SIZE;
+            if (ak.fusedLayers[i]) widestTiles = std::max(widestTiles, mt * kt + (l.useBias ? mt : 0));
+        }
+        ak.adjoint.sharedMemorySize = std::max(roundUp(ak.adjoint.sharedMemorySize, 16) + (ak.adjoint.blockSize / WARP_SIZE)
+                                                   * fusedWeightUpdateTransposeHalves() * static_cast<int>(sizeof(half)),
+                                               widestTiles * 256 * static_cast<int>(sizeof(float)));
+    }
     const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients);
     ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
     {
@@ -1166,9 +1265,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
                       ak.adjoint.blockSize, ak.adjoint.sharedMemorySize, ak.adjoint.fun.numVgprs(),
                       ak.adjoint.fun.scratchBytes(), ak.adjoint.fullGrid);
     }
-    int adjointChannels = 0;
-    for (const auto& l : layers_) adjointChannels += l.channelsOut;
-    ak.perEntryAdjointMemoryBytes = hasNetworkGradients ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
+    ak.perEntryAdjointMemoryBytes = storedAdjointChannels(flags, sliceGradients) * static_cast<int>(sizeof(half));
     // behind the adjoint pre-activations: the adjoint of the encoded rows for the records kernels
     if (sliceGradients && (flags & GRADIENTS_INPUT_ENCODINGS)) ak.perEntryAdjointMemoryBytes += sliceGradientBytesPerPoint();
 
@@ -1212,7 +1309,8 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
         ak.reduce.blockSize = 1024;
         ak.reduce.fun = kl->getKernel("qmlp::kernel::WeightUpdateReduceKernel", source, loaderFlags(compileOnly)).value();
         ak.layers.resize(layers_.size());
-        for (size_t layer = 0; layer < layers_.size(); ++layer) {
+        for (size_t layer = 0; layer < ak.layers.size(); ++layer) {
+            if (ak.fusedLayers[layer]) continue;   // summed by the adjoint kernel
             auto& wk = ak.layers[layer];
             int tiles = 0;
             const std::string name = weightUpdateKernelName(static_cast<int>(layer), wk.numChunks, tiles);
@@ -1608,11 +1706,9 @@ size_t FusedNetwork::adjointMemoryAsGiven(int numElements, AdjointModeFlags adjo
 {
     if (adjointFlags <= 0 || adjointFlags >= ADJOINT_MODE_MAX_COMBINATIONS)
         throw std::runtime_error("At least one derivative must be enabled");
-    int adjointChannels = 0;
-    for (const auto& l : layers_) adjointChannels += l.channelsOut;
-    int perEntry = (adjointFlags & GRADIENTS_NETWORK_WEIGHTS) ? adjointChannels * static_cast<int>(sizeof(half)) : 0;
     // batches that take the gradient slice kernels: the adjoint of the encoded rows, which the records kernels read
     const bool sliceGradients = useSliceGradients(numElements, adjointFlags);
+    int perEntry = storedAdjointChannels(adjointFlags, sliceGradients) * static_cast<int>(sizeof(half));
     if (sliceGradients) perEntry += sliceGradientBytesPerPoint();
     numElements = roundUp(numElements, WARP_SIZE);
     size_t bytes = static_cast<size_t>(perEntry) * static_cast<size_t>(numElements);
@@ -1753,25 +1849,28 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     {
         const auto& ck = ak.adjoint;
         const int waves = ck.blockSize / WARP_SIZE;
-        const int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+        int grid = std::min(divUp(numTiles, waves), ck.fullGrid);
+        // every workgroup stores its sums of the weight gradients as one of the slices of the batch that the
+        // reduction adds up (and zeroes its share of the slices beyond the grid)
+        int partialSlices = weightUpdateSlices(numTiles);
+        if (ak.fusedWeightUpdate) grid = std::min(grid, partialSlices);
         auto inputAcc = sortedInput;
         auto adjOutputAcc = sortedAdjOutput;
         auto adjInputAcc = sortedAdjInput;
         const half* networkParams = parametersInference_.dataPtr<half>();
         const half* forwardTmpMemory = static_cast<const half*>(tmpMemoryForward);
         half* adjointTmpMemory = static_cast<half*>(tmpMemoryAdjoint);
+        float* partialGradients = reinterpret_cast<float*>(static_cast<char*>(tmpMemoryAdjoint)
+                                                           + static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64));
         std::vector<void*> args = {&numel, &inputAcc, &adjOutputAcc, &adjInputAcc, &networkParams,
-                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights};
+                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights, &partialGradients, &partialSlices};
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
     }
     // parameter gradients of the grids, slice by slice, from the adjoint of the encoded rows the kernel above stored
     if (!ak.sliceGradients.empty()) {
-        int adjointChannels = 0;
-        if (hasNetworkGradients)
-            for (const auto& l : layers_) adjointChannels += l.channelsOut;
-        const half* adjEncoded = static_cast<const half*>(tmpMemoryAdjoint) + static_cast<ptrdiff_t>(adjointChannels) * numel64;
+        const half* adjEncoded = static_cast<const half*>(tmpMemoryAdjoint) + static_cast<ptrdiff_t>(storedAdjointChannels(adjointFlags, true)) * numel64;
         // the workspace is the last part of the adjoint memory: everything in front of it
         size_t offset = static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64);
         if (hasNetworkGradients) offset += static_cast<size_t>(weightUpdateSlices(numTiles)) * numParameters_ * sizeof(float);
@@ -1828,6 +1927,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     float* partial = reinterpret_cast<float*>(static_cast<char*>(tmpMemoryAdjoint)
                                               + static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64));
     for (size_t layer = 0; layer < layers_.size(); ++layer) {
+        if (ak.fusedLayers[layer]) continue;
         const auto& ls = layers_[layer];
         const auto& ali = backwardInfo_[layer];
         const auto& wk = ak.layers[layer];

@@ -127,6 +127,44 @@ def test_python_suite_shapes(widths, act, N):
     check_gradients(case, X, adj, FLAG_INPUT | FLAG_WEIGHTS, got)
 
 
+@pytest.mark.parametrize("widths,acts,N", [([32, 32, 16], ["relu", "celu", "identity"], 5000),
+                                          ([64, 64, 16], ["celu", "relu", "identity"], 20001),
+                                          ([64, 128, 16], ["relu", "celu", "identity"], 131073)])
+def test_weight_gradients_summed_in_the_backward_kernel_match_the_weight_update_kernels(widths, acts, N):
+    """options.fused_weight_update: 0 = one weight-update kernel per layer reads the adjoint pre-activations that the
+    backward kernel stored; -1 (default) = the backward kernel sums the gradient tiles of the layers with the fewest
+    tiles itself (Layer::weightGradient), up to 16 tiles; 1 = up to 32 tiles. Same products, another order of the
+    fp32 sums: all three against each other and, the smallest batch, against the oracles. The backward kernel of the
+    last network takes 108 KB of LDS: one workgroup per compute unit, fewer than the 512 batch slices of 131 073
+    points, so it also zeroes the slices beyond its grid."""
+    n_in = 16
+    rng = np.random.default_rng(len(widths))
+    X = rng.uniform(-1, 1, (N, n_in)).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, widths[-1])) / np.sqrt(N)).astype(np.float32)
+    params = None
+    got = {}
+    for mode in (0, -1, 1):
+        cfg = identity_cfg(n_in, widths, acts, [True] * (len(widths) - 1) + [False])
+        cfg["options"] = {"fused_weight_update": mode}
+        case = Case(cfg)
+        if params is None:
+            params = random_parameters(case.oracle, rng)
+        case.set_parameters(params)
+        src = case.net.generated_source("backward", FLAG_INPUT | FLAG_WEIGHTS)
+        assert ("::template weightGradient<" in src) == (mode != 0)
+        flags = FLAG_INPUT | FLAG_WEIGHTS
+        got[mode] = case.gpu_train(X, adj, flags)
+        # (the larger batches only mode against mode, which is the tighter comparison: with gradient entries of order
+        # one, sums over tens of thousands of points with ReLU units that an fp16 rounding switches leave the
+        # tolerances of the oracle comparison, for the weight-update kernels as for the fused sums)
+        if N <= 5000:
+            check_gradients(case, X, adj, flags, got[mode], kinks=True, what="fused_weight_update %d: " % mode)
+    scale = float(np.abs(got[0]["grads"]).max())
+    for mode in (-1, 1):
+        assert np.allclose(got[mode]["grads"] / scale, got[0]["grads"] / scale, rtol=1e-3, atol=1e-5), mode
+        assert np.array_equal(got[mode]["adj_x"], got[0]["adj_x"]) and np.array_equal(got[mode]["out"], got[0]["out"])
+
+
 def test_round_mode_oracle_is_tighter():
     """Against the oracle that rounds where the device rounds, the error shrinks by an order."""
     case = Case(identity_cfg(16, [64, 64, 4], ["relu", "celu", "identity"], [True, True, True]))
