@@ -292,6 +292,8 @@ struct Layer
     /**
      * Adds this tile's share to the gradients of the layer's weights and bias: dW (COUT x CIN) += dpre^T * in and
      * db += dpre^T * 1 on the matrix cores, the 64 points of the tile as contraction index (two k-blocks of 32).
+     * The bias sums of all output tiles share one accumulator tile: output tile m is multiplied with a B operand
+     * that is one in column m and zero elsewhere, so column m of the tile receives its 16 sums.
      * The A operand needs 8 consecutive points of one channel per lane, the registers hold 4 channels of 4 points:
      * adjoint<true, .., T_STRIDE> has written the adjoint pre-activations into rows of 64 points per channel in
      * this wavefront's LDS tile. The B
@@ -303,11 +305,14 @@ struct Layer
      */
     template <typename InputActivation>
     __device__ __forceinline__ static void weightGradient(const f16* sTile, const f16* __restrict__ inTile,
-                                                          f32x4 (&accW)[MT][KT], f32x4 (&accB)[MT], int lane)
+                                                          f32x4 (&accW)[MT][KT], f32x4& accB, int lane)
     {
+        static_assert(MT <= 16, "one column of the bias tile per output tile");
         const int g = lane >> 4, r = lane & 15;
+        __builtin_amdgcn_sched_barrier(0);
         waveLdsSync();
         const f16x8 ones = {1, 1, 1, 1, 1, 1, 1, 1};
+        const f16x8 zeros = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int kb = 0; kb < TILE_POINTS / 32; ++kb) {
             f16x8 b[KT];
@@ -322,10 +327,11 @@ struct Layer
                 const f16x8 a = *reinterpret_cast<const f16x8*>(sTile + (16 * m + r) * T_STRIDE + 32 * kb + 8 * g);
 #pragma unroll
                 for (int k = 0; k < KT; ++k) accW[m][k] = mfma32(a, b[k], accW[m][k]);
-                if constexpr (BIAS) accB[m] = mfma32(a, ones, accB[m]);
+                if constexpr (BIAS) accB = mfma32(a, r == m ? ones : zeros, accB);
             }
         }
         waveLdsSync();   // the next layer writes its rows over these
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     /**
@@ -333,31 +339,31 @@ struct Layer
      * after the other (so that the sum rounds the same way in every run), and stored as this workgroup's partial sums,
      * (COUT, CIN) row-major and COUT bias sums, into slice blockIdx.x of numSlices slices that lie sliceStride floats
      * apart; the slices beyond the grid are zeroed, each by one workgroup. All threads of the workgroup call this;
-     * sAcc: (MT * KT + MT) * 256 floats.
+     * sAcc: (MT * KT + 1) * 256 floats.
      */
     template <int WAVES>
-    __device__ __forceinline__ static void storeWeightGradient(const f32x4 (&accW)[MT][KT], const f32x4 (&accB)[MT], float* sAcc,
+    __device__ __forceinline__ static void storeWeightGradient(const f32x4 (&accW)[MT][KT], const f32x4& accB, float* sAcc,
                                                                float* __restrict__ partialWeights, float* __restrict__ partialBias,
                                                                int numSlices, int sliceStride, int wave, int lane)
     {
         const int g = lane >> 4, r = lane & 15;
-        constexpr int TILES = MT * KT + (BIAS ? MT : 0);
+        constexpr int TILES = MT * KT + (BIAS ? 1 : 0);
         __syncthreads();   // whatever used this LDS before is done
         for (int i = threadIdx.x; i < TILES * 256; i += blockDim.x) sAcc[i] = 0.f;
         __syncthreads();
         for (int w = 0; w < WAVES; ++w) {
             if (wave == w) {
 #pragma unroll
-                for (int m = 0; m < MT; ++m) {
+                for (int m = 0; m < MT; ++m)
 #pragma unroll
                     for (int k = 0; k < KT; ++k)
 #pragma unroll
                         for (int i = 0; i < 4; ++i) sAcc[(m * KT + k) * 256 + (4 * g + i) * 16 + r] += accW[m][k][i];
-                    if constexpr (BIAS) {
-                        if (r == 0) {
+                if constexpr (BIAS) {
+                    // column r of the bias tile: the sums of the channels 16r + 4g .. + 3
+                    if (r < MT) {
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) sAcc[(MT * KT + m) * 256 + 4 * g + i] += accB[m][i];
-                        }
+                        for (int i = 0; i < 4; ++i) sAcc[MT * KT * 256 + 16 * r + 4 * g + i] += accB[i];
                     }
                 }
             }
@@ -369,7 +375,7 @@ struct Layer
             partialWeights[(16 * m + (within >> 4)) * CIN + 16 * k + (within & 15)] = sAcc[e];
         }
         if constexpr (BIAS) {
-            for (int e = threadIdx.x; e < COUT; e += blockDim.x) partialBias[e] = sAcc[(MT * KT + (e >> 4)) * 256 + (e & 15)];
+            for (int e = threadIdx.x; e < COUT; e += blockDim.x) partialBias[e] = sAcc[MT * KT * 256 + e];
         }
         for (int slice = blockIdx.x + gridDim.x; slice < numSlices; slice += gridDim.x) {
             const long long offset = static_cast<long long>(slice - static_cast<int>(blockIdx.x)) * sliceStride;

@@ -616,9 +616,13 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
     }
     for (int p : weightPlacement(true))
         if (p != WEIGHTS_RESIDENT) return fused;
-    // a workgroup of 8 wavefronts leaves 128 registers to each: none to spare
+    // a workgroup of 8 wavefronts leaves 128 registers to each: none to spare; nor do layers of more than 64
+    // channels, whose activations fill 64 registers and more (16 -> 128 -> 64 -> 48 -> 16 with sine activations
+    // and workgroups of 4 wavefronts: a train step of 1.27 instead of 0.67 ms with two layers summed in the kernel)
     const int blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
     if (blockSize != DEFAULT_BLOCK_SIZE) return fused;
+    for (const auto& l : layers_)
+        if (std::max(l.channelsIn, l.channelsOut) > 64) return fused;
     // room for the transposed tiles beside the weights and staging rows (32 KiB are kept for the gradients of a coarse grid level)
     const int lds = ldsParamHalves(true) * static_cast<int>(sizeof(half))
         + (blockSize / WARP_SIZE) * (stageBytesPerWave(true) + fusedWeightUpdateTransposeHalves() * static_cast<int>(sizeof(half)));
@@ -630,7 +634,7 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
     std::vector<std::pair<int, int>> byTiles;
     for (size_t i = 0; i < layers_.size(); ++i) {
         const int mt = layers_[i].channelsOut / MATRIX_SIZE, kt = layers_[i].channelsIn / MATRIX_SIZE;
-        byTiles.push_back({mt * kt + (layers_[i].useBias ? mt : 0), static_cast<int>(i)});
+        byTiles.push_back({mt * kt + (layers_[i].useBias ? 1 : 0), static_cast<int>(i)});   // the bias sums share a tile
     }
     std::sort(byTiles.begin(), byTiles.end());
     int tiles = 0;
@@ -885,8 +889,8 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
             callLayers << "        Layer" << i << "::template weightGradient<" << inputActivation << ">(sTranspose,\n"
                        << "            forwardTmpMemory + (" << backwardInfo_[i].offsetIn << "ll * numel64 + static_cast<long long>(tileRead) * ("
                        << l.channelsIn << " * TILE_POINTS)), accW" << i << ", accB" << i << ", lane);\n";
-            declareGradients << "    f32x4 accW" << i << "[Layer" << i << "::MT][Layer" << i << "::KT], accB" << i << "[Layer" << i << "::MT];\n"
-                             << "    zeroTiles(accW" << i << ");\n    zeroTiles(accB" << i << ");\n";
+            declareGradients << "    f32x4 accW" << i << "[Layer" << i << "::MT][Layer" << i << "::KT], accB" << i << " = {0.f, 0.f, 0.f, 0.f};\n"
+                             << "    zeroTiles(accW" << i << ");\n";
             storeGradients << "    Layer" << i << "::template storeWeightGradient<WAVES>(accW" << i << ", accB" << i
                            << ", reinterpret_cast<float*>(sMemory),\n        partialGradients + (static_cast<long long>(blockIdx.x) * NUM_PARAMETERS + "
                            << l.weightsStart << "), partialGradients + (static_cast<long long>(blockIdx.x) * NUM_PARAMETERS + "
@@ -1243,7 +1247,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
         for (size_t i = 0; i < layers_.size(); ++i) {
             const auto& l = layers_[i];
             const int mt = l.channelsOut / MATRIX_SIZE, kt = l.channelsIn / MATRIX_SIZE;
-            if (ak.fusedLayers[i]) widestTiles = std::max(widestTiles, mt * kt + (l.useBias ? mt : 0));
+            if (ak.fusedLayers[i]) widestTiles = std::max(widestTiles, mt * kt + (l.useBias ? 1 : 0));
         }
         ak.adjoint.sharedMemorySize = std::max(roundUp(ak.adjoint.sharedMemorySize, 16) + (ak.adjoint.blockSize / WARP_SIZE)
                                                    * fusedWeightUpdateTransposeHalves() * static_cast<int>(sizeof(half)),

@@ -203,18 +203,19 @@ def test_temporary_memory_of_networks_whose_backward_kernel_sums_the_weight_grad
         return qmlp.Network(json.dumps(cfg))
     n = 4096
     slices = 4096 // 64 // 4
-    small = [32, 32, 16]            # gradient tiles with the bias tiles: 2 + 2, 4 + 2, 2 + 1 = 13
+    small = [32, 32, 16]            # gradient tiles, one more each for the bias sums: 2 + 1, 4 + 1, 2 + 1 = 11
     params = net(small, 0).num_network_parameters()
     assert net(small, 0).adjoint_memory(n, 3) == 2 * (32 + 32 + 16) * n + slices * params * 4
     assert net(small, -1).adjoint_memory(n, 3) == slices * params * 4
     assert "::template weightGradient<" not in net(small, 0).generated_source("backward", 3)
     assert net(small, -1).generated_source("backward", 3).count("::template weightGradient<") == 3
-    mixed = [64, 64, 16]            # 4 + 4, 16 + 4, 4 + 1: the middle layer keeps its weight-update kernel
+    mixed = [64, 64, 16]            # 4 + 1, 16 + 1, 4 + 1: the middle layer keeps its weight-update kernel
     params = net(mixed, 0).num_network_parameters()
     assert net(mixed, -1).adjoint_memory(n, 3) == 2 * (64 + 64 + 16) * n + slices * params * 4
     src = net(mixed, -1).generated_source("backward", 3)
     assert src.count("::template weightGradient<") == 2 and "Layer1::template weightGradient<" not in src
-    assert net(mixed, 1).generated_source("backward", 3).count("::template weightGradient<") == 2   # 13 + 20 tiles > 32
+    assert net(mixed, 1).generated_source("backward", 3).count("::template weightGradient<") == 3   # 27 tiles <= 32
+    assert net(mixed, 1).adjoint_memory(n, 3) == slices * params * 4
     # without weight gradients nothing changes
     assert "::template weightGradient<" not in net(small, -1).generated_source("backward", 1)
 
