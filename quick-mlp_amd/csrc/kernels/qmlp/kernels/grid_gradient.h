@@ -309,7 +309,7 @@ struct GridGradientRecords
             }
             if constexpr (INPUT_GRADIENTS && !DEFER_ENTRIES) {
                 // the entries of all corners, for this grid's share of dL/dinput (a dense 4-D grid with 8 features
-                // holds 64 registers: used at once; held until the end of the level 304 against 282 us)
+                // holds 64 registers: used at once; held until the end of the level 302 against 275 us)
                 loadHeld<LEVEL>(s, params, held);
                 positionGradient<LEVEL>(p, s, held, adjEncoded, adjPos);
             }
