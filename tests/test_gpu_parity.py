@@ -159,6 +159,13 @@ def test_weight_gradients_summed_in_the_backward_kernel_match_the_weight_update_
         # tolerances of the oracle comparison, for the weight-update kernels as for the fused sums)
         if N <= 5000:
             check_gradients(case, X, adj, flags, got[mode], kinks=True, what="fused_weight_update %d: " % mode)
+    # the layers that keep a weight-update kernel may run on streams of their own beside the caller's: same sums
+    cfg = identity_cfg(n_in, widths, acts, [True] * (len(widths) - 1) + [False])
+    cfg["options"] = {"fused_weight_update": -1, "parallel_weight_update": True}
+    case = Case(cfg)
+    case.set_parameters(params)
+    side_by_side = case.gpu_train(X, adj, FLAG_INPUT | FLAG_WEIGHTS)
+    assert np.array_equal(side_by_side["grads"], got[-1]["grads"])
     scale = float(np.abs(got[0]["grads"]).max())
     for mode in (-1, 1):
         assert np.allclose(got[mode]["grads"] / scale, got[0]["grads"] / scale, rtol=1e-3, atol=1e-5), mode
