@@ -48,28 +48,33 @@ __device__ __forceinline__ f16 fromHalf(half v) { return static_cast<__half_raw>
  */
 namespace fastmath
 {
+/** x * c in fp32 from the fp16 x. Written as a fused multiply-add with a zero addend (the same value, bit for
+ *  bit): the compiler then takes v_fma_mix_f32, which reads either half of a register as its fp16 operand, instead
+ *  of a conversion (and a shift for the upper half) followed by a multiply. */
+__device__ __forceinline__ float scaled(half x, float c)
+{
+    return __builtin_fmaf(__half2float(x), c, 0.0f);
+}
 struct Sin
 {
     __device__ __forceinline__ half operator()(half x) const
     {
         // v_sin_f32 takes revolutions and is defined on [-256, 256]
-        const float rev = __half2float(x) * 0.15915494309189535f;
-        return __float2half(__builtin_amdgcn_sinf(__builtin_amdgcn_fractf(rev)));
+        return __float2half(__builtin_amdgcn_sinf(__builtin_amdgcn_fractf(scaled(x, 0.15915494309189535f))));
     }
 };
 struct Cos
 {
     __device__ __forceinline__ half operator()(half x) const
     {
-        const float rev = __half2float(x) * 0.15915494309189535f;
-        return __float2half(__builtin_amdgcn_cosf(__builtin_amdgcn_fractf(rev)));
+        return __float2half(__builtin_amdgcn_cosf(__builtin_amdgcn_fractf(scaled(x, 0.15915494309189535f))));
     }
 };
 struct Exp
 {
     __device__ __forceinline__ half operator()(half x) const
     {
-        return __float2half(__builtin_amdgcn_exp2f(__half2float(x) * 1.4426950408889634f));
+        return __float2half(__builtin_amdgcn_exp2f(scaled(x, 1.4426950408889634f)));
     }
 };
 }
