@@ -244,7 +244,8 @@ struct GridGradientRecords
     {
         typedef typename Cfg::table_t table_t;
         constexpr int ENTRY_BYTES = F * static_cast<int>(sizeof(table_t));
-        constexpr int ALIGN = ENTRY_BYTES >= 8 ? 8 : ENTRY_BYTES >= 4 ? 4 : static_cast<int>(sizeof(table_t));
+        // entries lie at multiples of their size: aligned to the largest power of two that divides it
+        constexpr int ALIGN = (ENTRY_BYTES & -ENTRY_BYTES) >= 8 ? 8 : (ENTRY_BYTES & -ENTRY_BYTES);
         typedef table_t pair_t __attribute__((ext_vector_type(2 * F), aligned(ALIGN)));
         const int lower = cornerOfPair<LEVEL>(c, false), upper = cornerOfPair<LEVEL>(c, true);   // constants once the loop over c is unrolled
         if (idxH == idxL + 1u) {

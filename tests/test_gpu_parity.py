@@ -464,6 +464,8 @@ SLICE_GRIDS = [
           combination_mode="add"), "float"),
     (dict(n_in=1, n_levels=3, n_features_per_level=1, log2_hashmap_size=4, min_resolution=2, max_resolution=64), "float"),
     (dict(n_in=6, n_levels=2, n_features_per_level=1, log2_hashmap_size=12, min_resolution=2, max_resolution=5), "half"),
+    # entries of 6 bytes: a pair of them is loaded at once from an address that is a multiple of 2 only
+    (dict(n_in=2, n_levels=3, n_features_per_level=3, log2_hashmap_size=9, min_resolution=4, max_resolution=90), "half"),
 ]
 
 
