@@ -34,7 +34,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 # device code has changed since (or that has no counter run) reports traffic null.
 MEASURED_TRAFFIC_BYTES = {
     "cfg2-inference": {"points": 1 << 20, "fetch": 105187.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
-                       "kernels": "70f4a64d66af8916"},
+                       "kernels": "4ad4add129c4ab5d"},
 }
 
 

@@ -107,7 +107,8 @@ template <int F, typename T>
 __device__ __forceinline__ void loadPair(const T* __restrict__ p, float (&a)[F], float (&b)[F])
 {
     constexpr int ENTRY_BYTES = F * static_cast<int>(sizeof(T));
-    constexpr int ALIGN = ENTRY_BYTES >= 16 ? 16 : ENTRY_BYTES >= 8 ? 8 : ENTRY_BYTES >= 4 ? 4 : static_cast<int>(sizeof(T));
+    // the largest power of two that divides the size of an entry (12-byte entries: 4, 6-byte entries: 2)
+    constexpr int ALIGN = (ENTRY_BYTES & -ENTRY_BYTES) >= 16 ? 16 : (ENTRY_BYTES & -ENTRY_BYTES);
     typedef T pair_t __attribute__((ext_vector_type(2 * F), aligned(ALIGN)));
     const pair_t t = *reinterpret_cast<const pair_t*>(p);
 #pragma unroll
