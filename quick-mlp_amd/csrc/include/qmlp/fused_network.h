@@ -74,7 +74,8 @@ public:
 
         // Parameter gradients of grid encodings: summed slice by slice in LDS by a kernel of its own
         // (kernels/grid_gradient.h) instead of scattered with float atomics by the backward kernel.
-        // <0 (default): for batches of SLICE_GRADIENTS_MIN_BATCH points or more; 0: never; >0: always.
+        // <0 (default): for batches of SLICE_GRADIENTS_MIN_BATCH points or more (of half as many for grids of 8
+        // levels or more); 0: never; >0: always.
         int sliceGradients = -1;
 
         // Gradients of the layer weights: summed inside the backward kernel, which holds the adjoint
@@ -215,9 +216,12 @@ private:
     std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2];
     // Below this the two slice kernels cost more than the atomics they save (their work items zero and write
     // back whole slices whatever the batch): a train step of a 16-level hash grid at 2^14 / 2^15 / 2^16 / 2^17
-    // points 0.18 / 0.24 / 0.37 / 0.63 ms with atomics, 0.28 / 0.28 / 0.29 / 0.34 ms by slices; a dense 4-D grid
-    // crosses over at the same size.
+    // points 0.18 / 0.24 / 0.37 / 0.63 ms with atomics, 0.18 / 0.19 / 0.22 / 0.30 ms by slices; of one dense
+    // 4-D level with 8 features 0.08 / 0.09 / 0.12 / 0.19 against 0.10 / 0.11 / 0.12 / 0.23 ms. The atomics of a
+    // point grow with the number of levels, the fixed work of the slice kernels with the size of the table: grids
+    // of 8 levels or more take the slices from half the batch size on.
     static constexpr int SLICE_GRADIENTS_MIN_BATCH = 1 << 16;
+    static constexpr int SLICE_GRADIENTS_MIN_BATCH_MANY_LEVELS = 1 << 15;
     /** True if some encoding of the network offers gradient slices (the adjoint memory then has room for the adjoint of the encoded rows). */
     bool hasSliceGradients() const;
     /** Bytes per point of adjoint memory for the adjoint of the encoded rows (read by the records kernels); 0 without them. */

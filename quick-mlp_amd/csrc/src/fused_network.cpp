@@ -787,7 +787,13 @@ size_t FusedNetwork::sliceGradientWorkspaceBytes(long long numel) const
 bool FusedNetwork::useSliceGradients(int numel, int flags) const
 {
     if (!(flags & GRADIENTS_INPUT_ENCODINGS) || !hasSliceGradients()) return false;
-    return compileOptions_.sliceGradients > 0 || numel >= SLICE_GRADIENTS_MIN_BATCH;
+    if (compileOptions_.sliceGradients > 0 || numel >= SLICE_GRADIENTS_MIN_BATCH) return true;
+    if (numel < SLICE_GRADIENTS_MIN_BATCH_MANY_LEVELS) return false;
+    for (const auto& e : encodings_) {
+        IEncoding::GradientSliceLayout layout;
+        if (offersSlices(*e, &layout) && layout.slicesPerLevel.size() >= 8) return true;
+    }
+    return false;
 }
 
 int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients) const

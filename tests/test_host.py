@@ -172,11 +172,12 @@ def test_temporary_memory_sizes():
         assert net.adjoint_memory(n, 2) == per_adj * padded + slices * n_params * 4
         assert net.adjoint_memory(n, 3) == per_adj * padded + slices * n_params * 4
         assert net.adjoint_memory(n, 1) == 0
-        if n < (1 << 16):
+        if n < (1 << 15):
             # small batches scatter their grid gradients with atomics and need nothing for it
             assert net.adjoint_memory(n, 7) == per_adj * padded + slices * n_params * 4
             assert net.adjoint_memory(n, 5) == 0
-    # From 2^16 points on the grid gradients are summed slice by slice: the adjoint of the encoded rows
+    # From 2^15 points on (a grid of 16 levels; from 2^16 for grids of fewer than 8 levels) the grid gradients are
+    # summed slice by slice: the adjoint of the encoded rows
     # (32 halves per point) joins the adjoint pre-activations, and behind everything else come the
     # bucket cursors and the records (4 words each; per level, slices x (1.25 x share + 2048) of them:
     # the table of a level holds 8192 .. 1 048 576 floats, a slice 8192).
@@ -188,6 +189,9 @@ def test_temporary_memory_sizes():
     base = (per_adj + 2 * 32) * n + 512 * n_params * 4
     assert net.adjoint_memory(n, 7) == -(-base // 256) * 256 + cursors + -(-records * 16 // 256) * 256
     assert net.adjoint_memory(n, 4) == 2 * 32 * n + cursors + -(-records * 16 // 256) * 256
+    assert net.adjoint_memory((1 << 15) - 64, 5) == 0 and net.adjoint_memory(1 << 15, 5) > 0
+    few_levels = qmlp.Network(json.dumps(bc.CONFIGS[5]["cfg"]))
+    assert few_levels.adjoint_memory((1 << 16) - 64, 4) == 0 and few_levels.adjoint_memory(1 << 16, 4) > 0
     with pytest.raises(qmlp.QmlpError, match="At least one derivative"):
         net.adjoint_memory(10, 0)
 
