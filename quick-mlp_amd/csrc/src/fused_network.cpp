@@ -1026,7 +1026,8 @@ std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFl
 {
     if (kind == "inference" || kind == "forward") {
         int ppl = 1;
-        const int blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeForward, false, &ppl);
+        const int blockSize = forwardBlockSize(kind == "forward" ? compileOptions_.overwriteBlocksizeForward
+                                                                  : compileOptions_.overwriteBlocksizeInference, false, &ppl);
         return forwardSource(blockSize, ppl);
     }
     if (kind == "shapes") {
@@ -1055,7 +1056,7 @@ std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFl
     // the shape with the encoded rows in registers, whether or not the network would get it
     if (kind == "forward_registers") return forwardSource(2 * DEFAULT_BLOCK_SIZE, std::min(8, 256 / layers_[0].channelsIn), true);
     if (kind == "backward") return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true));
-    if (kind == "weight_update") return weightUpdateSource(DEFAULT_BLOCK_SIZE);
+    if (kind == "weight_update") return weightUpdateSource(weightUpdateBlockSize());
     throw std::runtime_error("unknown kernel kind '" + kind + "'");
 }
 

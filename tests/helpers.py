@@ -30,6 +30,16 @@ def require_gpu(encoding_cfg=None, adjoint_modes=(3,)):
         pytest.skip("no GPU in this environment")
 
 
+def warm_cache(*cfgs):
+    """In a CPU cache-warming pass: compiles the kernels of all these specifications into the
+    in-tree kernel cache and stops the test (a test that builds several networks calls this first,
+    because the first Case of a warming pass ends the test)."""
+    if os.environ.get("QMLP_WARM_CACHE"):
+        for cfg in cfgs:
+            qmlp.Network(json.dumps(cfg)).precompile(7)
+        pytest.skip("kernel cache warmed")
+
+
 def identity_cfg(n_in, widths, acts, biases, extra_acts=()):
     return {"num_inputs": n_in, "num_outputs": widths[-1],
             "activation_specification": ["qmlp/builtin-activations.json", *extra_acts],

@@ -534,3 +534,69 @@ def test_rows_in_registers_shape_is_not_offered_to_single_table_or_gather_heavy_
     cfg = json.loads(json.dumps(bc.CONFIGS[2]["cfg"]))
     cfg["options"] = {"register_staging": False}
     assert not any(shape == "registers" for _, shape in shapes(cfg))
+
+
+@pytest.mark.parametrize("option,value,flags,kind", [
+    ("overwrite_blocksize_inference", 96, 0, "inference"),
+    ("overwrite_blocksize_inference", 2048, 0, "inference"),
+    ("overwrite_blocksize_forward", 100, 1, "forward"),
+    ("overwrite_blocksize_backward", 32, 1, "backward"),
+    ("overwrite_blocksize_backward", 1088, 3, "backward"),
+    ("overwrite_blocksize_weight_update", 100, 2, "weight_update"),
+    ("overwrite_blocksize_weight_update", 4096, 2, "weight_update"),
+])
+def test_launch_options_out_of_range_are_refused(option, value, flags, kind):
+    """Workgroups are whole wavefronts of 64 lanes, at most 16 of them (the reference takes any
+    multiple of its warp size up to the device limit, src_cpp/src/fused_network.cpp:472-485)."""
+    cfg = json.loads(json.dumps(BASE))
+    cfg["options"] = {option: value}
+    net = qmlp.Network(json.dumps(cfg))          # options are parsed here, applied when a kernel is generated
+    message = "multiple of 64 and at most 1024, but is %d" % value
+    with pytest.raises(qmlp.QmlpError, match=message) as ei:
+        net.precompile(flags)
+    assert ei.value.code == 1                    # configuration_error
+    with pytest.raises(qmlp.QmlpError, match=message):
+        net.generated_source(kind, flags) if kind == "backward" else net.generated_source(kind)
+    # the kernels the option does not concern still generate
+    other = "backward" if kind != "backward" else "forward"
+    assert "__launch_bounds__(256)" in (net.generated_source(other, 1) if other == "backward" else net.generated_source(other))
+
+
+def test_launch_options_shape_the_generated_kernels():
+    cfg = json.loads(json.dumps(BASE))
+    cfg["options"] = {"overwrite_blocksize_inference": 64, "overwrite_blocksize_forward": 512,
+                      "overwrite_blocksize_backward": 1024, "overwrite_blocksize_weight_update": 128,
+                      "skew_shared_memory": True, "parallel_weight_update": False}
+    net = qmlp.Network(json.dumps(cfg))
+    assert "__launch_bounds__(64)" in net.generated_source("inference")
+    assert "__launch_bounds__(512)" in net.generated_source("forward")
+    assert "__launch_bounds__(1024)" in net.generated_source("backward", 3)
+    assert "__launch_bounds__(128)" in net.generated_source("weight_update")
+    shapes = json.loads(net.generated_source("shapes"))
+    assert {(s["pass"], s["block"]) for s in shapes} == {("inference", 64), ("forward", 512)}
+    # zero and negative values mean "not overwritten", as in the reference (values > 0 are taken)
+    cfg["options"] = {"overwrite_blocksize_inference": -1, "overwrite_blocksize_backward": 0}
+    net = qmlp.Network(json.dumps(cfg))
+    assert "__launch_bounds__(256)" in net.generated_source("inference")
+    assert "__launch_bounds__(256)" in net.generated_source("backward", 3)
+
+
+def test_staging_rows_beyond_the_lds_are_a_configuration_error():
+    """A workgroup shrinks until the staging rows of its wavefronts fit into the LDS beside the
+    weights; a network whose one staging tile does not fit is refused (the reference shrinks its
+    blocks the same way, src_cpp/src/fused_network.cpp:476-485, and then fails at the launch)."""
+    wide = {"num_inputs": 2048, "num_outputs": 16, "activation_specification": [bc.BUILTIN],
+            "encodings": [{"id": "Identity", "start_in": 0, "n_in": 2048}],
+            "network": [{"n_out": 16, "bias": False, "activation": "relu"}]}
+    net = qmlp.Network(json.dumps(wide))
+    with pytest.raises(qmlp.QmlpError, match="too large for the fused kernels") as ei:
+        net.generated_source("backward", 1)
+    assert ei.value.code == 1
+    # 1024 asked for, but 16 wavefronts x 64 rows x 264 halves exceed the LDS beside the weights
+    mid = json.loads(json.dumps(wide))
+    mid["num_inputs"] = 256
+    mid["encodings"][0]["n_in"] = 256
+    mid["options"] = {"overwrite_blocksize_backward": 1024}
+    src = qmlp.Network(json.dumps(mid)).generated_source("backward", 1)
+    m = re.search(r"__launch_bounds__\((\d+)\) [^;]*NetworkKernelBackward", src)
+    assert m and int(m.group(1)) % 64 == 0 and 64 <= int(m.group(1)) < 1024
