@@ -170,7 +170,10 @@ int qmlp_encoding_hashgrid_corners(qmlp_encoding_t encoding, const qmlp_tensor* 
  * that the gathers of the fused forward / inference kernels use, including their paired loads
  * (needs a bound table, src_cpp/include/qmlp/kernels/encoding_hashgrid.cuh:267-336 is what they
  * replace); mode 2: the entries and weights the gradient scatter of the fused backward kernel
- * adds to (encoding_hashgrid.cuh:345-369; nothing is added); mode 0 = qmlp_encoding_hashgrid_corners.
+ * adds to (encoding_hashgrid.cuh:345-369; nothing is added); mode 3: the entries and weights that
+ * the gradient records of large batches stand for (slice of the record's bucket + 16-bit offsets,
+ * and the entries of other slices that the records kernel adds itself; grids that offer gradient
+ * slices only); mode 0 = qmlp_encoding_hashgrid_corners.
  * The order of the 2^dim corners of a level is the order the code visits them. input = NULL only
  * compiles the kernel of that mode into the kernel cache (needs no GPU). */
 int qmlp_encoding_hashgrid_trace(qmlp_encoding_t encoding, const qmlp_tensor* input, int mode, uint32_t* indices,

@@ -112,7 +112,7 @@ public:
 
 private:
     [[nodiscard]] std::string configName() const;
-    std::optional<KernelFunction> cornersKernel_[3];
+    std::optional<KernelFunction> cornersKernel_[4];
 };
 
 QUICKMLP_NAMESPACE_END

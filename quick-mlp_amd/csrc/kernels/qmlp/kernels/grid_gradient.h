@@ -258,6 +258,58 @@ struct GridGradientRecords
         }
     }
 
+    /** What happens to an upper entry that lies in another slice than its record: the product adds it to the
+     *  gradient tensor right away. */
+    struct AddToTensor
+    {
+        float* __restrict__ gradients;
+        __device__ __forceinline__ void operator()(unsigned element, float weight, const unsigned (&adjWords)[(F + 1) / 2]) const
+        {
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                const unsigned short bits = static_cast<unsigned short>(adjWords[i / 2] >> (16 * (i % 2)));
+                unsafeAtomicAdd(gradients + element + i, weight * static_cast<float>(__builtin_bit_cast(f16, bits)));
+            }
+        }
+    };
+
+    /**
+     * The record of pair c of a point in one level: the offsets of its two entries within the slice of the lower
+     * one, their weights and the adjoint words. Returns the slice (= bucket within the level) that files it.
+     * \param otherSlice called with (element of feature 0 in the table, weight, adjWords) for an upper entry that
+     *    lies in another slice (an entry next to a slice boundary; in a hashed level one pair in thousands): the
+     *    record then keeps the lower entry only
+     */
+    template <int LEVEL, typename OtherSlice>
+    __device__ __forceinline__ static int buildRecord(const typename Grid::LevelSetup& s, int c,
+                                                      const unsigned (&adjWords)[(F + 1) / 2], unsigned (&rec)[RW],
+                                                      const OtherSlice& otherSlice)
+    {
+        constexpr int PD = Cfg::hashed[LEVEL] ? 0 : D - 1;
+        constexpr unsigned base = static_cast<unsigned>(Cfg::memoryOffset[LEVEL]);
+        unsigned idxL, idxH;
+        float w;
+        pairEntries<LEVEL>(s, c, idxL, idxH, w);
+        const int bucket = static_cast<int>(idxL * F / SLICE_FLOATS);   // the slice of the lower entry files the record
+        const unsigned sliceStart = static_cast<unsigned>(bucket) * SLICE_FLOATS;
+        const unsigned eL = idxL * F - sliceStart;
+        unsigned eH = idxH * F - sliceStart;                     // wraps if the upper entry lies below the slice
+        float wH = w * s.f[PD];
+        if (eH >= static_cast<unsigned>(SLICE_FLOATS)) {
+            otherSlice(base + idxH * F, wH, adjWords);
+            eH = eL;
+            wH = 0.f;
+        }
+        rec[0] = eL | (eH << 16);
+        rec[1] = __builtin_bit_cast(unsigned, w * (1.f - s.f[PD]));
+        rec[2] = __builtin_bit_cast(unsigned, wH);
+#pragma unroll
+        for (int i = 0; i < (F + 1) / 2; ++i) rec[3 + i] = adjWords[i];
+#pragma unroll
+        for (int v = Layout::RECORD_WORDS_USED; v < RW; ++v) rec[v] = 0u;
+        return bucket;
+    }
+
     /** Adds a record to the gradient tensor itself (its bucket was full); grad: element 0 of the record's slice. */
     __device__ __forceinline__ static void addToTensor(const unsigned (&rec)[RW], float* __restrict__ grad)
     {
@@ -316,33 +368,7 @@ struct GridGradientRecords
             }
 #pragma unroll
             for (int c = 0; c < PAIRS; ++c) {
-                unsigned idxL, idxH;
-                float w;
-                pairEntries<LEVEL>(s, c, idxL, idxH, w);
-                bucket[c] = static_cast<int>(idxL * F / SLICE_FLOATS);   // the slice of the lower entry files the record
-                const unsigned sliceStart = static_cast<unsigned>(bucket[c]) * SLICE_FLOATS;
-                const unsigned eL = idxL * F - sliceStart;
-                unsigned eH = idxH * F - sliceStart;                     // wraps if the upper entry lies below the slice
-                float wH = w * s.f[PD];
-                if (eH >= static_cast<unsigned>(SLICE_FLOATS)) {
-                    // the upper entry lies in another slice (an entry next to a slice boundary; in a hashed
-                    // level one pair in thousands): added right here, the record keeps the lower entry only
-#pragma unroll
-                    for (int i = 0; i < F; ++i) {
-                        const unsigned short bits = static_cast<unsigned short>(adjWords[i / 2] >> (16 * (i % 2)));
-                        unsafeAtomicAdd(params.parametersBackward + base + idxH * F + i,
-                                        wH * static_cast<float>(__builtin_bit_cast(f16, bits)));
-                    }
-                    eH = eL;
-                    wH = 0.f;
-                }
-                rec[c][0] = eL | (eH << 16);
-                rec[c][1] = __builtin_bit_cast(unsigned, w * (1.f - s.f[PD]));
-                rec[c][2] = __builtin_bit_cast(unsigned, wH);
-#pragma unroll
-                for (int i = 0; i < (F + 1) / 2; ++i) rec[c][3 + i] = adjWords[i];
-#pragma unroll
-                for (int v = Layout::RECORD_WORDS_USED; v < RW; ++v) rec[c][v] = 0u;
+                bucket[c] = buildRecord<LEVEL>(s, c, adjWords, rec[c], AddToTensor{params.parametersBackward});
                 // (a level of one slice needs no sorting: every lane has fixed places)
                 rank[c] = NS == 1 ? tid * PAIRS + c : atomicAdd(sHist + bucket[c], 1);
             }
@@ -538,6 +564,72 @@ __global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
     __syncthreads();
     if (threadIdx.x == 0 && sHist[0] != 0)
         atomicMax(cursors + GridGradientLayout<Cfg, SLICE_FLOATS>::firstBucket(Cfg::Levels), sHist[0]);
+}
+
+template <typename Cfg, int SLICE_FLOATS, int LEVEL>
+struct GridGradientTraceLevels
+{
+    template <typename Words>
+    __device__ __forceinline__ static void run(const float (&pos)[Cfg::Dim], const Words& adjWords, unsigned* idx, float* w)
+    {
+        if constexpr (LEVEL < Cfg::Levels) {
+            typedef GridGradientRecords<Cfg, 16, 0, SLICE_FLOATS, 256> Impl;
+            typedef EncodingHashGrid<Cfg> Grid;
+            constexpr int NC = Grid::NC;
+            const typename Grid::LevelSetup s = Grid::setupLevel(LEVEL, pos);
+#pragma unroll
+            for (int c = 0; c < Impl::PAIRS; ++c) {
+                unsigned rec[Impl::RW];
+                unsigned otherElement = 0u;
+                float otherWeight = 0.f;
+                bool other = false;
+                const int bucket = Impl::template buildRecord<LEVEL>(s, c, adjWords, rec,
+                    [&](unsigned element, float weight, const Words&) { other = true; otherElement = element; otherWeight = weight; });
+                const unsigned sliceStart = static_cast<unsigned>(Cfg::memoryOffset[LEVEL]) + static_cast<unsigned>(bucket) * SLICE_FLOATS;
+                idx[LEVEL * NC + 2 * c] = sliceStart + (rec[0] & 0xffffu);
+                w[LEVEL * NC + 2 * c] = __builtin_bit_cast(float, rec[1]);
+                if (NC > 1) {
+                    idx[LEVEL * NC + 2 * c + 1] = other ? otherElement : sliceStart + (rec[0] >> 16);
+                    w[LEVEL * NC + 2 * c + 1] = other ? otherWeight : __builtin_bit_cast(float, rec[2]);
+                }
+            }
+            GridGradientTraceLevels<Cfg, SLICE_FLOATS, LEVEL + 1>::run(pos, adjWords, idx, w);
+        }
+    }
+};
+
+/**
+ * Test aid: for every point (one per lane) and level, the table elements and weights that the records of
+ * GridGradientRecords::buildRecord stand for, decoded as the slice kernel decodes them (slice of the bucket +
+ * 16-bit offset), and the entries the records kernel adds itself because they lie in another slice.
+ * Slots as in CornerTrace: level * 2^Dim + 2 * pair (+ 1 for the upper entry).
+ */
+template <typename Cfg, int SLICE_FLOATS>
+__global__ void __launch_bounds__(256) GridGradientTraceKernel(
+    long long numel, const Tensor2Read<float> inputs, unsigned* __restrict__ indices, float* __restrict__ weights,
+    const HashGridParams<typename Cfg::table_t, Cfg::Dim> params)
+{
+    typedef GridGradientRecords<Cfg, 16, 0, SLICE_FLOATS, 256> Impl;
+    typedef EncodingHashGrid<Cfg> Grid;
+    constexpr int D = Cfg::Dim, F = Cfg::Features, NC = Grid::NC;
+    for (long long index = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x; index < numel;
+         index += static_cast<long long>(blockDim.x) * gridDim.x)
+    {
+        float pos[D];
+        {
+#pragma clang fp contract(off)
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                pos[d] = (inputs.data_[index * inputs.strides_[0] + static_cast<long long>(d + Cfg::Start) * inputs.strides_[1]]
+                          - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
+        }
+        unsigned* idx = indices + index * (Cfg::Levels * NC);
+        float* w = weights + index * (Cfg::Levels * NC);
+        unsigned adjWords[(F + 1) / 2];
+#pragma unroll
+        for (int i = 0; i < (F + 1) / 2; ++i) adjWords[i] = 0x3c003c00u;   // 1.0 | 1.0
+        GridGradientTraceLevels<Cfg, SLICE_FLOATS, 0>::run(pos, adjWords, idx, w);
+    }
 }
 
 template <typename Cfg, int SLICE_FLOATS>

@@ -178,7 +178,8 @@ void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* we
     CHECK_DIM(input, 2);
     CHECK_DTYPE(input, Tensor::FLOAT);
     CHECK_ERROR(input.size(1) > maxInputChannel());
-    CHECK_ERROR(mode >= 0 && mode <= 2, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter");
+    CHECK_ERROR(mode >= 0 && mode <= 3, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter, "
+                                        "3: the gradient records of the slice kernels");
     CHECK_ERROR(mode != 2 || (numFeaturesPerLevel_ & (numFeaturesPerLevel_ - 1)) == 0 && numFeaturesPerLevel_ <= 32,
                 "the tile-wide gradient scatter exists for 1, 2, 4 .. 32 features per level");
     CHECK_ERROR(mode == 0 || hasParameterTensor(Tensor::INFERENCE), "the traces read the table: bind one first");
@@ -194,13 +195,33 @@ void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* we
     const int grid = static_cast<int>(std::min<long long>(divUp<long long>(numel, block), fun.fullGridSize(block, 0)));
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     int perPoint = numLevels() * (1 << ndim());
+    if (mode == 3) {
+        void* args[] = {&numel, &inputAcc, &indices, &weights, paramBytes.data()};
+        fun.launch(grid, block, 0, stream, args);
+        return;
+    }
     void* args[] = {&numel, &inputAcc, &indices, &weights, &perPoint, paramBytes.data()};
     fun.launch(grid, block, 0, stream, args);
 }
 
 void EncodingHashGrid::precompileCorners(int mode, bool compileOnly)
 {
-    CHECK_ERROR(mode >= 0 && mode <= 2, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter");
+    CHECK_ERROR(mode >= 0 && mode <= 3, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter, "
+                                        "3: the gradient records of the slice kernels");
+    if (mode == 3) {
+        // the record building of kernels/grid_gradient.h with the slice size the fused network uses for this grid
+        GradientSliceLayout layout;
+        CHECK_ERROR(gradientSlices(layout), "this grid has no gradient slices");
+        std::stringstream source;
+        fillCode(source);
+        source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient.h");
+        const int flags = QuickMLP::Instance().getCompileFlags() | (compileOnly ? KernelLoader::CompileOnly : 0);
+        auto kernel = QuickMLP::Instance().kernelLoader()->getKernel(
+            "qmlp::kernel::GridGradientTraceKernel<" + layout.configType + ", " + std::to_string(layout.sliceFloats) + ">",
+            source.str(), flags);
+        if (!compileOnly) cornersKernel_[mode] = kernel.value();
+        return;
+    }
     {
         const std::string name = qualifiedName();
         const std::string source = standaloneSource(

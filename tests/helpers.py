@@ -148,12 +148,16 @@ def check_gradients(case, X, adj, flags, got, kinks=False, what="", kink_fractio
     return ref0
 
 
-def baseline_case(cfg_id, table_scale=None, seed=None):
-    """A Case for BASELINE config cfg_id with its seeded parameters (and tables)."""
+def baseline_case(cfg_id, table_scale=None, seed=None, options=None):
+    """A Case for BASELINE config cfg_id with its seeded parameters (and tables); options are
+    added to the "options" of the specification."""
     c = bc.CONFIGS[cfg_id]
     seed = bc.PARAMETER_SEED[cfg_id] if seed is None else seed
     rng = np.random.default_rng(seed)
-    case = Case(c["cfg"], bc.ORACLE_ACTIVATIONS)
+    cfg = json.loads(json.dumps(c["cfg"]))
+    if options:
+        cfg.setdefault("options", {}).update(options)
+    case = Case(cfg, bc.ORACLE_ACTIVATIONS)
     case.set_parameters(bc.make_parameters(cfg_id, rng).astype(np.float32))
     for i, e in enumerate(case.oracle.encodings):
         if e[0] == "hashgrid":

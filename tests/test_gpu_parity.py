@@ -257,6 +257,23 @@ GRID_SPECS = [
 ]
 
 
+SLICE_GRIDS = [
+    # 3-D, 6 levels, dense and hashed (several slices per level only in the large variants below)
+    (dict(n_in=3, n_levels=6, n_features_per_level=2, log2_hashmap_size=10, min_resolution=4, max_resolution=128), "half"),
+    # hashed levels of 2^16 entries x 2 features = 4 slices each, dense levels of 1, 1 and 3 slices
+    (dict(n_in=3, n_levels=7, n_features_per_level=2, log2_hashmap_size=16, min_resolution=8, max_resolution=300), "float"),
+    # one dense 4-D level of 20^4 x 8 features: 40 slices, pairs along the last coordinate straddle slice borders
+    (dict(n_in=4, n_levels=1, n_features_per_level=8, log2_hashmap_size=-1, min_resolution=20, max_resolution=20), "half"),
+    # dense 2-D levels up to 400^2 cells, 3 features (slices of 10 922 entries), levels summed ("add")
+    (dict(n_in=2, n_levels=4, n_features_per_level=3, log2_hashmap_size=-1, min_resolution=5, max_resolution=400,
+          combination_mode="add"), "float"),
+    (dict(n_in=1, n_levels=3, n_features_per_level=1, log2_hashmap_size=4, min_resolution=2, max_resolution=64), "float"),
+    (dict(n_in=6, n_levels=2, n_features_per_level=1, log2_hashmap_size=12, min_resolution=2, max_resolution=5), "half"),
+    # entries of 6 bytes: a pair of them is loaded at once from an address that is a multiple of 2 only
+    (dict(n_in=2, n_levels=3, n_features_per_level=3, log2_hashmap_size=9, min_resolution=4, max_resolution=90), "half"),
+]
+
+
 def _grid_cfg(spec, precision="float", start=0):
     d = spec["n_in"]
     cfg = {"id": "HashGrid", "start_in": start, "combination_mode": "concat",
@@ -282,20 +299,31 @@ def _per_point_sets(idx, w):
     return idx, np.where(last, acc, 0.0)
 
 
-@pytest.mark.parametrize("spec", GRID_SPECS + [bc.hashgrid3d("float"), bc.hashgrid3d("half"), bc.densegrid4d("half")])
+@pytest.mark.parametrize("spec", GRID_SPECS + [bc.hashgrid3d("float"), bc.hashgrid3d("half"), bc.densegrid4d("half")]
+                         + [dict(s, parameter_precision=p) for s, p in SLICE_GRIDS[1:4] + SLICE_GRIDS[6:]])
 def test_grid_indices_are_bit_exact(spec):
     """The table entries the device code touches, against the oracle's restatement of the
     reference's index arithmetic (encoding_hashgrid.cuh:17-60,279-287): the index function on its
     own (mode 0, corner by corner in the reference's order), and the entries that the code of the
     fused kernels really uses -- the paired gathers of the forward pass (mode 1: dense pairs
     along the last coordinate, hashed pairs idx / idx^1) and the lane-group gradient scatter of
-    the backward pass (mode 2) -- as sets per point and level, bit for bit, with their weights."""
+    the backward pass (mode 2) -- as sets per point and level, bit for bit, with their weights.
+    Mode 3, for grids of up to four dimensions: what the gradient records of large batches stand
+    for (kernels/grid_gradient.h: the slice of the record's bucket plus the two 16-bit offsets
+    as the slice kernel decodes them, and the entries of other slices that the records kernel adds
+    itself)."""
     import json
     import qmlp
-    cfg = _grid_cfg(spec) if "id" not in spec else spec
+    cfg = _grid_cfg(spec, spec.get("parameter_precision", "float")) if "id" not in spec else spec
     enc = qmlp.Encoding(json.dumps(cfg))
     f = cfg["n_features_per_level"]
     modes = [0, 1] + ([2] if f & (f - 1) == 0 and f <= 32 else [])
+    try:
+        enc.hashgrid_corners(None, 3)       # compiles the kernel of mode 3, or says that the grid has no slices
+        modes.append(3)
+    except qmlp.QmlpError as e:
+        # more than four dimensions, or a level of more than 512 slices
+        assert "no gradient slices" in str(e) and (cfg["n_in"] > 4 or cfg["max_resolution"] == 2048)
     if os.environ.get("QMLP_WARM_CACHE"):
         for m in modes:
             enc.hashgrid_corners(None, m)
@@ -450,23 +478,6 @@ def test_network_with_two_grids_against_oracle():
     got = case.gpu_train(X, adj, flags)
     assert_close(got["out"], case.oracle.forward(X), "forward")
     check_gradients(case, X, adj, flags, got)
-
-
-SLICE_GRIDS = [
-    # 3-D, 6 levels, dense and hashed (several slices per level only in the large variants below)
-    (dict(n_in=3, n_levels=6, n_features_per_level=2, log2_hashmap_size=10, min_resolution=4, max_resolution=128), "half"),
-    # hashed levels of 2^16 entries x 2 features = 4 slices each, dense levels of 1, 1 and 3 slices
-    (dict(n_in=3, n_levels=7, n_features_per_level=2, log2_hashmap_size=16, min_resolution=8, max_resolution=300), "float"),
-    # one dense 4-D level of 20^4 x 8 features: 40 slices, pairs along the last coordinate straddle slice borders
-    (dict(n_in=4, n_levels=1, n_features_per_level=8, log2_hashmap_size=-1, min_resolution=20, max_resolution=20), "half"),
-    # dense 2-D levels up to 400^2 cells, 3 features (slices of 10 922 entries), levels summed ("add")
-    (dict(n_in=2, n_levels=4, n_features_per_level=3, log2_hashmap_size=-1, min_resolution=5, max_resolution=400,
-          combination_mode="add"), "float"),
-    (dict(n_in=1, n_levels=3, n_features_per_level=1, log2_hashmap_size=4, min_resolution=2, max_resolution=64), "float"),
-    (dict(n_in=6, n_levels=2, n_features_per_level=1, log2_hashmap_size=12, min_resolution=2, max_resolution=5), "half"),
-    # entries of 6 bytes: a pair of them is loaded at once from an address that is a multiple of 2 only
-    (dict(n_in=2, n_levels=3, n_features_per_level=3, log2_hashmap_size=9, min_resolution=4, max_resolution=90), "half"),
-]
 
 
 @pytest.mark.parametrize("spec,precision", SLICE_GRIDS)
@@ -656,9 +667,12 @@ def test_baseline_inference_published_table_scale(cfg_id):
                  rel=5e-3, abs_=1e-3, allowed_fraction=1e-3)
 
 
-@pytest.mark.parametrize("cfg_id,N", [(3, 1 << 14), (4, 1 << 13), (5, 1 << 14)])
-def test_baseline_train_step(cfg_id, N):
-    case, rng = baseline_case(cfg_id, table_scale=1.0 if cfg_id in (3, 5) else None)
+@pytest.mark.parametrize("cfg_id,N,slices", [(3, 1 << 14, -1), (4, 1 << 13, -1), (5, 1 << 14, -1), (3, 1 << 14, 1), (5, 1 << 14, 1)])
+def test_baseline_train_step(cfg_id, N, slices):
+    """slices = 1: the grid gradients summed per slice of the table (the path the benchmark's batch sizes take, which
+    a batch of this size would not take by itself), so that the table gradients of the 16-level grid meet the oracle
+    through the records and slice kernels."""
+    case, rng = baseline_case(cfg_id, table_scale=1.0 if cfg_id in (3, 5) else None, options={"slice_gradients": slices})
     X = bc.make_inputs(cfg_id, N, rng)
     target = bc.make_targets(cfg_id, X)
     out_ref = case.oracle.forward(X)
