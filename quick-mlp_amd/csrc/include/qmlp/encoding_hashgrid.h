@@ -76,6 +76,8 @@ public:
     [[nodiscard]] int numSweptTables() const override { return numLevels_; }
     [[nodiscard]] int gatherRegistersPerPoint() const override;
     [[nodiscard]] bool pointOrderKey(kernel::PointOrderKey& key, long long numPoints = 0) const override;
+    /** pointOrderKey() for grids that do not qualify through their dense levels: slabs of multi-level hashed grids. */
+    [[nodiscard]] bool hashedPointOrderKey(kernel::PointOrderKey& key, long long numPoints) const;
     [[nodiscard]] int channelsWrittenTogether() const override { return numFeaturesPerLevel_; }
     void setParameter(const Tensor& tensor, Tensor::Usage usage) override;
     [[nodiscard]] bool hasParameterTensor(Tensor::Usage usage) const override

@@ -1,6 +1,6 @@
-// Orders the points of a batch by the slab of a dense grid they fall into, so that the
+// Orders the points of a batch by the slab of a grid they fall into, so that the
 // wavefronts that run side by side gather from the same few megabytes of the table and
-// find them in L1 / L2. A counting sort over at most 1024 slabs in three launches, without
+// find them in L1 / L2, and the lanes of one gather instruction fall onto fewer cache lines. A counting sort over at most 1024 slabs in three launches, without
 // atomics on device memory (a first version reserved the ranges with one returning atomic per
 // slab and workgroup: 256 workgroups on the same 64 cache lines took 120 us):
 //   PointOrderCount   one histogram per workgroup (summed in LDS) over its chunk of the batch,
@@ -22,17 +22,34 @@ constexpr int POINT_ORDER_MAX_SLABS = 1024;
 constexpr int POINT_ORDER_BLOCK = 1024;
 constexpr int POINT_ORDER_POINTS_PER_THREAD = 8;    // a workgroup's chunk: 8192 points (offsets in it take 13 bits)
 
-/** Slab of the point in row `index`: the two leading grid coordinates, clamped to the box. */
+/** Slab of one coordinate, clamped to the box (the comparisons are false for NaN, which then lands in slab 0). */
+__device__ __forceinline__ int pointOrderSlab1(const float* row, long long channelStride, int channel, float lo, float scale, int slabs)
+{
+    const float p = (row[static_cast<long long>(channel) * channelStride] - lo) * scale;
+    return p > 0.f ? static_cast<int>(fminf(p, static_cast<float>(slabs - 1))) : 0;
+}
+
+/** Slab of the point in row `index`: up to three grid coordinates, clamped to the box. */
 __device__ __forceinline__ int pointOrderSlab(const Tensor2Read<float>& inputs, long long index, const PointOrderKey& key)
 {
     const float* row = inputs.data_ + index * inputs.strides_[0];
-    const float p0 = (row[static_cast<long long>(key.channel0) * inputs.strides_[1]] - key.min0) * key.scale0;
-    // the comparisons are false for NaN, which then lands in slab 0
-    int s = p0 > 0.f ? static_cast<int>(fminf(p0, static_cast<float>(key.slabs0 - 1))) : 0;
+    int s = pointOrderSlab1(row, inputs.strides_[1], key.channel0, key.min0, key.scale0, key.slabs0);
     if (key.slabs1 > 1) {
-        const float p1 = (row[static_cast<long long>(key.channel1) * inputs.strides_[1]] - key.min1) * key.scale1;
-        const int s1 = p1 > 0.f ? static_cast<int>(fminf(p1, static_cast<float>(key.slabs1 - 1))) : 0;
-        s = s * key.slabs1 + s1;
+        const int s1 = pointOrderSlab1(row, inputs.strides_[1], key.channel1, key.min1, key.scale1, key.slabs1);
+        if (key.slabs2 > 1) {
+            const int s2 = pointOrderSlab1(row, inputs.strides_[1], key.channel2, key.min2, key.scale2, key.slabs2);
+            if (key.interleave12) {
+                // bit b of s1 to position 2b + 1, of s2 to 2b (at most 5 bits each)
+                int z = 0;
+#pragma unroll
+                for (int b = 0; b < 5; ++b) z |= ((s1 >> b) & 1) << (2 * b + 1) | ((s2 >> b) & 1) << (2 * b);
+                s = s * (key.slabs1 * key.slabs2) + z;
+            } else {
+                s = (s * key.slabs1 + s1) * key.slabs2 + s2;
+            }
+        } else {
+            s = s * key.slabs1 + s1;
+        }
     }
     return s;
 }
@@ -109,19 +126,39 @@ __device__ __forceinline__ int pointOrderBlockScan(int value, int* sWaveSum)
     return before + inclusive - value;
 }
 
-/** The channels of one input row; one 16-byte load where the layout allows it. */
+/** The channels of one input row; one load of 8, 12 or 16 bytes where the layout allows it (vectorChannels > 0:
+ *  rows of that many channels with unit stride between them, aligned to the vector). */
 template <int MAX_CHANNELS>
-__device__ __forceinline__ void pointOrderLoadRow(const Tensor2Read<float>& inputs, long long index, bool vector4, float (&row)[MAX_CHANNELS])
+__device__ __forceinline__ void pointOrderLoadRow(const Tensor2Read<float>& inputs, long long index, int vectorChannels, float (&row)[MAX_CHANNELS])
 {
     const float* src = inputs.data_ + index * inputs.strides_[0];
-    if (vector4) {
+    typedef float f32x3a __attribute__((ext_vector_type(3), aligned(4)));
+    if (MAX_CHANNELS >= 4 && vectorChannels == 4) {
         const float4 v = *reinterpret_cast<const float4*>(src);
-        row[0] = v.x; row[1] = v.y; row[2] = v.z; row[3] = v.w;
+        row[0] = v.x; row[1] = v.y; row[2 % MAX_CHANNELS] = v.z; row[3 % MAX_CHANNELS] = v.w;
+    } else if (MAX_CHANNELS >= 3 && vectorChannels == 3) {
+        const f32x3a v = *reinterpret_cast<const f32x3a*>(src);
+        row[0] = v[0]; row[1] = v[1]; row[2 % MAX_CHANNELS] = v[2];
+    } else if (MAX_CHANNELS >= 2 && vectorChannels == 2) {
+        const float2 v = *reinterpret_cast<const float2*>(src);
+        row[0] = v.x; row[1] = v.y;
     } else {
 #pragma unroll
         for (int c = 0; c < MAX_CHANNELS; ++c)
             row[c] = c < inputs.sizes_[1] ? src[static_cast<long long>(c) * inputs.strides_[1]] : 0.f;
     }
+}
+
+/** How the rows of inputs can be loaded as one vector each (pointOrderLoadRow), 0 if they cannot. */
+__device__ __forceinline__ int pointOrderVectorChannels(const Tensor2Read<float>& inputs)
+{
+    const int channels = inputs.sizes_[1];
+    if (inputs.strides_[1] != 1) return 0;
+    const unsigned long long base = reinterpret_cast<unsigned long long>(inputs.data_);
+    if (channels == 4 && inputs.strides_[0] % 4 == 0 && base % 16 == 0) return 4;
+    if (channels == 3) return 3;   // three words from an address that is a multiple of four
+    if (channels == 2 && inputs.strides_[0] % 2 == 0 && base % 8 == 0) return 2;
+    return 0;
 }
 
 /**
@@ -176,8 +213,7 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
     __syncthreads();
 
     const int channels = inputs.sizes_[1];
-    const bool vector4 = channels == 4 && inputs.strides_[1] == 1 && inputs.strides_[0] % 4 == 0
-        && reinterpret_cast<unsigned long long>(inputs.data_) % 16 == 0;
+    const int vectorChannels = pointOrderVectorChannels(inputs);
 #pragma unroll 4
     for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
         const int j = k * POINT_ORDER_BLOCK + t;
@@ -186,11 +222,17 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
         const long long index = chunk + (entry & 0xffffu);
         const int s = static_cast<int>(entry >> 16);
         float row[MAX_CHANNELS];
-        pointOrderLoadRow<MAX_CHANNELS>(inputs, index, vector4, row);
+        pointOrderLoadRow<MAX_CHANNELS>(inputs, index, vectorChannels, row);
         const long long position = sStart[s] + (j - sLocalStart[s]);
         order[position] = static_cast<int>(index);
-        if (vector4) {
-            *reinterpret_cast<float4*>(sortedInputs + position * 4) = make_float4(row[0], row[1], row[2], row[3]);
+        typedef float f32x3a __attribute__((ext_vector_type(3), aligned(4)));
+        if (MAX_CHANNELS >= 4 && vectorChannels == 4) {
+            *reinterpret_cast<float4*>(sortedInputs + position * 4) = make_float4(row[0], row[1], row[2 % MAX_CHANNELS], row[3 % MAX_CHANNELS]);
+        } else if (MAX_CHANNELS >= 3 && vectorChannels == 3) {
+            const f32x3a v = {row[0], row[1], row[2 % MAX_CHANNELS]};
+            *reinterpret_cast<f32x3a*>(sortedInputs + position * 3) = v;
+        } else if (MAX_CHANNELS >= 2 && vectorChannels == 2) {
+            *reinterpret_cast<float2*>(sortedInputs + position * 2) = make_float2(row[0], row[1]);
         } else {
 #pragma unroll
             for (int c = 0; c < MAX_CHANNELS; ++c)

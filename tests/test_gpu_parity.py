@@ -954,6 +954,54 @@ def test_inference_sorted_by_grid_slab_gives_the_same_bits_as_the_order_given():
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dim", [3, 2])
+def test_hashed_grid_sorted_on_request_gives_the_same_bits(dim):
+    """options.sort_points = 1 on a multi-level hashed grid: the batch is ordered by slabs of the grid's second and
+    third coordinate (32 x 32 along a Z curve; 1024 slabs of the second one in 2-D) in front of the fused kernel.
+    Inference agrees bit for bit with the batch as given (rows of three floats move as one 12-byte load and store),
+    a train step gives the same outputs and input gradients and the same sums for the other gradients."""
+    spec = dict(n_in=dim, n_levels=8, n_features_per_level=2, log2_hashmap_size=12, min_resolution=4, max_resolution=128)
+    grid = _grid_cfg(spec, "half")
+    nets = []
+    for mode in (1, 0):
+        cfg = {"num_inputs": dim, "num_outputs": 1, "activation_specification": [bc.BUILTIN], "encodings": [dict(grid)],
+               "network": [{"n_out": 32, "bias": False, "activation": "celu"}, {"n_out": 1, "bias": False, "activation": "identity"}],
+               "options": {"sort_points": mode}}
+        rng = np.random.default_rng(3)
+        case = Case(cfg)
+        case.set_parameters(random_parameters(case.oracle, rng))
+        case.set_table(0, rng.uniform(-1, 1, case.oracle.encodings[0][1].n_params))
+        nets.append(case)
+    sorted_, plain = nets
+    lo = np.array(grid["bounding_box_min"], np.float32)
+    sz = np.array(grid["bounding_box_size"], np.float32)
+    rng = np.random.default_rng(4)
+    for N in (1, 777, 8193, (1 << 17) + 5):
+        X = (lo + sz * rng.uniform(-0.05, 1.05, (N, dim))).astype(np.float32)
+        if N > 100:
+            X[::13, 1] = np.nan
+            X[5::13, 0] = np.inf
+        a, b = sorted_.gpu_inference(X), plain.gpu_inference(X)
+        assert np.array_equal(np.isnan(a), np.isnan(b)) and np.array_equal(a[~np.isnan(a)], b[~np.isnan(b)])
+    N = 20000
+    rng = np.random.default_rng(4)
+    X = (lo + sz * rng.uniform(0, 1, (N, dim))).astype(np.float32)
+    assert_close(sorted_.gpu_inference(X), sorted_.oracle.forward(X), "sorted inference against the oracle")
+    adj = (rng.uniform(-1, 1, (N, 1)) / 16).astype(np.float32)
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    got, ref = sorted_.gpu_train(X, adj, flags), plain.gpu_train(X, adj, flags)
+    assert np.array_equal(got["out"], ref["out"]) and np.array_equal(got["adj_x"], ref["adj_x"])
+    oracle = sorted_.oracle.backward(X, adj, flags, round_mode=0)
+    for name, a, e in (("input", got["adj_x"], oracle["adj_x"]), ("weight", got["grads"], oracle["grads"]),
+                       ("grid", got["table_grads"][0], oracle["table_grads"][0])):
+        s_ = max(1.0, float(np.abs(e).max()))
+        assert_close(a / s_, e / s_, name + " gradients of the sorted batch vs fp32 oracle")
+    scale = np.abs(ref["table_grads"][0]).max()
+    assert np.allclose(got["table_grads"][0] / scale, ref["table_grads"][0] / scale, rtol=1e-4, atol=1e-6)
+    scale = np.abs(ref["grads"]).max()
+    assert np.allclose(got["grads"] / scale, ref["grads"] / scale, rtol=1e-3, atol=1e-5)
+
+
 @pytest.mark.parametrize("slices", [0, 1])
 def test_training_sorted_by_grid_slab_matches_the_order_given(slices):
     """The same network trains its large batches in the sorted order too (``sort_training``): the
