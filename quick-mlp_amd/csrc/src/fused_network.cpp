@@ -1389,7 +1389,8 @@ void FusedNetwork::precompile(int adjointFlags)
     }
     kernel::PointOrderKey key{};
     for (const auto& e : encodings_)
-        if (compileOptions_.sortPoints != 0 && e->pointOrderKey(key)) {
+        // asked for, or chosen by itself for batches that are large enough
+        if (compileOptions_.sortPoints != 0 && e->pointOrderKey(key, compileOptions_.sortPoints > 0 ? 0 : (1ll << 30))) {
             auto kl = QuickMLP::Instance().kernelLoader();
             const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
             const std::string scatter = "PointOrderScatter<" + std::to_string(channelsIn_ <= 4 ? 4 : channelsIn_ <= 8 ? 8 : 16) + ">";

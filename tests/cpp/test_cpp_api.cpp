@@ -70,7 +70,9 @@ static void hostPart()
 
     // Which grids offer a slab key for sorting inference batches: a dense 32^4 grid with 8 fp16
     // features (16.8 MB) does, in 31 x 31 slabs of one cell over its box [1,3] x [0,4];
-    // a 16-level hash grid whose dense levels are small does not, nor does a small dense grid.
+    // a 16-level hash grid whose dense levels are small offers one (32 x 32 slabs of its second and third coordinate
+    // along a Z curve) when asked whether an order exists, never for a batch size (its sort costs more than it
+    // gains); a small dense grid has none.
     {
         auto dense = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 1, "n_in": 4,
             "n_levels": 1, "n_features_per_level": 8, "log2_hashmap_size": -1, "min_resolution": 32, "max_resolution": 32,
@@ -78,12 +80,15 @@ static void hostPart()
             "parameter_precision": "half"})json"));
         kernel::PointOrderKey key{};
         CHECK(dense->pointOrderKey(key));
-        CHECK(key.channel0 == 1 && key.channel1 == 2 && key.slabs0 == 31 && key.slabs1 == 31);
+        CHECK(key.channel0 == 1 && key.channel1 == 2 && key.slabs0 == 31 && key.slabs1 == 31 && key.slabs2 == 1);
         CHECK(key.min0 == 1.f && key.min1 == 0.f && key.scale0 == 15.5f && key.scale1 == 7.75f);
         auto hashed = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 0, "n_in": 3,
             "n_levels": 16, "n_features_per_level": 2, "log2_hashmap_size": 19, "min_resolution": 16, "max_resolution": 4096,
             "combination_mode": "concat", "bounding_box_min": [0, 0, 0], "bounding_box_size": [1, 1, 1]})json"));
-        CHECK(!hashed->pointOrderKey(key));
+        CHECK(hashed->pointOrderKey(key));
+        CHECK(key.slabs0 == 1 && key.slabs1 == 32 && key.slabs2 == 32 && key.interleave12 == 1);
+        CHECK(key.channel1 == 1 && key.channel2 == 2 && key.scale1 == 32.f && key.min2 == 0.f);
+        CHECK(!hashed->pointOrderKey(key, 1 << 20) && !hashed->pointOrderKey(key, 1 << 24));
         auto small = EncodingFactory::Instance().create(json::parse(R"json({"id": "HashGrid", "start_in": 0, "n_in": 3,
             "n_levels": 1, "n_features_per_level": 2, "log2_hashmap_size": -1, "min_resolution": 64, "max_resolution": 64,
             "combination_mode": "concat", "bounding_box_min": [0, 0, 0], "bounding_box_size": [1, 1, 1]})json"));
