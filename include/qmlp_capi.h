@@ -129,7 +129,10 @@ int qmlp_network_precompile(qmlp_network_t network, int adjoint_flags);
  * themselves only enqueue kernels (for callers that capture them into a HIP graph). No counterpart in the
  * reference, whose first call on a network compiles its kernels. */
 int qmlp_network_prepare(qmlp_network_t network, int numel, int adjoint_flags);
-/* The generated device source; kind = "forward" | "backward" | "weight_update". */
+/* The generated device source; kind = "inference" | "forward" | "backward" | "weight_update". Diagnostics as JSON:
+ * "shapes" (the shapes of the forward kernel the network may launch), "backward_resources" and
+ * "backward_slices_resources" (workgroup size, LDS, registers and scratch bytes of the loaded backward kernel;
+ * these two need a device). */
 int qmlp_network_generated_source(qmlp_network_t network, const char* kind, int adjoint_flags, char** source);
 
 /* ---- qmlp::IEncoding (src_cpp/include/qmlp/iencoding.h:36-140) ---- */

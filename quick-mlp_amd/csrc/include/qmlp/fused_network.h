@@ -401,8 +401,10 @@ private:
     int weightUpdateBlockSize() const;
     // number of batch slices whose partial weight gradients are kept in the adjoint memory
     int weightUpdateSlices(int numTiles) const;
-    /** Layers whose weight gradients the backward kernel sums itself (options.fused_weight_update). */
-    std::vector<bool> fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients) const;
+    /** Layers whose weight gradients the backward kernel sums itself (options.fused_weight_update).
+     *  wideRegisters: receives whether that kernel runs one wavefront per SIMD with 512 registers (the gradient
+     *  tiles of all layers in its accumulation registers). */
+    std::vector<bool> fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients, bool* wideRegisters = nullptr) const;
     /** LDS halves per wavefront of the backward kernel for the tile that Layer::weightGradient transposes. */
     int fusedWeightUpdateTransposeHalves() const;
     /** Channels of adjoint pre-activations that the backward kernel stores per point for the weight-update kernels. */

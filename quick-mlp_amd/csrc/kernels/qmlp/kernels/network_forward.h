@@ -170,14 +170,6 @@ $$TILE_LOOP_PRAGMA$$
         (void)tmpTile;
         const f16* sTile = sStage + (REGISTER_STAGING ? 0 : q) * (TILE_POINTS * STAGE_STRIDE);
         (void)sTile;
-        // where the rows of this tile's results go (-1: outside the batch); with a sorted batch that is read from
-        // memory: asked for here, used behind the layers
-        long long outputRow[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int p = tile * TILE_POINTS + 4 * r + nt;
-            outputRow[nt] = p < numel ? (pointOrder ? pointOrder[p] : p) : -1;
-        }
         if (REGISTER_STAGING) {
             // the lane's row of this tile: registers -> staging row, 8 bytes at a time
             if (q > 0) waveLdsSync();   // the operands of the previous tile have been read
@@ -262,6 +254,12 @@ $$CALL_NETWORK_LAYERS$$
 
         // output: lane holds channels 16m+4g+i of the points 4r+nt
         const int actualChannelsOut = outputs.sizes_[1];
+        long long outputRow[NT];   // -1: outside the batch
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int p = tile * TILE_POINTS + 4 * r + nt;
+            outputRow[nt] = p < numel ? (pointOrder ? pointOrder[p] : p) : -1;
+        }
         // output channels that lie side by side in memory leave four at a time (a lane holds
         // channels 16m+4g .. +3 of its points), rows of two channels as one 8-byte store
         const bool rowsOfFloat2 = actualChannelsOut == 2 && outputs.strides_[1] == 1 && outputs.strides_[0] % 2 == 0

@@ -604,9 +604,10 @@ int FusedNetwork::weightUpdateSlices(int numTiles) const
     return std::max(1, std::min(divUp(numTiles, waves), MAX_WEIGHT_UPDATE_SLICES));
 }
 
-std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients) const
+std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients, bool* wideRegisters) const
 {
     std::vector<bool> fused(layers_.size(), false);
+    if (wideRegisters) *wideRegisters = false;
     if (compileOptions_.fusedWeightUpdate == 0 || !(adjointFlags & GRADIENTS_NETWORK_WEIGHTS)) return fused;
     // a backward kernel that gathers from or scatters into the tables of an encoding itself has no registers to spare
     // (32 -> 64 -> 64 -> 16 behind a hash grid: 320 bytes of scratch per lane without any gradient tile)
@@ -630,11 +631,24 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
     // Four accumulator registers per gradient tile and lane, for as long as the kernel runs: the layers with the
     // fewest tiles first, up to 16 tiles (all 28 tiles of a 32 -> 64 -> 64 -> 16 network: 1 KB of scratch per lane
     // and a backward kernel of 116 instead of 31 us; the weight-update kernels it replaced took 62 us).
-    const int budget = compileOptions_.fusedWeightUpdate > 0 ? 32 : 16;
+    int budget = compileOptions_.fusedWeightUpdate > 0 ? 32 : 16;
     std::vector<std::pair<int, int>> byTiles;
+    int allTiles = 0;
     for (size_t i = 0; i < layers_.size(); ++i) {
         const int mt = layers_[i].channelsOut / MATRIX_SIZE, kt = layers_[i].channelsIn / MATRIX_SIZE;
         byTiles.push_back({mt * kt + (layers_[i].useBias ? 1 : 0), static_cast<int>(i)});   // the bias sums share a tile
+        allTiles += byTiles.back().first;
+    }
+    // One wavefront per SIMD has 512 registers, half of them accumulation registers, where gradient tiles that are
+    // only read once at the end of the kernel cost nothing: taken where that fuses *every* layer (no weight-update
+    // kernel and no stored adjoints remain) and 16 tiles did not -- the kernel then runs half as many wavefronts.
+    // Measured, backward + weight updates: 32 -> 64 -> 64 -> 16 (28 tiles) 39 + 25 -> 51 us; forward + backward of
+    // 64 -> 64 -> 64 -> 16 (36 tiles) on 10^6 points 530 -> 505 us. Networks that 16 tiles fuse completely lose
+    // 8-14 % with one wavefront per SIMD, 64 x 4 hidden layers (68 tiles, partly fused) gain nothing.
+    if (wideRegisters) *wideRegisters = false;
+    if (compileOptions_.fusedWeightUpdate < 0 && allTiles > budget && allTiles <= 48) {
+        budget = allTiles;
+        if (wideRegisters) *wideRegisters = true;
     }
     std::sort(byTiles.begin(), byTiles.end());
     int tiles = 0;
@@ -828,7 +842,9 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     std::string code = kl->findFile("qmlp/kernels/network_backward.h").value();
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
-    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", kernelAttributes(blockSize));
+    bool wideRegisters = false;
+    (void)fusedWeightUpdateLayers(flags, sliceGradients, &wideRegisters);
+    replaceAll(code, "$$KERNEL_ATTRIBUTES$$", wideRegisters ? std::string("__attribute__((amdgpu_waves_per_eu(1, 1)))") : kernelAttributes(blockSize));
     // (set below: input gradients that the kernels of the gradient slices compute are none of this kernel's)
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
     replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
@@ -1057,6 +1073,15 @@ std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFl
     if (kind == "forward_registers") return forwardSource(2 * DEFAULT_BLOCK_SIZE, std::min(8, 256 / layers_[0].channelsIn), true);
     if (kind == "backward") return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true));
     if (kind == "weight_update") return weightUpdateSource(weightUpdateBlockSize());
+    if (kind == "backward_resources" || kind == "backward_slices_resources") {
+        // what the loaded backward kernel takes (needs a device): for tests of the register budget
+        const bool slices = kind == "backward_slices_resources";
+        compileBackwardKernel(adjointFlags, slices);
+        const auto& ak = backwardKernel_[adjointFlags][slices ? 1 : 0].value();
+        return format("{\"block\": %d, \"lds_bytes\": %d, \"registers\": %d, \"scratch_bytes\": %d, \"full_grid\": %d}",
+                      ak.adjoint.blockSize, ak.adjoint.sharedMemorySize, ak.adjoint.fun.numVgprs(), ak.adjoint.fun.scratchBytes(),
+                      ak.adjoint.fullGrid);
+    }
     throw std::runtime_error("unknown kernel kind '" + kind + "'");
 }
 

@@ -154,6 +154,12 @@ def test_weight_gradients_summed_in_the_backward_kernel_match_the_weight_update_
         assert ("::template weightGradient<" in src) == (mode != 0)
         flags = FLAG_INPUT | FLAG_WEIGHTS
         got[mode] = case.gpu_train(X, adj, flags)
+        if mode == -1 and widths == [64, 64, 16]:
+            # 27 gradient tiles, the 16 of the 64 x 64 layer among them: all in the accumulation registers of a
+            # kernel that runs one wavefront per SIMD, none of them spilled
+            assert src.count("::template weightGradient<") == 3 and "amdgpu_waves_per_eu(1, 1)" in src
+            res = json.loads(case.net.generated_source("backward_resources", flags))
+            assert res["scratch_bytes"] == 0 and 256 < res["registers"] <= 512 and res["block"] == 256, res
         # (the larger batches only mode against mode, which is the tighter comparison: with gradient entries of order
         # one, sums over tens of thousands of points with ReLU units that an fp16 rounding switches leave the
         # tolerances of the oracle comparison, for the weight-update kernels as for the fused sums)
@@ -747,7 +753,7 @@ def test_full_size_properties_cfg3_train():
                  allowed_fraction=2e-2)
     # At this size the grid gradients are summed by slices and the input gradients come from the records
     # kernel; the same network with the scatter inside the backward kernel (one atomic per contribution):
-    # outputs, input and weight gradients bit for bit, grid gradients up to the order of the fp32 additions.
+    # outputs and input gradients bit for bit, weight and grid gradients up to the order of the fp32 additions.
     cfg = json.loads(json.dumps(bc.CONFIGS[3]["cfg"]))
     cfg.setdefault("options", {})["slice_gradients"] = 0
     scatter = Case(cfg, bc.ORACLE_ACTIVATIONS)
@@ -756,7 +762,10 @@ def test_full_size_properties_cfg3_train():
     c = scatter.gpu_train(X, adj, flags)
     assert np.array_equal(c["out"], a["out"])
     assert np.array_equal(c["adj_x"], a["adj_x"])
-    assert np.array_equal(c["grads"], a["grads"])
+    # (the backward kernel in front of the slice kernels sums the weight gradients of all layers itself, the one that
+    # scatters leaves them to the weight-update kernels: the same products in another order of the fp32 sums)
+    scale = float(np.abs(c["grads"]).max())
+    assert np.allclose(a["grads"] / scale, c["grads"] / scale, rtol=1e-3, atol=1e-5)
     tc = c["table_grads"][0]
     assert_close(ta, tc, "grid gradients by slices against the atomic scatter", rel=1e-3, abs_=1e-5 * float(np.abs(tc).max()))
     assert float(np.abs(tc).max()) > 0

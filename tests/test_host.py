@@ -169,7 +169,10 @@ def test_temporary_memory_sizes():
     n_params = net.num_network_parameters()
     for n, padded, slices in ((1, 64, 1), (64, 64, 1), (65, 128, 1), (1000, 1024, 4), (1 << 18, 1 << 18, 512)):
         assert net.forward_memory(n, 7) == per_fwd * padded
-        assert net.adjoint_memory(n, 2) == per_adj * padded + slices * n_params * 4
+        # weight gradients alone: the backward kernel sums the tiles of all three layers itself (28 tiles in the
+        # accumulation registers of one wavefront per SIMD) and stores no adjoints
+        assert net.adjoint_memory(n, 2) == slices * n_params * 4
+        # a backward kernel that gathers from the grid for the input gradients has no registers for that
         assert net.adjoint_memory(n, 3) == per_adj * padded + slices * n_params * 4
         assert net.adjoint_memory(n, 1) == 0
         if n < (1 << 15):
@@ -186,7 +189,7 @@ def test_temporary_memory_sizes():
     slices_per_level = [-(-f // 8192) for f in floats]
     records = sum(s * (((5 * n * 4 // 4) // s + 2048) & ~3) for s in slices_per_level)
     cursors = -(-(sum(slices_per_level) + 1) * 4 // 256) * 256
-    base = (per_adj + 2 * 32) * n + 512 * n_params * 4
+    base = 2 * 32 * n + 512 * n_params * 4       # (all weight gradients are summed in the backward kernel)
     assert net.adjoint_memory(n, 7) == -(-base // 256) * 256 + cursors + -(-records * 16 // 256) * 256
     assert net.adjoint_memory(n, 4) == 2 * 32 * n + cursors + -(-records * 16 // 256) * 256
     assert net.adjoint_memory((1 << 15) - 64, 5) == 0 and net.adjoint_memory(1 << 15, 5) > 0
@@ -213,13 +216,20 @@ def test_temporary_memory_of_networks_whose_backward_kernel_sums_the_weight_grad
     assert net(small, -1).adjoint_memory(n, 3) == slices * params * 4
     assert "::template weightGradient<" not in net(small, 0).generated_source("backward", 3)
     assert net(small, -1).generated_source("backward", 3).count("::template weightGradient<") == 3
-    mixed = [64, 64, 16]            # 4 + 1, 16 + 1, 4 + 1: the middle layer keeps its weight-update kernel
+    # 4 + 1, 16 + 1, 4 + 1 = 27 tiles: more than the 16 that fit beside two wavefronts per SIMD, so the kernel runs
+    # one wavefront per SIMD with 512 registers and sums all of them
+    mixed = [64, 64, 16]
     params = net(mixed, 0).num_network_parameters()
-    assert net(mixed, -1).adjoint_memory(n, 3) == 2 * (64 + 64 + 16) * n + slices * params * 4
     src = net(mixed, -1).generated_source("backward", 3)
-    assert src.count("::template weightGradient<") == 2 and "Layer1::template weightGradient<" not in src
+    assert src.count("::template weightGradient<") == 3 and "amdgpu_waves_per_eu(1, 1)" in src
+    assert net(mixed, -1).adjoint_memory(n, 3) == slices * params * 4
+    assert "amdgpu_waves_per_eu(1, 1)" not in net(small, -1).generated_source("backward", 3)
     assert net(mixed, 1).generated_source("backward", 3).count("::template weightGradient<") == 3   # 27 tiles <= 32
+    assert "amdgpu_waves_per_eu(1, 1)" not in net(mixed, 1).generated_source("backward", 3)
     assert net(mixed, 1).adjoint_memory(n, 3) == slices * params * 4
+    # 61 tiles, and weights that call for workgroups of 8 wavefronts (128 registers each): nothing is summed in the kernel
+    deep = net([64, 64, 64, 64, 16], -1).generated_source("backward", 3)
+    assert "amdgpu_waves_per_eu(1, 1)" not in deep and "::template weightGradient<" not in deep
     # without weight gradients nothing changes
     assert "::template weightGradient<" not in net(small, -1).generated_source("backward", 1)
 
