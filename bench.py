@@ -293,10 +293,49 @@ def layer_gemm_report(device, steps, warmup, only="", n=1 << 20):
     return out
 
 
+def torch_baseline(width, widths, n, device, half, trials=10, startup=2):
+    """The reference's own comparison on the same device (tests_py/qmlp_tests/profile_network.py:27-60,
+    149-177): a stack of torch.nn.Linear layers without bias, ReLU between them, in fp32 or (input cast to half,
+    output cast back) in fp16; wall clock of a call between two synchronisations, 10 trials of which the first
+    two are dropped; inference under no_grad, then forward + backward with the gradient of the input."""
+    import numpy as np
+    import torch
+    layers, last = [], width
+    for i, w in enumerate(widths):
+        layers.append(torch.nn.Linear(last, w, bias=False))
+        if i + 1 < len(widths):
+            layers.append(torch.nn.ReLU())
+        last = w
+    net = torch.nn.Sequential(*layers).to(device)
+    if half:
+        net = net.half()
+    run = (lambda x: net(x.half()).float()) if half else net
+    x = torch.randn((n, width), device=device, dtype=torch.float32, requires_grad=True)
+    grad_out = torch.randn((n, widths[-1]), device=device, dtype=torch.float32)
+    times = [[], []]
+    with torch.no_grad():
+        for _ in range(trials):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            run(x)
+            torch.cuda.synchronize()
+            times[0].append(time.perf_counter() - t0)
+    for _ in range(trials):
+        x.grad = None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = run(x)
+        torch.autograd.backward(out, grad_out)
+        torch.cuda.synchronize()
+        times[1].append(time.perf_counter() - t0)
+    return [1e3 * float(np.mean(t[startup:])) for t in times]
+
+
 def reference_grid(device, steps, warmup, only=""):
     """The benchmark grid of the reference (tests_py/qmlp_tests/profile_network.py:107-190):
     10^6 points, 2 or 4 hidden layers of 16, 32 or 64 neurons (as many inputs), ReLU, 4 outputs,
-    no bias, identity encoding; inference and forward + backward (input and weight gradients)."""
+    no bias, identity encoding; inference and forward + backward (input and weight gradients), next to the
+    PyTorch-32 and PyTorch-16 networks that the reference times beside its own."""
     n = 1000 * 1000
     rows = []
     for width, widths in REFERENCE_GRID:
@@ -305,7 +344,11 @@ def reference_grid(device, steps, warmup, only=""):
             inf_ms, inf_wall = run_mlp(width, widths, n, device, steps, warmup)
             trn_ms, trn_wall = run_mlp(width, widths, n, device, max(3, steps // 2), min(warmup, 3), train=True)
             flop = mlp_flops(width, widths, False)
+            t32, t16 = torch_baseline(width, widths, n, device, False), torch_baseline(width, widths, n, device, True)
             rows.append({"network": "%d x %d" % (width, hidden), "points": n,
+                         # stated baselines on the same device, not targets: torch.nn.Linear stacks, wall clock per call
+                         "torch_fp32_inference_ms": t32[0], "torch_fp32_forward_backward_ms": t32[1],
+                         "torch_fp16_inference_ms": t16[0], "torch_fp16_forward_backward_ms": t16[1],
                          "inference_ms": inf_ms, "inference_wall_ms": inf_wall,
                          "forward_backward_ms": trn_ms, "forward_backward_wall_ms": trn_wall,
                          "inference_mfma_frac": flop * n / (inf_ms * 1e-3) / 1e12 / MFMA_FP16_PEAK_TFLOPS,

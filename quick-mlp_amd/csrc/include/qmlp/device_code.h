@@ -20,4 +20,12 @@ int fillAsync(void* ptr, int value, size_t bytes, void* stream, std::string& err
  */
 int staticScratch(void** ptr, size_t* bytes, std::string& error);
 
+/**
+ * Notes that work on `stream` is about to use the static scratch buffer of the current device. All calls on a
+ * device share the buffer: a call on another stream than the last one is accepted only if that stream's work has
+ * finished (and this stream is not being captured, when other streams may not be asked). Allocates nothing.
+ * Returns 0 or sets `error`.
+ */
+int claimStaticScratch(void* stream, std::string& error);
+
 }} // namespace qmlp::device_code

@@ -32,7 +32,9 @@
 // largest adjoint of the batch (which the records kernel finds on its way) and the number of
 // records, such that no sum can overflow: at least 37 bits remain below the largest possible
 // contribution at 2^24 records, and the sums do not depend on the order of the additions. Batches whose
-// adjoints are not finite take the float additions, so that NaN and infinity reach the gradients.
+// adjoints are not finite take the float additions, so that NaN and infinity reach the gradients. Weights
+// are at most one for points inside the box; the records of points outside of it (extrapolated with weights
+// beyond one, or NaN for a NaN coordinate) are added to the gradient tensor by the records kernel itself.
 // Two forms that were measured and dropped: a workgroup per slice that tests every point of
 // the batch against its slice and recomputes the hits (the work of a hit falls to one lane of
 // 64, 890 us for 2^18 points and 16 levels), and the same with the hits queued in LDS first (the
@@ -263,7 +265,7 @@ struct GridGradientRecords
     struct AddToTensor
     {
         float* __restrict__ gradients;
-        __device__ __forceinline__ void operator()(unsigned element, float weight, const unsigned (&adjWords)[(F + 1) / 2]) const
+        __device__ __forceinline__ void operator()(unsigned element, float weight, const unsigned (&adjWords)[(F + 1) / 2], bool /*upper*/) const
         {
 #pragma unroll
             for (int i = 0; i < F; ++i) {
@@ -276,9 +278,10 @@ struct GridGradientRecords
     /**
      * The record of pair c of a point in one level: the offsets of its two entries within the slice of the lower
      * one, their weights and the adjoint words. Returns the slice (= bucket within the level) that files it.
-     * \param otherSlice called with (element of feature 0 in the table, weight, adjWords) for an upper entry that
+     * \param otherSlice called with (element of feature 0 in the table, weight, adjWords, whether it is the upper entry of the pair) for an upper entry that
      *    lies in another slice (an entry next to a slice boundary; in a hashed level one pair in thousands): the
-     *    record then keeps the lower entry only
+     *    record then keeps the lower entry only; and for both entries of a pair whose weights exceed one in
+     *    magnitude or are not finite (points outside the box): the record then adds nothing
      */
     template <int LEVEL, typename OtherSlice>
     __device__ __forceinline__ static int buildRecord(const typename Grid::LevelSetup& s, int c,
@@ -295,13 +298,27 @@ struct GridGradientRecords
         const unsigned eL = idxL * F - sliceStart;
         unsigned eH = idxH * F - sliceStart;                     // wraps if the upper entry lies below the slice
         float wH = w * s.f[PD];
+        float wL = w * (1.f - s.f[PD]);
+        bool upperAdded = false;
         if (eH >= static_cast<unsigned>(SLICE_FLOATS)) {
-            otherSlice(base + idxH * F, wH, adjWords);
+            otherSlice(base + idxH * F, wH, adjWords, true);
             eH = eL;
             wH = 0.f;
+            upperAdded = true;
+        }
+        // The sums of the slice kernel are fixed point with a scale that counts on weights of at most one, which
+        // holds for every point inside the box. A point outside of it is extrapolated (the fractional position is
+        // not clamped) with weights that grow with its distance, a NaN coordinate gives NaN weights: such records
+        // go the way of the entries of other slices, and add nothing to the sums.
+        if (!(fabsf(wL) <= 1.f && fabsf(wH) <= 1.f)) {
+            otherSlice(base + idxL * F, wL, adjWords, false);
+            if (!upperAdded) otherSlice(base + idxH * F, wH, adjWords, true);
+            wL = 0.f;
+            wH = 0.f;
+            eH = eL;
         }
         rec[0] = eL | (eH << 16);
-        rec[1] = __builtin_bit_cast(unsigned, w * (1.f - s.f[PD]));
+        rec[1] = __builtin_bit_cast(unsigned, wL);
         rec[2] = __builtin_bit_cast(unsigned, wH);
 #pragma unroll
         for (int i = 0; i < (F + 1) / 2; ++i) rec[3 + i] = adjWords[i];
@@ -580,17 +597,21 @@ struct GridGradientTraceLevels
 #pragma unroll
             for (int c = 0; c < Impl::PAIRS; ++c) {
                 unsigned rec[Impl::RW];
-                unsigned otherElement = 0u;
-                float otherWeight = 0.f;
-                bool other = false;
+                unsigned otherElement[2] = {0u, 0u};
+                float otherWeight[2] = {0.f, 0.f};
+                bool other[2] = {false, false};
                 const int bucket = Impl::template buildRecord<LEVEL>(s, c, adjWords, rec,
-                    [&](unsigned element, float weight, const Words&) { other = true; otherElement = element; otherWeight = weight; });
+                    [&](unsigned element, float weight, const Words&, bool upper) {
+                        other[upper] = true;
+                        otherElement[upper] = element;
+                        otherWeight[upper] = weight;
+                    });
                 const unsigned sliceStart = static_cast<unsigned>(Cfg::memoryOffset[LEVEL]) + static_cast<unsigned>(bucket) * SLICE_FLOATS;
-                idx[LEVEL * NC + 2 * c] = sliceStart + (rec[0] & 0xffffu);
-                w[LEVEL * NC + 2 * c] = __builtin_bit_cast(float, rec[1]);
+                idx[LEVEL * NC + 2 * c] = other[0] ? otherElement[0] : sliceStart + (rec[0] & 0xffffu);
+                w[LEVEL * NC + 2 * c] = other[0] ? otherWeight[0] : __builtin_bit_cast(float, rec[1]);
                 if (NC > 1) {
-                    idx[LEVEL * NC + 2 * c + 1] = other ? otherElement : sliceStart + (rec[0] >> 16);
-                    w[LEVEL * NC + 2 * c + 1] = other ? otherWeight : __builtin_bit_cast(float, rec[2]);
+                    idx[LEVEL * NC + 2 * c + 1] = other[1] ? otherElement[1] : sliceStart + (rec[0] >> 16);
+                    w[LEVEL * NC + 2 * c + 1] = other[1] ? otherWeight[1] : __builtin_bit_cast(float, rec[2]);
                 }
             }
             GridGradientTraceLevels<Cfg, SLICE_FLOATS, LEVEL + 1>::run(pos, adjWords, idx, w);

@@ -21,6 +21,8 @@ static __device__ __align__(256) unsigned char scratch[QMLP_STATIC_SCRATCH_BYTES
 
 constexpr int MAX_DEVICES = 64;
 void* g_scratchAddress[MAX_DEVICES] = {};   // per device: where that device holds its copy
+hipStream_t g_scratchStream[MAX_DEVICES] = {};   // per device: the stream of the last call that used it
+bool g_scratchUsed[MAX_DEVICES] = {};
 std::mutex g_scratchMutex;
 
 __global__ void __launch_bounds__(256) FillBytesKernel(unsigned char* __restrict__ p, unsigned char value, size_t bytes)
@@ -54,9 +56,13 @@ int fillAsync(void* ptr, int value, size_t bytes, void* stream, std::string& err
     if (bytes == 0) return 0;
     const size_t blocks = (bytes / 16 + 255) / 256 + 1;
     const unsigned grid = static_cast<unsigned>(blocks < 4096 ? blocks : 4096);
-    hipLaunchKernelGGL(FillBytesKernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<unsigned char*>(ptr), static_cast<unsigned char>(value), bytes);
-    const hipError_t e = hipGetLastError();
+    // launched through the call that returns this launch's own status: hipGetLastError() would also report (and
+    // clear) an error that another library left on this thread, e.g. hipErrorNotReady of an event query
+    unsigned char* p = static_cast<unsigned char*>(ptr);
+    unsigned char v = static_cast<unsigned char>(value);
+    void* args[] = {&p, &v, &bytes};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(FillBytesKernel), dim3(grid), dim3(256), args, 0,
+                                         static_cast<hipStream_t>(stream));
     if (e != hipSuccess) {
         error = describe(e, "launch of the fill kernel");
         return 1;
@@ -90,6 +96,36 @@ int staticScratch(void** ptr, size_t* bytes, std::string& error)
         g_scratchAddress[device] = address;
     }
     *ptr = g_scratchAddress[device];
+    return 0;
+}
+
+int claimStaticScratch(void* stream, std::string& error)
+{
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess || device < 0 || device >= MAX_DEVICES) {
+        error = describe(e, "hipGetDevice");
+        return 1;
+    }
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if (g_scratchUsed[device] && g_scratchStream[device] != s) {
+        // Work of another stream may still read or write the buffer. While this stream is being captured nothing
+        // may be asked of other streams; otherwise the other stream says whether it is done (a stream that its
+        // owner has destroyed meanwhile reports an error, which means that its work is over).
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capture) != hipSuccess) (void)hipGetLastError();
+        const bool busy = capture != hipStreamCaptureStatusNone || hipStreamQuery(g_scratchStream[device]) == hipErrorNotReady;
+        (void)hipGetLastError();   // a not-ready or invalid-handle answer is no error of this call
+        if (busy) {
+            error = "the static workspace of the call that allocates nothing was last used on another stream whose work has "
+                    "not finished (or this stream is being captured): calls that share it on one device must follow each "
+                    "other on one stream, or be synchronised by the caller";
+            return 1;
+        }
+    }
+    g_scratchUsed[device] = true;
+    g_scratchStream[device] = s;
     return 0;
 }
 

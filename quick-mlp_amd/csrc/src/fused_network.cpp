@@ -644,13 +644,20 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
     // kernel and no stored adjoints remain) and 16 tiles did not -- the kernel then runs half as many wavefronts.
     // Measured, backward + weight updates: 32 -> 64 -> 64 -> 16 (28 tiles) 39 + 25 -> 51 us; forward + backward of
     // 64 -> 64 -> 64 -> 16 (36 tiles) on 10^6 points 530 -> 505 us. Networks that 16 tiles fuse completely lose
-    // 8-14 % with one wavefront per SIMD, 64 x 4 hidden layers (68 tiles, partly fused) gain nothing.
+    // 8-14 % with one wavefront per SIMD, 64 x 4 hidden layers (68 tiles, partly fused) gain nothing, and where 16
+    // tiles leave out only a small layer (32 x 4 hidden layers: 16 of 18 tiles) the smaller kernel stays ahead
+    // (forward + backward 300 against 317 us).
+    std::sort(byTiles.begin(), byTiles.end());
+    int within = 0;
+    for (const auto& [count, layer] : byTiles) {
+        if (within + count > budget) break;
+        within += count;
+    }
     if (wideRegisters) *wideRegisters = false;
-    if (compileOptions_.fusedWeightUpdate < 0 && allTiles > budget && allTiles <= 48) {
+    if (compileOptions_.fusedWeightUpdate < 0 && allTiles <= 48 && allTiles - within >= 12) {
         budget = allTiles;
         if (wideRegisters) *wideRegisters = true;
     }
-    std::sort(byTiles.begin(), byTiles.end());
     int tiles = 0;
     for (const auto& [count, layer] : byTiles) {
         if (tiles + count > budget) break;
@@ -1599,6 +1606,8 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
         compileBackwardKernel(adjointFlags, sliceGradients);
         for (auto& sk : backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value().sliceGradients)
             (void)recordsKernelFor(sk, adjointFlags, numel);
+        // the streams and events on which the weight-update kernels of the layers run side by side
+        if ((adjointFlags & GRADIENTS_NETWORK_WEIGHTS) && compileOptions_.parallelWeightUpdate && layers_.size() > 1) ensureStreams();
     }
 }
 
@@ -1647,6 +1656,7 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
                 static_cast<long long>(scratchBytes),
                 // per point: its row, its index and its share of the histogram of its chunk
                 static_cast<long long>((scratchBytes / sizeof(float) - 2.0 * SLABS) / (channels + 1 + static_cast<double>(SLABS) / CHUNK))));
+        if (device_code::claimStaticScratch(stream, error) != 0) throw std::runtime_error(error);
         totals = static_cast<int*>(scratch);
     } else {
         if (po.capacityWords < words) {

@@ -10,9 +10,10 @@ import numpy as np
 import pytest
 import torch
 
+import qmlp
 import qmlp_oracle as qo
 from helpers import (ABS, REL, Case, FLAG_ENC, FLAG_INPUT, FLAG_WEIGHTS, assert_close, baseline_case,
-                     check_gradients, identity_cfg, random_parameters, require_gpu)
+                     check_gradients, identity_cfg, random_parameters, require_gpu, warm_cache)
 import baseline_configs as bc
 
 pytestmark = pytest.mark.gpu
@@ -502,6 +503,7 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
             "network": [{"n_out": 32, "bias": True, "activation": "celu"},
                         {"n_out": 2, "bias": False, "activation": "identity"}]}
     cases = {}
+    warm_cache(*[dict(base, options={"slice_gradients": mode}) for mode in (0, 1)])
     for mode in (0, 1):
         cfg = json.loads(json.dumps(base))
         cfg["options"] = {"slice_gradients": mode}
@@ -534,6 +536,43 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
                 assert np.array_equal(got[0]["adj_x"], got[1]["adj_x"])
             # (weight and input gradients are those of the other mode bit for bit: checked against the oracle elsewhere)
             check_gradients(cases[1], X, adj, FLAG_ENC, got[1], what="slices, N=%d flags=%d: " % (N, flags))
+    # Points several box widths outside are extrapolated with weights far above one (the reference does not clamp the
+    # fractional position either; 3 widths outside a level of resolution 128: |w| up to 5e7 in 3-D), while the
+    # fixed-point sums of the slice kernel count on weights of at most one: the records kernel adds such records to
+    # the gradient tensor itself. The corners of such a point coincide at the border of the grid, so an entry
+    # receives huge terms of both signs that cancel to the adjoint itself, and float additions leave rounding noise
+    # of the size of |w| x 2^-24 x |adjoint| there in either mode: the entries that these points touch stay at that
+    # level, all other entries agree as usual. A NaN coordinate gives NaN weights: the gradients of the entries it
+    # touches are NaN in both modes.
+    N = 70001
+    X = (lo + sz * rng.uniform(0, 1, (N, n_in))).astype(np.float32)
+    far = np.arange(7, N, 1000)
+    X[far] = (lo + sz * rng.uniform(-3.0, 4.0, (len(far), n_in))).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+    probe = qmlp.Encoding(json.dumps(grid))
+    probe.set_parameter(torch.zeros(probe.num_parameters(), device="cuda", dtype=probe.parameter_dtype()))
+    far_idx, far_w = probe.hashgrid_corners(torch.from_numpy(X[far]).cuda())
+    touched = np.zeros(probe.num_parameters(), bool)
+    for f in range(spec["n_features_per_level"]):
+        touched[far_idx.cpu().numpy().astype(np.int64).ravel() + f] = True
+    largest = float(far_w.abs().max())
+    assert largest > 100
+    got = {mode: c.gpu_train(X, adj, FLAG_ENC) for mode, c in cases.items()}
+    a, b = got[0]["table_grads"][1], got[1]["table_grads"][1]
+    assert np.isfinite(a).all() and np.isfinite(b).all()
+    scale = float(np.abs(a[~touched]).max())
+    assert scale > 0 and np.allclose(a[~touched] / scale, b[~touched] / scale, rtol=1e-4, atol=2e-6)
+    noise = 1.0 + len(far) * largest * 2.0 ** -20          # adjoints of the encoded features are below one
+    assert np.abs(a[touched]).max() < noise and np.abs(b[touched]).max() < noise, (np.abs(a[touched]).max(), np.abs(b[touched]).max())
+    X = (lo + sz * rng.uniform(0, 1, (N, n_in))).astype(np.float32)
+    X[5, 1] = np.nan
+    got = {mode: c.gpu_train(X, adj, FLAG_ENC) for mode, c in cases.items()}
+    a, b = got[0]["table_grads"][1], got[1]["table_grads"][1]
+    assert np.isnan(a).any() and np.array_equal(np.isnan(a), np.isnan(b))
+    ok = ~np.isnan(a)
+    scale = float(np.abs(a[ok]).max())
+    assert np.allclose(a[ok] / scale, b[ok] / scale, rtol=1e-4, atol=2e-6)
+    X[5, 1] = lo[1]
     # gradients are accumulated: a second call onto the same tensor doubles them
     x, a = torch.from_numpy(X).cuda(), torch.from_numpy(adj).cuda()
     c = cases[1]
