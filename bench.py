@@ -33,7 +33,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 # code: "kernels" is device_code_hash() at the time of the counter runs, and a workload whose
 # device code has changed since (or that has no counter run) reports traffic null.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2-inference": {"points": 1 << 20, "fetch": 105187.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
+    "cfg2-inference": {"points": 1 << 20, "fetch": 105169.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
                        "kernels": "4ad4add129c4ab5d"},
 }
 
@@ -134,6 +134,43 @@ def run_inference(case, steps, warmup):
     step()   # compiles (or loads from the kernel cache) outside of any timing
     torch.cuda.synchronize()
     return time_steps(step, steps, warmup)
+
+
+def ordered_batch_report(cfg_id, n, device, steps, warmup):
+    """The inference launch of a hash-grid network on the same batch in three orders: as given; ordered by the
+    library in front of the kernel (options.sort_points = 1: slabs of the grid's second and third coordinate,
+    the sort inside the timed step); and arriving in that order (sorted beforehand with torch, nothing for the
+    library to do: what a caller with coherent batches, e.g. rays of an image tile, gets)."""
+    import torch
+    import baseline_configs as bc
+    base = bc.CONFIGS[cfg_id]["cfg"]
+    out = {}
+    results = {}
+    try:
+        for name, mode in (("as_given", 0), ("sorted_by_the_library", 1), ("arrives_in_slab_order", 0)):
+            bc.CONFIGS[cfg_id]["cfg"] = json.loads(json.dumps(base))
+            bc.CONFIGS[cfg_id]["cfg"].setdefault("options", {})["sort_points"] = mode
+            case = build_case(cfg_id, n, device)
+            if name == "arrives_in_slab_order":
+                x = case["x"]
+                q = (x.clamp(0, 1 - 1e-7) * 32).long()
+                key = torch.zeros_like(q[:, 0])
+                for b in range(5):
+                    key |= ((q[:, 1] >> b) & 1) << (2 * b + 1) | ((q[:, 2] >> b) & 1) << (2 * b)
+                order = torch.argsort(key * n + torch.randperm(n, device=device))
+                case["x"] = x[order].contiguous()
+                results[name] = (case["net"].inference(case["x"], case["params"], case["enc_params"]), order)
+            else:
+                results[name] = (case["net"].inference(case["x"], case["params"], case["enc_params"]), None)
+            elapsed, launch_ms = run_inference(case, steps, warmup)
+            out[name] = {"ms_per_step": 1e3 * elapsed / steps, "launch_ms": launch_ms}
+            del case
+    finally:
+        bc.CONFIGS[cfg_id]["cfg"] = base
+    ref = results["as_given"][0]
+    out["same_bits"] = bool(torch.equal(ref, results["sorted_by_the_library"][0])
+                            and torch.equal(ref[results["arrives_in_slab_order"][1]], results["arrives_in_slab_order"][0]))
+    return out
 
 
 def run_train(case, steps, warmup, input_gradients=True, warmup_seconds=0.0):
@@ -436,6 +473,105 @@ def gather_ceiling(device, repeats=5):
     return result
 
 
+PATTERN_SOURCE = r"""
+#include <hip/hip_runtime.h>
+// What one gather instruction of a wavefront costs, by the cache lines its 64 lanes ask for. Every lane has a line
+// number and a word in that line that stay fixed over the loop; every iteration adds an offset that is the same for
+// the whole wavefront (so the per-load arithmetic is three vector instructions), eight loads are in flight per lane.
+__device__ __forceinline__ unsigned mix(unsigned x)
+{
+    x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+    return x;
+}
+template <int W>
+__device__ void body(const unsigned* __restrict__ table, unsigned lineMask, const unsigned* __restrict__ laneLine,
+                     const unsigned* __restrict__ laneWord, float* out, int iters)
+{
+    const unsigned gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned lane = threadIdx.x & 63;
+    const unsigned myLine = laneLine[lane], myWord = laneWord[lane];
+    unsigned acc = 0, h = mix(gid >> 6);
+    typedef unsigned vec __attribute__((ext_vector_type(W)));
+    for (int it = 0; it < iters; it += 8) {
+        vec v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            h = h * 1664525u + 1013904223u;
+            const unsigned line = (myLine + (h >> 8)) & lineMask;
+            v[j] = *reinterpret_cast<const vec*>(table + line * 32u + myWord);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            for (int w = 0; w < W; ++w) acc += v[j][w];
+    }
+    if (acc == 0x12345678u) out[gid] = 1.f;
+}
+extern "C" __global__ void __launch_bounds__(256) GatherPattern4(const unsigned* t, unsigned m, const unsigned* l, const unsigned* w, float* o, int n) { body<1>(t, m, l, w, o, n); }
+extern "C" __global__ void __launch_bounds__(256) GatherPattern8(const unsigned* t, unsigned m, const unsigned* l, const unsigned* w, float* o, int n) { body<2>(t, m, l, w, o, n); }
+"""
+
+
+def gather_patterns(device, repeats=3):
+    """Cycles of one compute unit per gather instruction of a wavefront, by the number of distinct 128-byte lines its
+    lanes ask for (1, 16 or 64), by how the lanes that share a line are placed (neighbours or spread), and by
+    whether the lines are found in the L1 (a region of 8 KiB) or come from the L2 (a region of 2 MiB, which is
+    the table of one level of the hash grid). The clock is taken as 2.4 GHz."""
+    import ctypes
+    import numpy as np
+    import torch
+    import qmlp
+    lib = qmlp._lib.lib
+    lib.qmlp_hip_last_error.restype = ctypes.c_char_p
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(lib.qmlp_hip_last_error().decode())
+
+    kernels = [b"GatherPattern4", b"GatherPattern8"]
+    module = ctypes.c_void_p()
+    names = (ctypes.c_char_p * len(kernels))(*kernels)
+    opts = (ctypes.c_char_p * 6)(b"-O3", b"-I/opt/rocm/include", b"-Xclang", b"-target-feature", b"-Xclang", b"-packed-fp32-ops")
+    ok(lib.qmlp_hip_module_compile(PATTERN_SOURCE.encode(), b"gather_patterns.hip", None, None, 0, names, len(kernels), opts, 6,
+                                   None, ctypes.byref(module), None))
+    ok(lib.qmlp_hip_module_load(module))
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    blocks, threads, iters = 8 * cus, 256, 512
+    table = torch.ones((4 << 20) // 4, dtype=torch.int32, device=device)
+    out = torch.zeros(blocks * threads, dtype=torch.float32, device=device)
+    stream = qmlp._lib.current_stream(device)
+    rng = np.random.default_rng(1)
+    rows = []
+    for kernel, width in zip(kernels, (1, 2)):
+        fn, lowered = ctypes.c_void_p(), ctypes.c_char_p()
+        ok(lib.qmlp_hip_module_lowered_name(module, kernel, ctypes.byref(lowered)))
+        ok(lib.qmlp_hip_module_get_function(module, lowered, ctypes.byref(fn)))
+        for region in (8 << 10, 2 << 20):
+            for lines, placement in ((1, "neighbours"), (16, "neighbours"), (16, "spread"), (64, "neighbours")):
+                lane = np.arange(64)
+                line = (lane // (64 // lines) if placement == "neighbours" else lane % lines) * 7919
+                word = rng.integers(0, 32 // width, 64) * width
+                d_line = torch.from_numpy(line.astype(np.int32)).to(device)
+                d_word = torch.from_numpy(word.astype(np.int32)).to(device)
+                a = [ctypes.c_void_p(table.data_ptr()), ctypes.c_uint32(region // 128 - 1), ctypes.c_void_p(d_line.data_ptr()),
+                     ctypes.c_void_p(d_word.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_int(iters)]
+                args = (ctypes.c_void_p * len(a))(*[ctypes.addressof(v) for v in a])
+                ok(lib.qmlp_hip_launch(fn, blocks, threads, 0, stream, args))
+                torch.cuda.synchronize()
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(repeats):
+                    ok(lib.qmlp_hip_launch(fn, blocks, threads, 0, stream, args))
+                stop.record()
+                torch.cuda.synchronize()
+                ms = start.elapsed_time(stop) / repeats
+                instructions_per_cu = blocks * threads / 64 * iters / cus
+                rows.append({"bytes_per_lane": 4 * width, "region_bytes": region, "lines_per_instruction": lines,
+                             "lanes_of_a_line": placement, "launch_ms": ms,
+                             "clocks_per_instruction_and_cu": ms * 1e-3 * 2.4e9 / instructions_per_cu})
+    ok(lib.qmlp_hip_module_destroy(module))
+    return rows
+
+
 LDS_SOURCE = r"""
 #include <hip/hip_runtime.h>
 // Reference patterns for reading the LDS bank-conflict counter: every kernel issues the same number
@@ -537,7 +673,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2-inference",
-                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "lds-calibration", "all"],
+                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "gather-patterns", "lds-calibration", "all"],
                     help="layer-gemm: the layers of the hash-grid network on their own; reference-grid: the reference's "
                          "own benchmark networks; gather-ceiling: request rate of random gathers; all: every workload")
     ap.add_argument("--points", type=int, default=0, help="override the number of points")
@@ -545,6 +681,7 @@ def main():
                                                "(e.g. cfg2_mlp_cached_input, '64 x 4')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the secondary train-step measurement")
+    ap.add_argument("--no-ordered", action="store_true", help="skip the secondary measurements on ordered batches")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (reference kernel for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -593,6 +730,11 @@ def main():
         print(json.dumps(dict(head, value=g["l2_hit"]["requests_per_s"], unit="line requests/s",
                               ms_per_step=g["l2_hit"]["launch_ms"],
                               config={"workload": "gather-ceiling", "loads": 2048 * 256 * 64}, gather=g)))
+        return
+    if args.workload == "gather-patterns":
+        rows = gather_patterns(device)
+        print(json.dumps(dict(head, value=1.0 / (rows[0]["launch_ms"] * 1e-3), unit="launches/s", ms_per_step=rows[0]["launch_ms"],
+                              config={"workload": "gather-patterns"}, patterns=rows)))
         return
     if args.workload == "lds-calibration":
         r = lds_calibration(device)
@@ -663,6 +805,9 @@ def main():
         # (the duration of the kernel as a profiler's kernel trace sees it: launches back to back)
         result["mfma"]["layer_gemm_frac"] = result["mfma"]["layer_gemm"]["cfg2_mlp_cached_input"]["frac_back_to_back"]
         result["roofline"]["request_ceiling"] = request_ceiling(gather_ceiling(device), n, 64.0, 0.03, launch_ms)
+    if not train and cfg_id == 2 and not args.no_ordered:
+        # the same launch on a batch that the library orders first, and on one that arrives ordered
+        result["ordered_batch"] = ordered_batch_report(cfg_id, n, device, max(10, args.steps // 2), args.warmup)
     if not train and cfg_id == 2 and not args.no_train:
         # the train step of the same network at its own batch size
         c3 = bc.CONFIGS[3]
