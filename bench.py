@@ -572,6 +572,102 @@ def gather_patterns(device, repeats=3):
     return rows
 
 
+OVERLAP_SOURCE = r"""
+#include <hip/hip_runtime.h>
+// Do the matrix cores and the vector ALUs of a SIMD work side by side? Per iteration 32 matrix instructions on
+// 8 independent accumulator tiles (MODE & 1) and 320 packed fp16 vector instructions on 16 independent registers
+// (MODE & 2); nothing one stream computes is used by the other.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <int MODE>
+__device__ void body(float* out, int iters)
+{
+    f16x8 a, b;
+    for (int i = 0; i < 8; ++i) { a[i] = (_Float16)(threadIdx.x * 0.001f + i); b[i] = (_Float16)(threadIdx.x * 0.002f - i); }
+    f32x4 acc[8];
+    for (int i = 0; i < 8; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f16x2 v[16];
+    for (int i = 0; i < 16; ++i) { v[i][0] = (_Float16)(threadIdx.x + i); v[i][1] = (_Float16)(i); }
+    const f16x2 lim = {(_Float16)0.5f, (_Float16)0.25f};
+    for (int it = 0; it < iters; ++it) {
+        if (MODE & 1) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[i], 0, 0, 0);
+        }
+        if (MODE & 2) {
+#pragma unroll
+            for (int r = 0; r < 10; ++r)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[i] = __builtin_elementwise_max(v[i] + lim, lim);
+        }
+    }
+    float s = 0.f;
+    for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][3];
+    for (int i = 0; i < 16; ++i) s += (float)v[i][0] + (float)v[i][1];
+    if (s == 12345.678f) out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+extern "C" __global__ void __launch_bounds__(256) OverlapMatrix(float* out, int iters) { body<1>(out, iters); }
+extern "C" __global__ void __launch_bounds__(256) OverlapVector(float* out, int iters) { body<2>(out, iters); }
+extern "C" __global__ void __launch_bounds__(256) OverlapBoth(float* out, int iters) { body<3>(out, iters); }
+"""
+
+
+def mfma_valu_overlap(device, iters=2000):
+    """Cycles per v_mfma_f32_16x16x32_f16 and per packed vector instruction of a SIMD that runs only the one or the
+    other, and the time of both streams together against their sum: what a layer of the fused kernels, whose matrix
+    results pass through conversions and activations on the vector ALUs, can at best overlap. 4 wavefronts per SIMD."""
+    import ctypes
+    import torch
+    import qmlp
+    lib = qmlp._lib.lib
+    lib.qmlp_hip_last_error.restype = ctypes.c_char_p
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(lib.qmlp_hip_last_error().decode())
+
+    kernels = [b"OverlapMatrix", b"OverlapVector", b"OverlapBoth"]
+    module = ctypes.c_void_p()
+    names = (ctypes.c_char_p * len(kernels))(*kernels)
+    opts = (ctypes.c_char_p * 6)(b"-O3", b"-I/opt/rocm/include", b"-Xclang", b"-target-feature", b"-Xclang", b"-packed-fp32-ops")
+    ok(lib.qmlp_hip_module_compile(OVERLAP_SOURCE.encode(), b"mfma_valu_overlap.hip", None, None, 0, names, len(kernels), opts, 6,
+                                   None, ctypes.byref(module), None))
+    ok(lib.qmlp_hip_module_load(module))
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    waves_per_simd = 4
+    blocks = cus * waves_per_simd
+    out = torch.zeros(blocks * 256, dtype=torch.float32, device=device)
+    stream = qmlp._lib.current_stream(device)
+    ms = {}
+    for name in kernels:
+        fn, lowered = ctypes.c_void_p(), ctypes.c_char_p()
+        ok(lib.qmlp_hip_module_lowered_name(module, name, ctypes.byref(lowered)))
+        ok(lib.qmlp_hip_module_get_function(module, lowered, ctypes.byref(fn)))
+        a_out, a_iters = ctypes.c_void_p(out.data_ptr()), ctypes.c_int(iters)
+        args = (ctypes.c_void_p * 2)(ctypes.addressof(a_out), ctypes.addressof(a_iters))
+        ok(lib.qmlp_hip_launch(fn, blocks, 256, 0, stream, args))
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        ok(lib.qmlp_hip_launch(fn, blocks, 256, 0, stream, args))
+        stop.record()
+        torch.cuda.synchronize()
+        ms[name.decode()] = start.elapsed_time(stop)
+    ok(lib.qmlp_hip_module_destroy(module))
+    per_simd = lambda t, n: t * 1e-3 * 2.4e9 / iters / waves_per_simd / n
+    return {"waves_per_simd": waves_per_simd, "launch_ms": ms,
+            "clocks_per_mfma_16x16x32_f16": per_simd(ms["OverlapMatrix"], 32),
+            "clocks_per_packed_valu": per_simd(ms["OverlapVector"], 320),
+            "both_over_sum": ms["OverlapBoth"] / (ms["OverlapMatrix"] + ms["OverlapVector"]),
+            "both_over_larger": ms["OverlapBoth"] / max(ms["OverlapMatrix"], ms["OverlapVector"]),
+            # what the matrix cores of the device deliver with this instruction when nothing else runs
+            "mfma_only_tflops": 16384.0 * 32 * iters * blocks * 4 / (ms["OverlapMatrix"] * 1e-3) / 1e12,
+            "clock_hz_assumed": 2.4e9}
+
+
 LDS_SOURCE = r"""
 #include <hip/hip_runtime.h>
 // Reference patterns for reading the LDS bank-conflict counter: every kernel issues the same number
@@ -673,7 +769,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2-inference",
-                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "gather-patterns", "lds-calibration", "all"],
+                    choices=sorted(WORKLOADS) + ["layer-gemm", "reference-grid", "gather-ceiling", "gather-patterns", "mfma-valu-overlap",
+                                              "lds-calibration", "all"],
                     help="layer-gemm: the layers of the hash-grid network on their own; reference-grid: the reference's "
                          "own benchmark networks; gather-ceiling: request rate of random gathers; all: every workload")
     ap.add_argument("--points", type=int, default=0, help="override the number of points")
@@ -735,6 +832,11 @@ def main():
         rows = gather_patterns(device)
         print(json.dumps(dict(head, value=1.0 / (rows[0]["launch_ms"] * 1e-3), unit="launches/s", ms_per_step=rows[0]["launch_ms"],
                               config={"workload": "gather-patterns"}, patterns=rows)))
+        return
+    if args.workload == "mfma-valu-overlap":
+        r = mfma_valu_overlap(device)
+        print(json.dumps(dict(head, value=r["mfma_only_tflops"], unit="TFLOP/s", ms_per_step=r["launch_ms"]["OverlapMatrix"],
+                              config={"workload": "mfma-valu-overlap"}, overlap=r)))
         return
     if args.workload == "lds-calibration":
         r = lds_calibration(device)
@@ -805,6 +907,17 @@ def main():
         # (the duration of the kernel as a profiler's kernel trace sees it: launches back to back)
         result["mfma"]["layer_gemm_frac"] = result["mfma"]["layer_gemm"]["cfg2_mlp_cached_input"]["frac_back_to_back"]
         result["roofline"]["request_ceiling"] = request_ceiling(gather_ceiling(device), n, 64.0, 0.03, launch_ms)
+        # What binds the launch: every gather instruction of a level with more cells than the batch has points brings
+        # 64 lines of 128 bytes from the L2 (4 pairs of corners per point and level, 16 levels), of which 8 bytes
+        # each are used. Between the L2 of a die and a compute unit pass 64 bytes per clock (a published figure of the
+        # architecture: 2 KiB per clock and die over its 32 compute units); the clock is taken as 2.4 GHz.
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        l2_bytes = 64.0 * 128.0 * n
+        l2_peak_gbs = cus * 64.0 * 2.4e9 / 1e9
+        result["roofline"]["l2_lines"] = {"bound": "l2", "lines_per_point": 64, "line_bytes": 128,
+                                          "achieved": l2_bytes / (launch_ms * 1e-3) / 1e9, "peak": l2_peak_gbs, "unit": "GB/s",
+                                          "frac": l2_bytes / (launch_ms * 1e-3) / 1e9 / l2_peak_gbs,
+                                          "used_bytes_per_line": 8}
     if not train and cfg_id == 2 and not args.no_ordered:
         # the same launch on a batch that the library orders first, and on one that arrives ordered
         result["ordered_batch"] = ordered_batch_report(cfg_id, n, device, max(10, args.steps // 2), args.warmup)
