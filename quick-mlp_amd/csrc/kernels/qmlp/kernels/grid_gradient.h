@@ -265,7 +265,7 @@ struct GridGradientRecords
     struct AddToTensor
     {
         float* __restrict__ gradients;
-        __device__ __forceinline__ void operator()(unsigned element, float weight, const unsigned (&adjWords)[(F + 1) / 2], bool /*upper*/) const
+        __device__ __forceinline__ void operator()(unsigned element, float weight, const unsigned (&adjWords)[(F + 1) / 2]) const
         {
 #pragma unroll
             for (int i = 0; i < F; ++i) {
@@ -278,10 +278,9 @@ struct GridGradientRecords
     /**
      * The record of pair c of a point in one level: the offsets of its two entries within the slice of the lower
      * one, their weights and the adjoint words. Returns the slice (= bucket within the level) that files it.
-     * \param otherSlice called with (element of feature 0 in the table, weight, adjWords, whether it is the upper entry of the pair) for an upper entry that
+     * \param otherSlice called with (element of feature 0 in the table, weight, adjWords) for an upper entry that
      *    lies in another slice (an entry next to a slice boundary; in a hashed level one pair in thousands): the
-     *    record then keeps the lower entry only; and for both entries of a pair whose weights exceed one in
-     *    magnitude or are not finite (points outside the box): the record then adds nothing
+     *    record then keeps the lower entry only
      */
     template <int LEVEL, typename OtherSlice>
     __device__ __forceinline__ static int buildRecord(const typename Grid::LevelSetup& s, int c,
@@ -298,24 +297,11 @@ struct GridGradientRecords
         const unsigned eL = idxL * F - sliceStart;
         unsigned eH = idxH * F - sliceStart;                     // wraps if the upper entry lies below the slice
         float wH = w * s.f[PD];
-        float wL = w * (1.f - s.f[PD]);
-        bool upperAdded = false;
+        const float wL = w * (1.f - s.f[PD]);
         if (eH >= static_cast<unsigned>(SLICE_FLOATS)) {
-            otherSlice(base + idxH * F, wH, adjWords, true);
+            otherSlice(base + idxH * F, wH, adjWords);
             eH = eL;
             wH = 0.f;
-            upperAdded = true;
-        }
-        // The sums of the slice kernel are fixed point with a scale that counts on weights of at most one, which
-        // holds for every point inside the box. A point outside of it is extrapolated (the fractional position is
-        // not clamped) with weights that grow with its distance, a NaN coordinate gives NaN weights: such records
-        // go the way of the entries of other slices, and add nothing to the sums.
-        if (!(fabsf(wL) <= 1.f && fabsf(wH) <= 1.f)) {
-            otherSlice(base + idxL * F, wL, adjWords, false);
-            if (!upperAdded) otherSlice(base + idxH * F, wH, adjWords, true);
-            wL = 0.f;
-            wH = 0.f;
-            eH = eL;
         }
         rec[0] = eL | (eH << 16);
         rec[1] = __builtin_bit_cast(unsigned, wL);
@@ -388,6 +374,40 @@ struct GridGradientRecords
                 bucket[c] = buildRecord<LEVEL>(s, c, adjWords, rec[c], AddToTensor{params.parametersBackward});
                 // (a level of one slice needs no sorting: every lane has fixed places)
                 rank[c] = NS == 1 ? tid * PAIRS + c : atomicAdd(sHist + bucket[c], 1);
+            }
+            // The sums of the slice kernel are fixed point with a scale that counts on weights of at most one, which
+            // holds while every fractional position lies in [0, 1]: for every point inside the box. A point outside of
+            // it is extrapolated (the fractional position is not clamped) with weights that grow with its distance, a
+            // NaN coordinate gives NaN weights: the records of such a point are added to the gradient tensor right
+            // here, as records are whose bucket is full, and go to the buckets with weights of zero.
+            bool inside = true;
+#pragma unroll
+            for (int d = 0; d < D; ++d) inside = inside && s.f[d] >= 0.f && s.f[d] <= 1.f;
+            if (!inside) {
+                // (rare: a loop that recomputes the pairs and reads the adjoints again, so that it costs the points
+                // inside the box neither registers nor code)
+                float* __restrict__ grad = params.parametersBackward + base;
+#pragma unroll 1
+                for (int c = 0; c < PAIRS; ++c) {
+                    unsigned idxL, idxH;
+                    float w;
+                    pairEntries<LEVEL>(s, c, idxL, idxH, w);
+                    const float wL = w * (1.f - s.f[PD]), wH = w * s.f[PD];
+                    // (an upper entry in another slice than the lower one has been added by buildRecord already)
+                    const unsigned sliceStart = idxL * F / SLICE_FLOATS * SLICE_FLOATS;
+                    const bool upperAdded = idxH * F - sliceStart >= static_cast<unsigned>(SLICE_FLOATS);
+#pragma unroll 1
+                    for (int i = 0; i < F; ++i) {
+                        const float adj = static_cast<float>(adjRow[i * TILE_POINTS]);
+                        unsafeAtomicAdd(grad + idxL * F + i, wL * adj);
+                        if (!upperAdded) unsafeAtomicAdd(grad + idxH * F + i, wH * adj);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < PAIRS; ++c) {
+                    rec[c][1] = 0u;
+                    rec[c][2] = 0u;
+                }
             }
         } else {
             // lanes beyond the batch: in a level of one slice they fill their fixed places with records that add nothing
@@ -597,21 +617,18 @@ struct GridGradientTraceLevels
 #pragma unroll
             for (int c = 0; c < Impl::PAIRS; ++c) {
                 unsigned rec[Impl::RW];
-                unsigned otherElement[2] = {0u, 0u};
-                float otherWeight[2] = {0.f, 0.f};
-                bool other[2] = {false, false};
+                unsigned otherElement = 0u;
+                float otherWeight = 0.f;
+                bool other = false;
                 const int bucket = Impl::template buildRecord<LEVEL>(s, c, adjWords, rec,
-                    [&](unsigned element, float weight, const Words&, bool upper) {
-                        other[upper] = true;
-                        otherElement[upper] = element;
-                        otherWeight[upper] = weight;
-                    });
+                    [&](unsigned element, float weight, const Words&) { other = true; otherElement = element; otherWeight = weight; });
+                // (the records of a point outside the box are added by the records kernel itself, entry by entry as decoded here)
                 const unsigned sliceStart = static_cast<unsigned>(Cfg::memoryOffset[LEVEL]) + static_cast<unsigned>(bucket) * SLICE_FLOATS;
-                idx[LEVEL * NC + 2 * c] = other[0] ? otherElement[0] : sliceStart + (rec[0] & 0xffffu);
-                w[LEVEL * NC + 2 * c] = other[0] ? otherWeight[0] : __builtin_bit_cast(float, rec[1]);
+                idx[LEVEL * NC + 2 * c] = sliceStart + (rec[0] & 0xffffu);
+                w[LEVEL * NC + 2 * c] = __builtin_bit_cast(float, rec[1]);
                 if (NC > 1) {
-                    idx[LEVEL * NC + 2 * c + 1] = other[1] ? otherElement[1] : sliceStart + (rec[0] >> 16);
-                    w[LEVEL * NC + 2 * c + 1] = other[1] ? otherWeight[1] : __builtin_bit_cast(float, rec[2]);
+                    idx[LEVEL * NC + 2 * c + 1] = other ? otherElement : sliceStart + (rec[0] >> 16);
+                    w[LEVEL * NC + 2 * c + 1] = other ? otherWeight : __builtin_bit_cast(float, rec[2]);
                 }
             }
             GridGradientTraceLevels<Cfg, SLICE_FLOATS, LEVEL + 1>::run(pos, adjWords, idx, w);
