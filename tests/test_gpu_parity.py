@@ -1003,19 +1003,20 @@ def test_inference_sorted_by_grid_slab_gives_the_same_bits_as_the_order_given():
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("dim", [3, 2])
-def test_hashed_grid_sorted_on_request_gives_the_same_bits(dim):
+@pytest.mark.parametrize("dim,slices", [(3, -1), (2, -1), (3, 1)])
+def test_hashed_grid_sorted_on_request_gives_the_same_bits(dim, slices):
     """options.sort_points = 1 on a multi-level hashed grid: the batch is ordered by slabs of the grid's second and
     third coordinate (32 x 32 along a Z curve; 1024 slabs of the second one in 2-D) in front of the fused kernel.
     Inference agrees bit for bit with the batch as given (rows of three floats move as one 12-byte load and store),
-    a train step gives the same outputs and input gradients and the same sums for the other gradients."""
+    a train step gives the same outputs and input gradients and the same sums for the other gradients (slices = 1:
+    with the grid gradients summed per slice of the table, in the sorted order as well)."""
     spec = dict(n_in=dim, n_levels=8, n_features_per_level=2, log2_hashmap_size=12, min_resolution=4, max_resolution=128)
     grid = _grid_cfg(spec, "half")
     nets = []
     for mode in (1, 0):
         cfg = {"num_inputs": dim, "num_outputs": 1, "activation_specification": [bc.BUILTIN], "encodings": [dict(grid)],
                "network": [{"n_out": 32, "bias": False, "activation": "celu"}, {"n_out": 1, "bias": False, "activation": "identity"}],
-               "options": {"sort_points": mode}}
+               "options": {"sort_points": mode, "slice_gradients": slices}}
         rng = np.random.default_rng(3)
         case = Case(cfg)
         case.set_parameters(random_parameters(case.oracle, rng))
