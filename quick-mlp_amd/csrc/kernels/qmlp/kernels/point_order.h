@@ -20,24 +20,25 @@ QUICKMLP_KERNEL_NAMESPACE_BEGIN
 
 constexpr int POINT_ORDER_MAX_SLABS = 1024;
 constexpr int POINT_ORDER_BLOCK = 1024;
-constexpr int POINT_ORDER_POINTS_PER_THREAD = 8;    // a workgroup's chunk: 8192 points (offsets in it take 13 bits)
+constexpr int POINT_ORDER_POINTS_PER_THREAD = 4;    // a workgroup's chunk: 4096 points (offsets in it take 12 bits)
+constexpr int POINT_ORDER_SCAN_SLABS = 16;          // slabs per workgroup of PointOrderScan
 
-/** Slab of one coordinate, clamped to the box (the comparisons are false for NaN, which then lands in slab 0). */
-__device__ __forceinline__ int pointOrderSlab1(const float* row, long long channelStride, int channel, float lo, float scale, int slabs)
+/** Slab of one coordinate value, clamped to the box (the comparisons are false for NaN, which then lands in slab 0). */
+__device__ __forceinline__ int pointOrderSlab1(float value, float lo, float scale, int slabs)
 {
-    const float p = (row[static_cast<long long>(channel) * channelStride] - lo) * scale;
+    const float p = (value - lo) * scale;
     return p > 0.f ? static_cast<int>(fminf(p, static_cast<float>(slabs - 1))) : 0;
 }
 
-/** Slab of the point in row `index`: up to three grid coordinates, clamped to the box. */
-__device__ __forceinline__ int pointOrderSlab(const Tensor2Read<float>& inputs, long long index, const PointOrderKey& key)
+/** Slab of a point: up to three grid coordinates, clamped to the box. channel(c): the value of input channel c. */
+template <typename Channel>
+__device__ __forceinline__ int pointOrderSlabOf(const Channel& channel, const PointOrderKey& key)
 {
-    const float* row = inputs.data_ + index * inputs.strides_[0];
-    int s = pointOrderSlab1(row, inputs.strides_[1], key.channel0, key.min0, key.scale0, key.slabs0);
+    int s = pointOrderSlab1(channel(key.channel0), key.min0, key.scale0, key.slabs0);
     if (key.slabs1 > 1) {
-        const int s1 = pointOrderSlab1(row, inputs.strides_[1], key.channel1, key.min1, key.scale1, key.slabs1);
+        const int s1 = pointOrderSlab1(channel(key.channel1), key.min1, key.scale1, key.slabs1);
         if (key.slabs2 > 1) {
-            const int s2 = pointOrderSlab1(row, inputs.strides_[1], key.channel2, key.min2, key.scale2, key.slabs2);
+            const int s2 = pointOrderSlab1(channel(key.channel2), key.min2, key.scale2, key.slabs2);
             if (key.interleave12) {
                 // bit b of s1 to position 2b + 1, of s2 to 2b (at most 5 bits each)
                 int z = 0;
@@ -52,6 +53,14 @@ __device__ __forceinline__ int pointOrderSlab(const Tensor2Read<float>& inputs, 
         }
     }
     return s;
+}
+
+/** Slab of the point in row `index` of the inputs. */
+__device__ __forceinline__ int pointOrderSlab(const Tensor2Read<float>& inputs, long long index, const PointOrderKey& key)
+{
+    const float* row = inputs.data_ + index * inputs.strides_[0];
+    const long long channelStride = inputs.strides_[1];
+    return pointOrderSlabOf([&](int c) { return row[static_cast<long long>(c) * channelStride]; }, key);
 }
 
 /** histogram: (workgroups, POINT_ORDER_MAX_SLABS), every entry is written. */
@@ -73,29 +82,30 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderCount(
 
 /**
  * histogram[w][slab] becomes the number of points of the slab in the chunks before w,
- * totals[slab] their number in all chunks. A workgroup takes 64 slabs (one per lane); its 16
- * wavefronts take a sixteenth of the chunks each: sum, exchange through LDS, running sum.
+ * totals[slab] their number in all chunks. A workgroup takes POINT_ORDER_SCAN_SLABS slabs; 64 groups of
+ * its threads take a 64th of the chunks each: sum, exchange through LDS, running sum. (64 workgroups: with
+ * 16 workgroups of 64 slabs the pass took 8 us for 256 chunks and 13 us for 512.)
  */
 __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScan(int chunks, int* __restrict__ histogram, int* __restrict__ totals)
 {
-    constexpr int WAVES = POINT_ORDER_BLOCK / WAVE_SIZE;
-    constexpr int BATCH = 16;   // loads in flight
-    __shared__ int sPartial[WAVES][WAVE_SIZE];
-    const int lane = threadIdx.x % WAVE_SIZE, wave = threadIdx.x / WAVE_SIZE;
-    const int slab = blockIdx.x * WAVE_SIZE + lane;
-    const int perWave = (chunks + WAVES - 1) / WAVES;
-    const int begin = min(wave * perWave, chunks), end = min(begin + perWave, chunks);
+    constexpr int GROUPS = POINT_ORDER_BLOCK / POINT_ORDER_SCAN_SLABS;
+    constexpr int BATCH = 8;   // loads in flight
+    __shared__ int sPartial[GROUPS][POINT_ORDER_SCAN_SLABS];
+    const int local = threadIdx.x % POINT_ORDER_SCAN_SLABS, group = threadIdx.x / POINT_ORDER_SCAN_SLABS;
+    const int slab = blockIdx.x * POINT_ORDER_SCAN_SLABS + local;
+    const int perGroup = (chunks + GROUPS - 1) / GROUPS;
+    const int begin = min(group * perGroup, chunks), end = min(begin + perGroup, chunks);
     int sum = 0;
     for (int w0 = begin; w0 < end; w0 += BATCH) {
 #pragma unroll
         for (int j = 0; j < BATCH; ++j)
             if (w0 + j < end) sum += histogram[(w0 + j) * POINT_ORDER_MAX_SLABS + slab];
     }
-    sPartial[wave][lane] = sum;
+    sPartial[group][local] = sum;
     __syncthreads();
     int running = 0;
-    for (int q = 0; q < wave; ++q) running += sPartial[q][lane];
-    if (wave == WAVES - 1) totals[slab] = running + sum;
+    for (int q = 0; q < group; ++q) running += sPartial[q][local];
+    if (group == GROUPS - 1) totals[slab] = running + sum;
     for (int w0 = begin; w0 < end; w0 += BATCH) {
         int v[BATCH];
 #pragma unroll
@@ -161,11 +171,34 @@ __device__ __forceinline__ int pointOrderVectorChannels(const Tensor2Read<float>
     return 0;
 }
 
+/** Writes the channels of one row of the sorted copy; one store of 8, 12 or 16 bytes where the rows came as vectors. */
+template <int MAX_CHANNELS>
+__device__ __forceinline__ void pointOrderStoreRow(float* __restrict__ sortedInputs, long long position, int channels, int vectorChannels,
+                                                   const float (&row)[MAX_CHANNELS])
+{
+    typedef float f32x3a __attribute__((ext_vector_type(3), aligned(4)));
+    if (MAX_CHANNELS >= 4 && vectorChannels == 4) {
+        *reinterpret_cast<float4*>(sortedInputs + position * 4) = make_float4(row[0], row[1], row[2 % MAX_CHANNELS], row[3 % MAX_CHANNELS]);
+    } else if (MAX_CHANNELS >= 3 && vectorChannels == 3) {
+        const f32x3a v = {row[0], row[1], row[2 % MAX_CHANNELS]};
+        *reinterpret_cast<f32x3a*>(sortedInputs + position * 3) = v;
+    } else if (MAX_CHANNELS >= 2 && vectorChannels == 2) {
+        *reinterpret_cast<float2*>(sortedInputs + position * 2) = make_float2(row[0], row[1]);
+    } else {
+#pragma unroll
+        for (int c = 0; c < MAX_CHANNELS; ++c)
+            if (c < channels) sortedInputs[position * channels + c] = row[c];
+    }
+}
+
 /**
- * The workgroup first sorts the indices of its chunk by slab in LDS, then walks the sorted
- * chunk with consecutive lanes on consecutive positions, so that the stores of a wavefront
- * fall into a few runs (a scatter straight from the unsorted chunk sent every lane's stores
- * to a line of their own and took 80 us for 2^21 points).
+ * The workgroup sorts its chunk by slab in LDS, then walks the sorted chunk with consecutive lanes on
+ * consecutive positions, so that the stores of a wavefront fall into a few runs (a scatter straight from the
+ * unsorted chunk sent every lane's stores to a line of their own and took 80 us for 2^21 points).
+ * Rows of up to four channels are read once, in the order given (consecutive lanes, consecutive rows), and wait
+ * in LDS at their sorted place. Reading them a second time in sorted order, as wider rows still are, asks for 64
+ * lines per instruction, many of which the chunks of the other workgroups have meanwhile pushed out of the L2:
+ * 14 of the 42 us of this kernel for 2^21 rows of 16 bytes (the stores of the rows take 13 us, everything else 14).
  * \tparam MAX_CHANNELS at least the number of input channels (4, 8, 16)
  */
 template <int MAX_CHANNELS>
@@ -177,11 +210,13 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
     int* __restrict__ order)            // (numel): sorted position -> index in the batch
 {
     constexpr int CHUNK = POINT_ORDER_BLOCK * POINT_ORDER_POINTS_PER_THREAD;
+    constexpr bool STAGE_ROWS = MAX_CHANNELS <= 4;
     __shared__ int sStart[POINT_ORDER_MAX_SLABS];        // first position of the chunk's points of a slab in the sorted batch
     __shared__ int sCount[POINT_ORDER_MAX_SLABS];
     __shared__ int sLocalStart[POINT_ORDER_MAX_SLABS];   // the same inside the sorted chunk
     __shared__ int sWaveSum[POINT_ORDER_BLOCK / WAVE_SIZE];
     __shared__ unsigned int sSorted[CHUNK];              // sorted chunk: slab << 16 | offset of the point in the chunk
+    __shared__ __align__(16) float sRows[STAGE_ROWS ? CHUNK * MAX_CHANNELS : 4];   // the rows of the sorted chunk
     const int t = threadIdx.x;
 
     sCount[t] = 0;
@@ -189,16 +224,31 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
     const int slabStart = pointOrderBlockScan(total, sWaveSum);   // holds a barrier after sCount = 0
     sStart[t] = slabStart + histogram[blockIdx.x * POINT_ORDER_MAX_SLABS + t];
 
+    const int channels = inputs.sizes_[1];
+    const int vectorChannels = pointOrderVectorChannels(inputs);
     const long long chunk = static_cast<long long>(blockIdx.x) * CHUNK;
     const int chunkPoints = static_cast<int>(min(static_cast<long long>(CHUNK), numel - chunk));
     int slab[POINT_ORDER_POINTS_PER_THREAD], rank[POINT_ORDER_POINTS_PER_THREAD];
+    float rows[STAGE_ROWS ? POINT_ORDER_POINTS_PER_THREAD : 1][MAX_CHANNELS] = {};
+    (void)rows;
 #pragma unroll
     for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
         const int j = k * POINT_ORDER_BLOCK + t;
         slab[k] = 0;
         rank[k] = 0;
         if (j < chunkPoints) {
-            slab[k] = pointOrderSlab(inputs, chunk + j, key);
+            if constexpr (STAGE_ROWS) {
+                pointOrderLoadRow<MAX_CHANNELS>(inputs, chunk + j, vectorChannels, rows[k]);
+                const float (&row)[MAX_CHANNELS] = rows[k];
+                slab[k] = pointOrderSlabOf([&](int c) {
+                    float v = row[0];
+#pragma unroll
+                    for (int i = 1; i < MAX_CHANNELS; ++i) v = c == i ? row[i] : v;
+                    return v;
+                }, key);
+            } else {
+                slab[k] = pointOrderSlab(inputs, chunk + j, key);
+            }
             rank[k] = atomicAdd(&sCount[slab[k]], 1);
         }
     }
@@ -208,12 +258,17 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
 #pragma unroll
     for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
         const int j = k * POINT_ORDER_BLOCK + t;
-        if (j < chunkPoints) sSorted[sLocalStart[slab[k]] + rank[k]] = static_cast<unsigned int>(slab[k]) << 16 | static_cast<unsigned int>(j);
+        if (j < chunkPoints) {
+            const int at = sLocalStart[slab[k]] + rank[k];
+            sSorted[at] = static_cast<unsigned int>(slab[k]) << 16 | static_cast<unsigned int>(j);
+            if constexpr (STAGE_ROWS) {
+#pragma unroll
+                for (int c = 0; c < MAX_CHANNELS; ++c) sRows[at * MAX_CHANNELS + c] = rows[k][c];
+            }
+        }
     }
     __syncthreads();
 
-    const int channels = inputs.sizes_[1];
-    const int vectorChannels = pointOrderVectorChannels(inputs);
 #pragma unroll 4
     for (int k = 0; k < POINT_ORDER_POINTS_PER_THREAD; ++k) {
         const int j = k * POINT_ORDER_BLOCK + t;
@@ -222,22 +277,15 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
         const long long index = chunk + (entry & 0xffffu);
         const int s = static_cast<int>(entry >> 16);
         float row[MAX_CHANNELS];
-        pointOrderLoadRow<MAX_CHANNELS>(inputs, index, vectorChannels, row);
+        if constexpr (STAGE_ROWS) {
+#pragma unroll
+            for (int c = 0; c < MAX_CHANNELS; ++c) row[c] = sRows[j * MAX_CHANNELS + c];
+        } else {
+            pointOrderLoadRow<MAX_CHANNELS>(inputs, index, vectorChannels, row);
+        }
         const long long position = sStart[s] + (j - sLocalStart[s]);
         order[position] = static_cast<int>(index);
-        typedef float f32x3a __attribute__((ext_vector_type(3), aligned(4)));
-        if (MAX_CHANNELS >= 4 && vectorChannels == 4) {
-            *reinterpret_cast<float4*>(sortedInputs + position * 4) = make_float4(row[0], row[1], row[2 % MAX_CHANNELS], row[3 % MAX_CHANNELS]);
-        } else if (MAX_CHANNELS >= 3 && vectorChannels == 3) {
-            const f32x3a v = {row[0], row[1], row[2 % MAX_CHANNELS]};
-            *reinterpret_cast<f32x3a*>(sortedInputs + position * 3) = v;
-        } else if (MAX_CHANNELS >= 2 && vectorChannels == 2) {
-            *reinterpret_cast<float2*>(sortedInputs + position * 2) = make_float2(row[0], row[1]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < MAX_CHANNELS; ++c)
-                if (c < channels) sortedInputs[position * channels + c] = row[c];
-        }
+        pointOrderStoreRow<MAX_CHANNELS>(sortedInputs, position, channels, vectorChannels, row);
     }
 }
 

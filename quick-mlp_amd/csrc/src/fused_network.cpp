@@ -1590,7 +1590,7 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
     kernel::PointOrderKey key{};
     if (pointOrderFor(numel, key)) {
         loadPointOrderKernels(adjointFlags > 0 && sortsTraining(numel));
-        constexpr long long SLABS = 1024, CHUNK = 8 * 1024;   // as in sortPoints()
+        constexpr long long SLABS = 1024, CHUNK = 4 * 1024;   // as in sortPoints()
         const long long words = (divUp<long long>(numel, CHUNK) + 1) * SLABS + static_cast<long long>(numel) * (channelsIn_ + 1);
         if (pointOrder_.capacityWords < words && words <= std::numeric_limits<int32_t>::max()) {
             pointOrder_.workspace = Tensor(Tensor::FLOAT, {static_cast<int32_t>(words)});
@@ -1635,7 +1635,7 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
         throw std::runtime_error("The kernels that order the batch are not loaded yet, and loading allocates: run "
                                  "inference() once on a batch of the same size first");
     loadPointOrderKernels(false);
-    constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 8 * BLOCK;   // as in point_order.h
+    constexpr int SLABS = 1024, BLOCK = 1024, CHUNK = 4 * BLOCK;   // as in point_order.h
     // words: slab totals and one histogram per chunk; then (unless the caller has room for them) sorted inputs and order
     const long long histogramWords = (divUp(numel, CHUNK) + 1ll) * SLABS;
     const long long rowWords = static_cast<long long>(numel) * (channels + 1);
@@ -1686,7 +1686,7 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     }
     {
         void* args[] = {&chunks, &histogram, &totals};
-        po.scan.value().launch(SLABS / WARP_SIZE, BLOCK, 0, stream, args);
+        po.scan.value().launch(SLABS / 16, BLOCK, 0, stream, args);   // 16 slabs per workgroup (POINT_ORDER_SCAN_SLABS)
     }
     {
         void* args[] = {&count, &inputAcc, &key, &histogram, &totals, &sortedData, &orderData};
