@@ -8,6 +8,7 @@
 #include "tensor.h"
 
 #include <optional>
+#include <unordered_map>
 #include <random>
 #include <vector>
 
@@ -78,6 +79,14 @@ public:
         // levels or more); 0: never; >0: always.
         int sliceGradients = -1;
 
+        // Input gradients through grid encodings whose parameter gradients take the slice kernels: a training
+        // pass (forward) also stores, per point and level, the derivatives of the interpolated features with
+        // respect to the position (16 bytes per level for a 3-D grid with 2 half features), and the adjoint pass
+        // reads them instead of gathering all corners of every cell a second time. <0 (default): when the
+        // adjoint flags announced last (forwardMemory(), adjoint()) ask for input and encoding gradients;
+        // 0: never (no room for them in the forward memory either); >0: every training pass.
+        int inputDerivatives = -1;
+
         // Gradients of the layer weights: summed inside the backward kernel, which holds the adjoint
         // pre-activations in registers (Layer::weightGradient), instead of by one kernel per layer that reads
         // them back from memory. <0 (default): the layers with the fewest gradient tiles, up to 16 tiles (64
@@ -133,9 +142,10 @@ private:
         int fullGrid = 0;
     };
     // [store intermediates][variant], see ForwardVariant
-    std::optional<CompiledKernel> forwardKernels_[2][4];
+    // [0]: inference, [1]: forward (stores the intermediates), [2]: forward that also stores position derivatives
+    std::optional<CompiledKernel> forwardKernels_[3][4];
     // set once the compiled REGISTERS shape turned out to spill heavily: it is not used then
-    bool registerShapeSpills_[2] = {false, false};
+    bool registerShapeSpills_[3] = {false, false, false};
 
     // counting sort of the batch by grid slab in front of the inference kernel
     struct PointOrder
@@ -196,6 +206,9 @@ private:
         // when a batch first asks for it: a batch of fewer points than the largest workgroups of all compute units
         // hold goes to smaller ones
         std::vector<std::optional<CompiledKernel>> records;
+        // the same with the input gradients from the position derivatives that the forward pass stored
+        std::vector<std::optional<CompiledKernel>> recordsFromDerivatives;
+        long long derivativeOffset = 0;   // bytes per point of the batch in front of this encoding's derivatives in the forward memory
         std::string recordsSource;
         int channelOffset = 0;
         CompiledKernel kernel;       // GridGradientSlicesKernel
@@ -232,6 +245,21 @@ private:
     bool useSliceGradients(int numel, int flags) const;
 
     int perEntryForwardMemoryBytes_;
+    /**
+     * Position derivatives of the grid encodings (options.input_derivatives): per encoding the bytes per point of
+     * the batch in front of its derivatives within their region of the forward memory (-1: the encoding keeps
+     * none), and the bytes per point of the whole region, which lies behind the intermediates.
+     */
+    std::vector<long long> derivativeOffsets_;
+    int derivativeBytesPerPoint_ = 0;
+    /** The adjoint flags that the caller announced last: forwardMemory(n, flags), adjoint(..., flags, ...). */
+    int announcedFlags_ = 0;
+    /** Forward memories whose last training pass stored position derivatives, with the size of that batch. */
+    std::unordered_map<const void*, int> derivativesStored_;
+    /** Bytes per point of the forward memory: intermediates and, where kept, position derivatives. */
+    size_t forwardBytesPerPoint() const { return static_cast<size_t>(perEntryForwardMemoryBytes_) + static_cast<size_t>(derivativeBytesPerPoint_); }
+    /** Whether a training pass over numel points that is followed by adjoint(flags) stores position derivatives. */
+    bool storesDerivatives(int numel, int flags) const;
     std::vector<AdjointLayerInfo> backwardInfo_;
     event_t adjointEvent_;
     bool streamsCreated_;
@@ -369,13 +397,13 @@ private:
     int registerVariantTiles(bool store) const;
     /** Workgroup size and tiles per wavefront of a shape of the forward kernel. */
     void forwardShape(bool store, int variant, int& blockSize, int& pointsPerLane) const;
-    void compileForwardKernel(bool store, int variant, bool compileOnly = false);
+    void compileForwardKernel(bool store, int variant, bool compileOnly = false, bool derivatives = false);
     /**
      * The kernel shape for the next launch over a batch of numTiles tiles and, in launchTiles,
      * how many of them that launch should take (whole steps of a large shape first; the caller
      * asks again for the rest).
      */
-    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr, bool noAlloc = false);
+    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr, bool noAlloc = false, bool derivatives = false);
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */
@@ -386,13 +414,13 @@ private:
     int directInputStart() const;
     /** Throws unless every encoding with parameters has a tensor bound for 'usage'. */
     void checkEncodingParameters(Tensor::Usage usage) const;
-    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false);
+    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false, bool derivatives = false);
     void compileBackwardKernel(int flags, bool sliceGradients = false, bool compileOnly = false);
     /** The records kernel of a batch of numel points (compiled on first use; compileOnly: all of them into the cache). */
-    const CompiledKernel& recordsKernelFor(SliceGradientKernel& sk, int flags, int numel);
-    void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly);
+    const CompiledKernel& recordsKernelFor(SliceGradientKernel& sk, int flags, int numel, bool fromDerivatives = false);
+    void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives = false);
 
-    std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false) const;
+    std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false, bool derivatives = false) const;
     std::string backwardSource(int flags, int blockSize, bool sliceGradients = false) const;
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const;

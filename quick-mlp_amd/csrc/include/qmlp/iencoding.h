@@ -140,6 +140,7 @@ public:
         int recordWords = 0;               // 32-bit words of a record
         int pairs = 0;                     // records per point and level
         int pointsPerWorkgroup = 0;        // most lanes of a workgroup of the records kernel (a power of two)
+        int derivativeBytesPerPoint = 0;   // of kernel::PositionDerivativeLayout: what a training pass may keep for the input gradients
         /** Dynamic LDS of the records kernel with this many lanes: its records of one level with the slice of each
          *  (16 bits), and per slice of the level (at most 512) room in the bucket, count and place among the records. */
         int recordsLdsBytes(int points) const { return points * pairs * (recordWords * 4 + 2) + 512 * 8 + (2 * 512 + 1) * 4 + 64; }

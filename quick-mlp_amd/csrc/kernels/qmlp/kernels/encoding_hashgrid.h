@@ -147,6 +147,82 @@ struct CornerTrace
 };
 
 /**
+ * Where a training pass keeps, per point and level, the derivatives of the interpolated features with respect to
+ * the position within the level (in cells: without the factor resolution - 1): d feature_i / d p_d at value
+ * i * Dim + d, in the precision of the table (half values are clamped to the finite range), padded with zeros to whole
+ * chunks of 16 bytes. Per tile of 64 points the chunks lie level by level, chunk by chunk, 64 points side by side:
+ * chunk k of level l of point j of tile t is chunk ((t * Levels + l) * CHUNKS + k) * 64 + j of the region. A lane
+ * writes and reads whole chunks, neighbouring lanes neighbouring chunks.
+ * With these the input gradients of the adjoint pass need no second gather of the table (2^Dim entries per point
+ * and level): they are sum_i adjoint_i * derivative_(i, d), read in one or a few coalesced loads.
+ */
+template <typename Cfg>
+struct PositionDerivativeLayout
+{
+    typedef typename Cfg::table_t value_t;
+    static constexpr int VALUES = Cfg::Dim * Cfg::Features;
+    static constexpr int PER_CHUNK = 16 / static_cast<int>(sizeof(value_t));
+    static constexpr int CHUNKS = (VALUES + PER_CHUNK - 1) / PER_CHUNK;
+    static constexpr int BYTES_PER_POINT = Cfg::Levels * CHUNKS * 16;
+    typedef value_t chunk_t __attribute__((ext_vector_type(PER_CHUNK)));
+
+    __device__ __forceinline__ static long long chunkIndex(long long tile, int level, int chunk, int lane)
+    {
+        return ((tile * Cfg::Levels + level) * CHUNKS + chunk) * TILE_POINTS + lane;
+    }
+
+    __device__ __forceinline__ static value_t narrow(float v)
+    {
+        if constexpr (sizeof(value_t) == 2) return static_cast<value_t>(fminf(fmaxf(v, -65504.f), 65504.f));
+        else return v;
+    }
+
+    /** The chunks of one level of one point from its VALUES derivatives. */
+    __device__ __forceinline__ static void store(chunk_t* __restrict__ level0, int level, const float (&values)[VALUES])
+    {
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            chunk_t c;
+#pragma unroll
+            for (int j = 0; j < PER_CHUNK; ++j)
+                c[j] = k * PER_CHUNK + j < VALUES ? narrow(values[k * PER_CHUNK + j < VALUES ? k * PER_CHUNK + j : 0]) : static_cast<value_t>(0);
+            level0[(level * CHUNKS + k) * TILE_POINTS] = c;
+        }
+    }
+
+    __device__ __forceinline__ static void load(const chunk_t* __restrict__ level0, int level, float (&values)[VALUES])
+    {
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k) {
+            const chunk_t c = level0[(level * CHUNKS + k) * TILE_POINTS];
+#pragma unroll
+            for (int j = 0; j < PER_CHUNK; ++j)
+                if (k * PER_CHUNK + j < VALUES) values[k * PER_CHUNK + j] = static_cast<float>(c[j]);
+        }
+    }
+};
+
+/** forwardBatch without derivatives with respect to the position (inference; training passes that need none). */
+struct NoPositionDerivatives
+{
+    static constexpr bool Enabled = false;
+};
+
+/** forwardBatch stores the derivatives with respect to the position (PositionDerivativeLayout). */
+template <typename Cfg>
+struct StorePositionDerivatives
+{
+    static constexpr bool Enabled = true;
+    typedef PositionDerivativeLayout<Cfg> Layout;
+    typename Layout::chunk_t* __restrict__ first;   // chunk 0 of level 0 of this lane's point of the lane's first tile
+    int tiles;                                      // the lane's tiles q = 0 .. tiles-1 lie inside the batch
+    __device__ __forceinline__ void store(int q, int level, const float (&values)[Layout::VALUES]) const
+    {
+        if (q < tiles) Layout::store(first + static_cast<long long>(q) * (Cfg::Levels * Layout::CHUNKS * TILE_POINTS), level, values);
+    }
+};
+
+/**
  * \tparam Cfg generated struct with
  *   static constexpr int Start, Dim, Levels, Features; static constexpr bool Concat, ResolutionFactor;
  *   typedef table_t (float or f16);
@@ -244,6 +320,20 @@ struct EncodingHashGrid
                                                        const table_t* __restrict__ table, float (&feat)[F],
                                                        const Trace& trace = Trace{})
     {
+        float none[F * D];
+        gatherLevelImpl<false>(l, pos, table, feat, none, trace);
+    }
+
+    /**
+     * \tparam DERIVATIVES also computes dfeat[i * D + d] = d feat[i] / d p_d, p the position in cells of the level:
+     *    sum over the corners of +-(product of the weights of the other dimensions) * value, from the values that
+     *    the interpolation has loaded anyway
+     */
+    template <bool DERIVATIVES, typename Trace = NoCornerTrace>
+    __device__ __forceinline__ static void gatherLevelImpl(int l, const float (&pos)[D],
+                                                           const table_t* __restrict__ table, float (&feat)[F],
+                                                           float (&dfeat)[F * D], const Trace& trace = Trace{})
+    {
         // no contraction into fused multiply-adds: the kernels of different shapes (tiles per
         // wave) would contract differently, and the same point has to give the same bits
         // whatever the batch size
@@ -254,6 +344,10 @@ struct EncodingHashGrid
         const unsigned base = static_cast<unsigned>(Cfg::memoryOffset[l]);
 #pragma unroll
         for (int i = 0; i < F; ++i) feat[i] = 0.f;
+        if constexpr (DERIVATIVES) {
+#pragma unroll
+            for (int i = 0; i < F * D; ++i) dfeat[i] = 0.f;
+        }
 
         if (!hashed && R >= 2) {
             // pairs along dimension D-1: entries (zb, zb+1) with zb = min(iL, R-2)
@@ -279,7 +373,19 @@ struct EncodingHashGrid
                 for (int i = 0; i < F; ++i) {
                     const float vL = lSecond ? e1[i] : e0[i];
                     const float vH = hSecond ? e1[i] : e0[i];
-                    feat[i] += w * (wzL * vL + wzH * vH);
+                    const float along = wzL * vL + wzH * vH;
+                    feat[i] += w * along;
+                    if constexpr (DERIVATIVES) {
+                        dfeat[i * D + PD] += w * (vH - vL);
+#pragma unroll
+                        for (int d = 0; d < PD; ++d) {
+                            float others = 1.f;
+#pragma unroll
+                            for (int e = PD - 1; e >= 0; --e)
+                                if (e != d) others = others * (((c >> e) & 1) ? s.f[e] : (1.f - s.f[e]));
+                            dfeat[i * D + d] += (((c >> d) & 1) ? others : -others) * along;
+                        }
+                    }
                 }
                 if constexpr (Trace::Enabled) {
                     trace.record(l * NC + 2 * c, pairElement + (lSecond ? F : 0), w * wzL);
@@ -320,7 +426,19 @@ struct EncodingHashGrid
 #pragma unroll
                 for (int i = 0; i < F; ++i) {
                     const float vL = (idxL & 1u) ? e1[i] : e0[i];
-                    feat[i] += w * (wxL * vL + wxH * vH[i]);
+                    const float along = wxL * vL + wxH * vH[i];
+                    feat[i] += w * along;
+                    if constexpr (DERIVATIVES) {
+                        dfeat[i * D] += w * (vH[i] - vL);
+#pragma unroll
+                        for (int d = 1; d < D; ++d) {
+                            float others = 1.f;
+#pragma unroll
+                            for (int e = D - 1; e >= 1; --e)
+                                if (e != d) others = others * (((c >> (e - 1)) & 1) ? s.f[e] : (1.f - s.f[e]));
+                            dfeat[i * D + d] += (((c >> (d - 1)) & 1) ? others : -others) * along;
+                        }
+                    }
                 }
             }
         } else {
@@ -333,6 +451,17 @@ struct EncodingHashGrid
 #pragma unroll
                 for (int i = 0; i < F; ++i) feat[i] += w * v[i];
                 if constexpr (Trace::Enabled) trace.record(l * NC + c, element, w);
+                if constexpr (DERIVATIVES) {
+#pragma unroll
+                    for (int d = 0; d < D; ++d) {
+                        float others = 1.f;
+#pragma unroll
+                        for (int e = D - 1; e >= 0; --e)
+                            if (e != d) others = others * (((c >> e) & 1) ? s.f[e] : (1.f - s.f[e]));
+#pragma unroll
+                        for (int i = 0; i < F; ++i) dfeat[i * D + d] += (((c >> d) & 1) ? others : -others) * v[i];
+                    }
+                }
             }
         }
     }
@@ -342,8 +471,9 @@ struct EncodingHashGrid
      * any starts level l+1, so that the workgroups of the device sweep through the level
      * tables together and a level's table stays in L2 while it is in use.
      */
-    template <int PPL, typename I, typename Os>
-    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], Os& outputs, const param_t& params)
+    template <int PPL, typename I, typename Os, typename Derivatives = NoPositionDerivatives>
+    __device__ __forceinline__ static void forwardBatch(const I (&inputs)[PPL], Os& outputs, const param_t& params,
+                                                        const Derivatives& derivatives = Derivatives{})
     {
         typedef typename RowsValueType<Os>::Type O_t;
         float pos[PPL][D];
@@ -358,7 +488,15 @@ struct EncodingHashGrid
         for (int l = 0; l < L; ++l) {
             float feat[PPL][F];
 #pragma unroll
-            for (int q = 0; q < PPL; ++q) gatherLevel(l, pos[q], params.parametersForward, feat[q]);
+            for (int q = 0; q < PPL; ++q) {
+                if constexpr (Derivatives::Enabled) {
+                    float dfeat[F * D];
+                    gatherLevelImpl<true>(l, pos[q], params.parametersForward, feat[q], dfeat);
+                    derivatives.store(q, l, dfeat);
+                } else {
+                    gatherLevel(l, pos[q], params.parametersForward, feat[q]);
+                }
+            }
 #pragma unroll
             for (int q = 0; q < PPL; ++q) {
                 if constexpr (Cfg::Concat && F % 2 == 0) {

@@ -21,7 +21,10 @@
 //       operation by operation): two entries that lie side by side with one load, issued after the
 //       bucket atomics of the level and used at its end, while the barriers in between (ldsBarrier)
 //       wait for LDS only, so the gathers stay in flight over the staging and the copy of the records
-//       (16 levels of a 3-D hash grid, 2^18 points: 203 -> 188 us; without the gathers 117 us);
+//       (16 levels of a 3-D hash grid, 2^18 points: 203 -> 188 us; without the gathers 117 us). Where the forward
+//       pass kept the derivatives of the features with respect to the position (PositionDerivativeLayout,
+//       INPUT_GRADIENTS == 2), the share is adjoint x derivative from one or two coalesced loads per level
+//       instead (same grid: 126 us);
 //   GridGradientSlicesKernel   runs one workgroup per work item (level, slice, part of the
 //       bucket): it streams through its records and adds weight * adjoint to the slice in LDS,
 //       then adds the slice to the gradient tensor (with atomics only for a coarse level, whose
@@ -154,6 +157,8 @@ struct GridGradientRecords
     static constexpr int PAIRS = Layout::PAIRS;
     static constexpr int RW = Layout::RECORD_WORDS;
     static constexpr int MAX_SLICES = 512;
+    typedef PositionDerivativeLayout<Cfg> DerivativeLayout;
+    typedef typename DerivativeLayout::chunk_t DerivativeChunk;
 
     /** The two table entries of pair c of a point (bit b of c: upper corner in the b-th dimension
      *  other than the pair's own) and the weight of the pair without its own dimension. */
@@ -327,13 +332,13 @@ struct GridGradientRecords
         }
     }
 
-    template <int LEVEL, bool INPUT_GRADIENTS>
+    template <int LEVEL, int INPUT_GRADIENTS>
     __device__ __forceinline__ static void runLevel(int p, bool valid, long long numel, const float (&pos)[D],
                                                     const f16* __restrict__ adjEncoded, const param_t& params,
                                                     unsigned* __restrict__ records, int* __restrict__ cursors,
                                                     unsigned* sStage, unsigned short* sBucketOf, int* sHist,
                                                     int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits,
-                                                    float (&adjPos)[D])
+                                                    float (&adjPos)[D], const DerivativeChunk* __restrict__ derivatives)
     {
         constexpr bool hashed = Cfg::hashed[LEVEL];
         constexpr int PD = hashed ? 0 : D - 1;
@@ -363,7 +368,7 @@ struct GridGradientRecords
                 // largest magnitude seen (as fp16 bits without the sign: ordered like the values, NaN above infinity)
                 maxAdjBits = max(maxAdjBits, bits & 0x7fffu);
             }
-            if constexpr (INPUT_GRADIENTS && !DEFER_ENTRIES) {
+            if constexpr (INPUT_GRADIENTS == 1 && !DEFER_ENTRIES) {
                 // the entries of all corners, for this grid's share of dL/dinput (a dense 4-D grid with 8 features
                 // holds 64 registers: used at once; held until the end of the level 302 against 275 us)
                 loadHeld<LEVEL>(s, params, held);
@@ -444,7 +449,7 @@ struct GridGradientRecords
         }
         ldsBarrier();
 
-        if constexpr (INPUT_GRADIENTS && DEFER_ENTRIES) {
+        if constexpr (INPUT_GRADIENTS == 1 && DEFER_ENTRIES) {
             // The entries of all corners, for this grid's share of dL/dinput, where they take few registers: loaded
             // here and used at the end of the level, so that the two steps in between hide their latency (the
             // barriers order LDS only). Not earlier: the first wavefront waits for its bucket atomics above, and
@@ -477,9 +482,39 @@ struct GridGradientRecords
             }
         }
 
-        if constexpr (INPUT_GRADIENTS && DEFER_ENTRIES) {
+        if constexpr (INPUT_GRADIENTS == 1 && DEFER_ENTRIES) {
             if (valid) positionGradient<LEVEL>(p, s, held, adjEncoded, adjPos);
         }
+        if constexpr (INPUT_GRADIENTS == 2) {
+            if (valid) positionGradientFromDerivatives<LEVEL>(p, derivatives, adjEncoded, adjPos);
+        }
+    }
+
+    /**
+     * This level's share of the gradient with respect to the position from the derivatives of the level's features
+     * that the forward pass stored (PositionDerivativeLayout): sum_i adjoint_i * d feature_i / d p_d, read with one
+     * or a few coalesced loads instead of a gather of all corners of the cell.
+     */
+    template <int LEVEL>
+    __device__ __forceinline__ static void positionGradientFromDerivatives(int p, const DerivativeChunk* __restrict__ derivatives,
+                                                                           const f16* __restrict__ adjEncoded, float (&adjPos)[D])
+    {
+        const f16* adjRow = adjEncoded + static_cast<long long>(p / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
+            + (CHANNEL_OFFSET + (Cfg::Concat ? LEVEL * F : 0)) * TILE_POINTS + (p % TILE_POINTS);
+        float values[DerivativeLayout::VALUES];
+        DerivativeLayout::load(derivatives + DerivativeLayout::chunkIndex(p / TILE_POINTS, 0, 0, p % TILE_POINTS), LEVEL, values);
+        float lvl[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) lvl[d] = 0.f;
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            const float adj = static_cast<float>(adjRow[i * TILE_POINTS]);
+#pragma unroll
+            for (int d = 0; d < D; ++d) lvl[d] += adj * values[i * D + d];
+        }
+        const float scale = Cfg::ResolutionFactor ? static_cast<float>(Cfg::resolution[LEVEL] - 1) : 1.f;
+#pragma unroll
+        for (int d = 0; d < D; ++d) adjPos[d] += scale * lvl[d];
     }
 
     /** Registers worth holding across the sort of a level's records: 64 bytes of table entries per lane. */
@@ -523,19 +558,19 @@ struct GridGradientRecords
         for (int d = 0; d < D; ++d) adjPos[d] += scale * lvl[d];
     }
 
-    template <int LEVEL, bool INPUT_GRADIENTS>
+    template <int LEVEL, int INPUT_GRADIENTS>
     __device__ __forceinline__ static void runLevels(int p, bool valid, long long numel, const float (&pos)[D],
                                                      const f16* __restrict__ adjEncoded, const param_t& params,
                                                      unsigned* __restrict__ records, int* __restrict__ cursors,
                                                      unsigned* sStage, unsigned short* sBucketOf, int* sHist,
                                                      int* sLocalBase, long long* sGlobalBase, unsigned& maxAdjBits,
-                                                     float (&adjPos)[D])
+                                                     float (&adjPos)[D], const DerivativeChunk* __restrict__ derivatives)
     {
         if constexpr (LEVEL < Cfg::Levels) {
             runLevel<LEVEL, INPUT_GRADIENTS>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf, sHist,
-                                             sLocalBase, sGlobalBase, maxAdjBits, adjPos);
+                                             sLocalBase, sGlobalBase, maxAdjBits, adjPos, derivatives);
             runLevels<LEVEL + 1, INPUT_GRADIENTS>(p, valid, numel, pos, adjEncoded, params, records, cursors, sStage, sBucketOf,
-                                                  sHist, sLocalBase, sGlobalBase, maxAdjBits, adjPos);
+                                                  sHist, sLocalBase, sGlobalBase, maxAdjBits, adjPos, derivatives);
         }
     }
 };
@@ -545,7 +580,7 @@ struct GridGradientRecords
  * records: room for levelOffset(Levels, layoutNumel) records; cursors: one int per bucket, then one word that
  * receives the largest magnitude among the adjoints (fp16 bits without the sign); all zeroed by the caller.
  */
-template <typename Cfg, int ROW_CHANNELS, int CHANNEL_OFFSET, int SLICE_FLOATS, int POINTS, bool INPUT_GRADIENTS>
+template <typename Cfg, int ROW_CHANNELS, int CHANNEL_OFFSET, int SLICE_FLOATS, int POINTS, int INPUT_GRADIENTS>
 __global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
     int numel,
     int layoutNumel,                          //points the buckets are laid out for (numel rounded up to whole tiles)
@@ -553,7 +588,8 @@ __global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
     const half* __restrict__ adjEncodedH,     //adjoint of the encoded rows: (tiles, ROW_CHANNELS, 64)
     const HashGridParams<typename Cfg::table_t, Cfg::Dim> params,
     unsigned* __restrict__ records, int* __restrict__ cursors,
-    Tensor2RW<float> adjInputs)               //INPUT_GRADIENTS: shape (numel, Cin), this grid's share of dL/dinput is added
+    Tensor2RW<float> adjInputs,               //INPUT_GRADIENTS: shape (numel, Cin), this grid's share of dL/dinput is added
+    const void* __restrict__ derivativesV)    //INPUT_GRADIENTS == 2: the position derivatives of this grid that the forward pass stored
 {
     typedef GridGradientRecords<Cfg, ROW_CHANNELS, CHANNEL_OFFSET, SLICE_FLOATS, POINTS> Impl;
     constexpr int D = Cfg::Dim;
@@ -582,8 +618,8 @@ __global__ void __launch_bounds__(POINTS) GridGradientRecordsKernel(
         for (int d = 0; d < D; ++d) adjPos[d] = 0.f;
         Impl::template runLevels<0, INPUT_GRADIENTS>(p, valid, layoutNumel, pos, reinterpret_cast<const f16*>(adjEncodedH), params,
                                                      records, cursors, sStage, sBucketOf, sHist, sLocalBase, sGlobalBase, maxAdjBits,
-                                                     adjPos);
-        if constexpr (INPUT_GRADIENTS) {
+                                                     adjPos, static_cast<const typename Impl::DerivativeChunk*>(derivativesV));
+        if constexpr (INPUT_GRADIENTS != 0) {
             // every point belongs to one lane of one workgroup: a plain read-modify-write
             if (valid) {
 #pragma unroll

@@ -42,8 +42,11 @@ __device__ __forceinline__ void bindEncodingRow(PackedRegisterRowsView<T, PPL, C
  * \tparam STORE false: inference. true: additionally stores, per 64-point tile and
  *   channel-major, the encoded network input and the pre-activations of every layer
  *   into forwardTmpMemory for the adjoint pass.
+ * \tparam DERIVATIVES with STORE: grid encodings additionally store, behind these regions, the derivatives of
+ *   their features with respect to the position (PositionDerivativeLayout), from which the adjoint pass forms
+ *   the input gradients without a second gather.
  */
-template <bool STORE>
+template <bool STORE, bool DERIVATIVES = false>
 __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkKernelInferenceAndForward(
     int numel,
     const Tensor2Read<float> inputs,  //shape (numel, Cin)

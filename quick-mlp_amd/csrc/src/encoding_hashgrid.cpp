@@ -340,6 +340,18 @@ bool EncodingHashGrid::gradientSlices(GradientSliceLayout& layout) const
     int points = 1024;
     while (points > 64 && points * layout.pairs * layout.recordWords * 4 > 96 * 1024) points /= 2;
     layout.pointsPerWorkgroup = points;
+    {
+        // as kernel::PositionDerivativeLayout: Dim * Features values per level in the precision of the table, in whole chunks of 16 bytes
+        // Kept where they are at most 32 bytes per point and level. The gathers they save the adjoint pass cost a
+        // line of the L2 per pair of corners in a hashed level (a 3-D grid with 2 half features: 4 lines against 16
+        // bytes of derivatives; records kernel of 16 such levels at 2^18 points 197 -> 126 us, forward pass 96 ->
+        // 103 us). A dense 4-D grid with 8 features would keep 64 bytes per point, which its forward kernel (4 tiles
+        // per wavefront, 64 registers of gathered entries per point) no longer holds in registers (219 -> 736 us),
+        // while its gathers of a batch sorted by slab mostly hit the L1 anyway (records kernel 281 -> 256 us).
+        const int perChunk = parameterPrecision_ == Tensor::HALF ? 8 : 4;
+        const int chunks = divUp(dimension_ * numFeaturesPerLevel_, perChunk);
+        layout.derivativeBytesPerPoint = chunks <= 2 ? numLevels_ * chunks * 16 : 0;
+    }
     if (layout.recordsLdsBytes(points) > lds) return false;
     // every level gets about this many work items: the bucket of a slice that holds more than its share is split
     constexpr int ITEMS_PER_LEVEL = 32;

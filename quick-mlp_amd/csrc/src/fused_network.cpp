@@ -43,6 +43,12 @@ int FusedNetwork::MaxSharedMemoryBytes()
     return value;
 }
 
+static bool offersSlices(const IEncoding& e, IEncoding::GradientSliceLayout* layout = nullptr)
+{
+    IEncoding::GradientSliceLayout local;
+    return e.hasParameters() && e.gradientSlices(layout ? *layout : local);
+}
+
 FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
     : channelsIn_(cfg.at("num_inputs").get<int>())
     , channelsOut_(cfg.at("num_outputs").get<int>())
@@ -78,6 +84,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         compileOptions_.sortTraining = options.value("sort_training", compileOptions_.sortTraining);
         compileOptions_.directInput = options.value("direct_input", compileOptions_.directInput);
         compileOptions_.sliceGradients = options.value("slice_gradients", compileOptions_.sliceGradients);
+        compileOptions_.inputDerivatives = options.value("input_derivatives", compileOptions_.inputDerivatives);
         compileOptions_.fusedWeightUpdate = options.value("fused_weight_update", compileOptions_.fusedWeightUpdate);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
@@ -210,6 +217,25 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         offsetFwd += layers_[i].channelsOut;
     }
     perEntryForwardMemoryBytes_ = offsetFwd * static_cast<int>(sizeof(half));
+
+    // behind the intermediates: the position derivatives of the grids whose gradients take the slice kernels
+    derivativeOffsets_.assign(encodings_.size(), -1);
+    derivativeBytesPerPoint_ = 0;
+    if (compileOptions_.inputDerivatives != 0 && hasSliceGradients()) {
+        for (size_t i = 0; i < encodings_.size(); ++i) {
+            IEncoding::GradientSliceLayout layout;
+            if (!offersSlices(*encodings_[i], &layout) || layout.derivativeBytesPerPoint <= 0) continue;
+            derivativeOffsets_[i] = derivativeBytesPerPoint_;
+            derivativeBytesPerPoint_ += layout.derivativeBytesPerPoint;
+        }
+    }
+}
+
+bool FusedNetwork::storesDerivatives(int numel, int flags) const
+{
+    if (derivativeBytesPerPoint_ <= 0) return false;
+    if (compileOptions_.inputDerivatives > 0) return true;
+    return (flags & GRADIENTS_INPUT) && useSliceGradients(numel, flags);
 }
 
 FusedNetwork::~FusedNetwork()
@@ -592,12 +618,6 @@ int FusedNetwork::weightUpdateBlockSize() const
     return blockSize;
 }
 
-static bool offersSlices(const IEncoding& e, IEncoding::GradientSliceLayout* layout = nullptr)
-{
-    IEncoding::GradientSliceLayout local;
-    return e.hasParameters() && e.gradientSlices(layout ? *layout : local);
-}
-
 int FusedNetwork::weightUpdateSlices(int numTiles) const
 {
     const int waves = weightUpdateBlockSize() / WARP_SIZE;
@@ -693,7 +713,7 @@ static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
     return ss.str();
 }
 
-std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool registerStaging) const
+std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool registerStaging, bool derivatives) const
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string code = kl->findFile("qmlp/kernels/network_forward.h").value();
@@ -745,9 +765,23 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool r
             callEncodings << "            {\n                StageRowArray<f16, CHANNELS_IN> encodingOutputK[PPL];\n"
                           << "#pragma unroll\n                for (int q = 0; q < PPL; ++q) encodingOutputK[q] = encodingOutput[q] + "
                           << encodingOffset << ";\n                ";
-        callEncodings << e->qualifiedName() << "::template forwardBatch<PPL>(encodingInput, encodingOutputK";
-        if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
-        callEncodings << ");\n            }\n";
+        IEncoding::GradientSliceLayout sliceLayout;
+        if (derivatives && derivativeOffsets_[encodingIdx] >= 0 && offersSlices(*e, &sliceLayout)) {
+            // the lane's chunks of its first tile; the tiles of a wave follow one another
+            callEncodings << "static_assert(STORE && DERIVATIVES, \"this source is that of the training pass that keeps position derivatives\");\n"
+                          << "                typedef PositionDerivativeLayout<" << sliceLayout.configType << "> DerivativeLayout;\n"
+                          << "                StorePositionDerivatives<" << sliceLayout.configType << "> derivatives{\n"
+                          << "                    reinterpret_cast<DerivativeLayout::chunk_t*>(reinterpret_cast<unsigned char*>(forwardTmpMemoryH) + "
+                          << (static_cast<long long>(perEntryForwardMemoryBytes_) + derivativeOffsets_[encodingIdx]) << "ll * numel64)\n"
+                          << "                        + DerivativeLayout::chunkIndex(tile0 + tmpTileOffset, 0, 0, lane),\n"
+                          << "                    numTiles - tile0};\n                ";
+            callEncodings << e->qualifiedName() << "::template forwardBatch<PPL>(encodingInput, encodingOutputK, cEncoding" << encodingIdx
+                          << ", derivatives);\n            }\n";
+        } else {
+            callEncodings << e->qualifiedName() << "::template forwardBatch<PPL>(encodingInput, encodingOutputK";
+            if (e->hasParameters()) callEncodings << ", cEncoding" << encodingIdx;
+            callEncodings << ");\n            }\n";
+        }
         encodingOffset += e->numOutputChannels();
     }
     replaceAll(code, "$$CALL_ENCODINGS$$", callEncodings.str());
@@ -1162,9 +1196,10 @@ void FusedNetwork::forwardShape(bool store, int variant, int& blockSize, int& po
     }
 }
 
-void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnly)
+void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnly, bool derivatives)
 {
-    auto& slot = forwardKernels_[store ? 1 : 0][variant];
+    derivatives = derivatives && store;
+    auto& slot = forwardKernels_[derivatives ? 2 : store ? 1 : 0][variant];
     if (slot.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
@@ -1172,27 +1207,29 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
     const bool registerStaging = variant == VARIANT_REGISTERS;
     ck.sharedMemorySize = ldsParamHalves(false) * static_cast<int>(sizeof(half))
         + (ck.blockSize / WARP_SIZE) * (registerStaging ? 1 : ck.pointsPerLane) * stageBytesPerWave(false);
-    ck.fun = kl->getKernel(store ? "qmlp::kernel::NetworkKernelInferenceAndForward<true>"
-                                 : "qmlp::kernel::NetworkKernelInferenceAndForward<false>",
-                           forwardSource(ck.blockSize, ck.pointsPerLane, registerStaging), loaderFlags(compileOnly)).value();
+    ck.fun = kl->getKernel(derivatives ? "qmlp::kernel::NetworkKernelInferenceAndForward<true, true>"
+                           : store     ? "qmlp::kernel::NetworkKernelInferenceAndForward<true>"
+                                       : "qmlp::kernel::NetworkKernelInferenceAndForward<false>",
+                           forwardSource(ck.blockSize, ck.pointsPerLane, registerStaging, derivatives), loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
     QuickMLP::Instance().getLogger()->debug(
         "%s kernel, %d tile(s) per wave: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
-        store ? "forward" : "inference", ck.pointsPerLane, ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(),
+        derivatives ? "forward (with position derivatives)" : store ? "forward" : "inference", ck.pointsPerLane, ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(),
         ck.fun.scratchBytes(), ck.fullGrid);
     slot = std::move(ck);
 }
 
-const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles, bool noAlloc)
+const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles, bool noAlloc, bool derivatives)
 {
-    const int s = store ? 1 : 0;
+    derivatives = derivatives && store;
+    const int s = derivatives ? 2 : store ? 1 : 0;
     // loading a kernel allocates device memory: a call that must not allocate only takes what is loaded
     auto loaded = [&](int variant) -> const CompiledKernel& {
         if (noAlloc && !forwardKernels_[s][variant].has_value())
             throw std::runtime_error("The kernel for a batch of this size is not loaded yet, and loading allocates: run "
                                      "inference() once on a batch of the same size first");
-        compileForwardKernel(store, variant);
+        compileForwardKernel(store, variant, false, derivatives);
         return forwardKernels_[s][variant].value();
     };
     if (launchTiles) *launchTiles = numTiles;
@@ -1256,7 +1293,7 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
         QuickMLP::Instance().getLogger()->debug("the forward kernel with rows in registers spills %d bytes per lane, not used",
                                                 forwardKernels_[s][best].value().fun.scratchBytes());
         registerShapeSpills_[s] = true;
-        return forwardKernelFor(store, numTiles, launchTiles, noAlloc);
+        return forwardKernelFor(store, numTiles, launchTiles, noAlloc, derivatives);
     }
     return forwardKernels_[s][best].value();
 }
@@ -1327,10 +1364,16 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
             source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient.h");
             sk.recordsSource = source.str();
             sk.channelOffset = offset;
-            for (int points = layout.pointsPerWorkgroup; points >= std::min(128, layout.pointsPerWorkgroup); points /= 2)
+            for (int points = layout.pointsPerWorkgroup; points >= std::min(128, layout.pointsPerWorkgroup); points /= 2) {
                 sk.records.emplace_back();
+                sk.recordsFromDerivatives.emplace_back();
+            }
+            sk.derivativeOffset = derivativeOffsets_[i];
             if (compileOnly)
-                for (size_t v = 0; v < sk.records.size(); ++v) compileRecordsKernel(sk, flags, v, true);
+                for (size_t v = 0; v < sk.records.size(); ++v) {
+                    compileRecordsKernel(sk, flags, v, true);
+                    if ((flags & GRADIENTS_INPUT) && sk.derivativeOffset >= 0) compileRecordsKernel(sk, flags, v, true, true);
+                }
             sk.kernel.blockSize = 1024;
             sk.kernel.sharedMemorySize = layout.sliceFloats * static_cast<int>(sizeof(long long));
             sk.kernel.fun = kl->getKernel(format("qmlp::kernel::GridGradientSlicesKernel<%s, %d>", layout.configType.c_str(), layout.sliceFloats),
@@ -1373,7 +1416,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
     if (!compileOnly) backwardKernel_[flags][variant] = std::move(ak);
 }
 
-void FusedNetwork::compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly)
+void FusedNetwork::compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives)
 {
     const auto& layout = sk.layout;
     const int points = layout.pointsPerWorkgroup >> variant;
@@ -1381,17 +1424,19 @@ void FusedNetwork::compileRecordsKernel(SliceGradientKernel& sk, int flags, size
     ck.blockSize = points;
     ck.sharedMemorySize = layout.recordsLdsBytes(points);
     ck.fun = QuickMLP::Instance().kernelLoader()->getKernel(
-        format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d, %s>", layout.configType.c_str(), layers_[0].channelsIn,
-               sk.channelOffset, layout.sliceFloats, points, (flags & GRADIENTS_INPUT) ? "true" : "false"),
+        // (last argument: no input gradients | from gathers of all corners | from the position derivatives of the forward pass)
+        format("qmlp::kernel::GridGradientRecordsKernel<%s, %d, %d, %d, %d, %d>", layout.configType.c_str(), layers_[0].channelsIn,
+               sk.channelOffset, layout.sliceFloats, points, !(flags & GRADIENTS_INPUT) ? 0 : fromDerivatives ? 2 : 1),
         sk.recordsSource, loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
-    QuickMLP::Instance().getLogger()->debug("records kernel of encoding %d with %d points per workgroup: %d VGPRs, full grid %d",
-                                            sk.encoding, points, ck.fun.numVgprs(), ck.fullGrid);
-    sk.records[variant] = std::move(ck);
+    QuickMLP::Instance().getLogger()->debug("records kernel of encoding %d with %d points per workgroup%s: %d VGPRs, full grid %d",
+                                            sk.encoding, points, fromDerivatives ? " (stored position derivatives)" : "",
+                                            ck.fun.numVgprs(), ck.fullGrid);
+    (fromDerivatives ? sk.recordsFromDerivatives : sk.records)[variant] = std::move(ck);
 }
 
-const FusedNetwork::CompiledKernel& FusedNetwork::recordsKernelFor(SliceGradientKernel& sk, int flags, int numel)
+const FusedNetwork::CompiledKernel& FusedNetwork::recordsKernelFor(SliceGradientKernel& sk, int flags, int numel, bool fromDerivatives)
 {
     // The table entries that a workgroup gathers for the input gradients and the records it writes pass through
     // one compute unit's memory pipeline: a batch that fills fewer workgroups than there are compute units leaves
@@ -1400,8 +1445,9 @@ const FusedNetwork::CompiledKernel& FusedNetwork::recordsKernelFor(SliceGradient
     const int computeUnits = KernelFunction::computeUnits();
     size_t variant = 0;
     while (variant + 1 < sk.records.size() && divUp(numel, sk.layout.pointsPerWorkgroup >> variant) < computeUnits) ++variant;
-    if (!sk.records[variant].has_value()) compileRecordsKernel(sk, flags, variant, false);
-    return sk.records[variant].value();
+    auto& kernels = fromDerivatives ? sk.recordsFromDerivatives : sk.records;
+    if (!kernels[variant].has_value()) compileRecordsKernel(sk, flags, variant, false, fromDerivatives);
+    return kernels[variant].value();
 }
 
 void FusedNetwork::precompile(int adjointFlags)
@@ -1413,6 +1459,15 @@ void FusedNetwork::precompile(int adjointFlags)
         if (ppl > 1) compileForwardKernel(store, VARIANT_NARROW, true);
         if (hasLargeVariant(store)) compileForwardKernel(store, VARIANT_LARGE, true);
         if (registerVariantTiles(store) > 0) compileForwardKernel(store, VARIANT_REGISTERS, true);
+    }
+    if (adjointFlags > 0 && storesDerivatives(1 << 30, adjointFlags)) {
+        // training passes that keep the position derivatives of their grids
+        compileForwardKernel(true, VARIANT_DEFAULT, true, true);
+        int ppl = 1;
+        forwardBlockSize(-1, false, &ppl);
+        if (ppl > 1) compileForwardKernel(true, VARIANT_NARROW, true, true);
+        if (hasLargeVariant(true)) compileForwardKernel(true, VARIANT_LARGE, true, true);
+        if (registerVariantTiles(true) > 0) compileForwardKernel(true, VARIANT_REGISTERS, true, true);
     }
     if (adjointFlags > 0) {
         if (compileOptions_.sliceGradients <= 0 || !hasSliceGradients() || !(adjointFlags & GRADIENTS_INPUT_ENCODINGS))
@@ -1511,7 +1566,7 @@ void FusedNetwork::inferenceNoAlloc(const Tensor& input, Tensor& output, stream_
     launchForward(false, input, output, nullptr, stream, true);
 }
 
-void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc)
+void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc, bool derivatives)
 {
     const int numel = input.size(0);
     int tmpNumTiles = divUp(numel, TILE_POINTS);
@@ -1527,7 +1582,7 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     for (long long start = 0; start < numel;) {
         // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
         int launchTiles = 0;
-        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, noAlloc);
+        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, noAlloc, derivatives);
         int count = static_cast<int>(std::min<long long>(
             {static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS, numel - start}));
         auto inputAcc = inputAll;
@@ -1579,10 +1634,12 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
     CHECK_ERROR(adjointFlags >= 0 && adjointFlags < ADJOINT_MODE_MAX_COMBINATIONS, "prepare(): unknown adjoint flags ", adjointFlags);
     if (numel == 0) return;
     // the forward kernels that launchForward() takes for the pieces of a batch of this size
+    if (adjointFlags > 0) announcedFlags_ = adjointFlags;
     for (int store = 0; store <= (adjointFlags > 0 ? 1 : 0); ++store)
         for (long long start = 0; start < numel;) {
             int launchTiles = 0;
-            const auto& ck = forwardKernelFor(store != 0, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles);
+            const auto& ck = forwardKernelFor(store != 0, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, false,
+                                              store != 0 && storesDerivatives(numel, adjointFlags));
             start += std::min<long long>({static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS,
                                           numel - start});
         }
@@ -1605,7 +1662,7 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
         const bool sliceGradients = useSliceGradients(numel, adjointFlags);
         compileBackwardKernel(adjointFlags, sliceGradients);
         for (auto& sk : backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value().sliceGradients)
-            (void)recordsKernelFor(sk, adjointFlags, numel);
+            (void)recordsKernelFor(sk, adjointFlags, numel, storesDerivatives(numel, adjointFlags) && sk.derivativeOffset >= 0);
         // the streams and events on which the weight-update kernels of the layers run side by side
         if ((adjointFlags & GRADIENTS_NETWORK_WEIGHTS) && compileOptions_.parallelWeightUpdate && layers_.size() > 1) ensureStreams();
     }
@@ -1619,7 +1676,7 @@ bool FusedNetwork::sortsTraining(int numel) const
 
 size_t FusedNetwork::sortedRowsOffset(int numel) const
 {
-    return roundUp(static_cast<size_t>(perEntryForwardMemoryBytes_) * static_cast<size_t>(roundUp(numel, WARP_SIZE)), size_t(256));
+    return roundUp(forwardBytesPerPoint() * static_cast<size_t>(roundUp(numel, WARP_SIZE)), size_t(256));
 }
 
 bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
@@ -1703,12 +1760,14 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
 
 size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlags)
 {
-    (void)adjointFlags;
-    // a batch that trains in sorted order: its sorted rows and the order, behind the intermediates
+    // The size does not depend on the flags (a caller may size the memory once for several kinds of passes); they
+    // announce what the adjoint pass will ask for, which decides whether forward() stores position derivatives.
+    if (adjointFlags > 0 && adjointFlags < ADJOINT_MODE_MAX_COMBINATIONS) announcedFlags_ = adjointFlags;
+    // a batch that trains in sorted order: its sorted rows and the order, behind the intermediates and the derivatives
     if (sortsTraining(numElements))
         return sortedRowsOffset(numElements) + roundUp(static_cast<size_t>(numElements) * (channelsIn() + 1) * sizeof(float), size_t(256));
     numElements = roundUp(numElements, WARP_SIZE);
-    return static_cast<size_t>(perEntryForwardMemoryBytes_) * static_cast<size_t>(numElements);
+    return forwardBytesPerPoint() * static_cast<size_t>(numElements);
 }
 
 size_t FusedNetwork::forwardMemory(const Tensor& input, AdjointModeFlags adjointFlags)
@@ -1734,7 +1793,10 @@ void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory,
     CHECK_ERROR(tmpMemory != nullptr, "forward() needs temporary memory of forwardMemory() bytes");
     CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemory) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
 
-    launchForward(true, input, output, static_cast<half*>(tmpMemory), stream);
+    const bool derivatives = storesDerivatives(numel, announcedFlags_);
+    if (derivatives) derivativesStored_[tmpMemory] = numel;
+    else derivativesStored_.erase(tmpMemory);
+    launchForward(true, input, output, static_cast<half*>(tmpMemory), stream, false, derivatives);
 }
 
 void FusedNetwork::zeroGradients()
@@ -1831,6 +1893,13 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
 
     const bool sliceGradients = useSliceGradients(numel, adjointFlags);
     CHECK_ERROR(!sliceGradients || numel < (1 << 27), "batches of 2^27 points or more: set options.slice_gradients to 0");
+    announcedFlags_ = adjointFlags;
+    // whether the forward pass that wrote this forward memory kept the position derivatives of the grids
+    bool derivativesStored = false;
+    {
+        const auto it = derivativesStored_.find(tmpMemoryForward);
+        derivativesStored = hasInputGradients && sliceGradients && it != derivativesStored_.end() && it->second == numel;
+    }
     const bool sortedPoints = sortsTraining(numel);
     compileBackwardKernel(adjointFlags, sliceGradients);
     auto& ak = backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value();
@@ -1938,8 +2007,11 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
             {
                 // the records kernel walks over the real points, but lays its buckets out for the padded batch
                 auto adjInputAcc = sortedAdjInput;   // this grid's share of dL/dinput (zeros in it if none is asked for: unused)
-                void* args[] = {&numel, &numelPadded, &inputAcc, &adjEncoded, params.data(), &records, &cursors, &adjInputAcc};
-                const CompiledKernel& rk = recordsKernelFor(sk, adjointFlags, numel);
+                const bool fromDerivatives = derivativesStored && sk.derivativeOffset >= 0;
+                const void* derivatives = static_cast<const char*>(tmpMemoryForward)
+                    + (static_cast<long long>(perEntryForwardMemoryBytes_) + std::max(0ll, sk.derivativeOffset)) * numel64;
+                void* args[] = {&numel, &numelPadded, &inputAcc, &adjEncoded, params.data(), &records, &cursors, &adjInputAcc, &derivatives};
+                const CompiledKernel& rk = recordsKernelFor(sk, adjointFlags, numel, fromDerivatives);
                 rk.fun.launch(std::min(divUp(numel, rk.blockSize), rk.fullGrid), rk.blockSize, rk.sharedMemorySize, stream, args);
             }
             const uint32_t* recordsRead = records;

@@ -503,10 +503,13 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
             "network": [{"n_out": 32, "bias": True, "activation": "celu"},
                         {"n_out": 2, "bias": False, "activation": "identity"}]}
     cases = {}
-    warm_cache(*[dict(base, options={"slice_gradients": mode}) for mode in (0, 1)])
-    for mode in (0, 1):
+    # 0: atomics; 1: slices; 2: slices, and the input gradients from a second gather of the table as in mode 0
+    # instead of from the position derivatives that the forward pass of mode 1 keeps
+    options = {0: {"slice_gradients": 0}, 1: {"slice_gradients": 1}, 2: {"slice_gradients": 1, "input_derivatives": 0}}
+    warm_cache(*[dict(base, options=o) for o in options.values()])
+    for mode, o in options.items():
         cfg = json.loads(json.dumps(base))
-        cfg["options"] = {"slice_gradients": mode}
+        cfg["options"] = o
         cases[mode] = Case(cfg)
     rng = np.random.default_rng(12)
     params = random_parameters(cases[0].oracle, rng)
@@ -527,15 +530,27 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
         X = (lo + sz * u).astype(np.float32)
         adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
         for flags in (FLAG_ENC, FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC):
-            got = {mode: c.gpu_train(X, adj, flags) for mode, c in cases.items()}
+            got = {mode: c.gpu_train(X, adj, flags) for mode, c in cases.items() if mode < 2 or flags & FLAG_INPUT}
             a, b = got[0]["table_grads"][1], got[1]["table_grads"][1]
             scale = max(1.0, float(np.abs(a).max()))
             assert np.allclose(a / scale, b / scale, rtol=1e-4, atol=2e-6), "N=%d flags=%d: %g" % (N, flags, np.abs(a - b).max())
             if flags & FLAG_WEIGHTS:
-                assert np.array_equal(got[0]["grads"], got[1]["grads"])
-                assert np.array_equal(got[0]["adj_x"], got[1]["adj_x"])
-            # (weight and input gradients are those of the other mode bit for bit: checked against the oracle elsewhere)
+                assert np.array_equal(got[0]["grads"], got[1]["grads"]) and np.array_equal(got[0]["grads"], got[2]["grads"])
+                # gathered a second time, in the same order of operations: the bits of the atomic path
+                assert np.array_equal(got[0]["adj_x"], got[2]["adj_x"])
+                # (fixed-point sums, but entries next to a slice boundary and coarse levels also receive float atomics)
+                assert np.allclose(got[1]["table_grads"][1] / scale, got[2]["table_grads"][1] / scale, rtol=1e-4, atol=2e-6)
+                # from the stored derivatives (kept in the precision of the table: relative 2^-11 each for half)
+                sx = float(np.abs(got[0]["adj_x"]).max())
+                assert np.allclose(got[1]["adj_x"] / sx, got[0]["adj_x"] / sx, rtol=2e-3, atol=1e-3 if precision == "half" else 1e-5)
+                assert np.array_equal(got[1]["out"], got[2]["out"])
+            # (weight gradients are those of the other mode bit for bit: checked against the oracle elsewhere)
             check_gradients(cases[1], X, adj, FLAG_ENC, got[1], what="slices, N=%d flags=%d: " % (N, flags))
+            if N == 3000 and flags & FLAG_INPUT:
+                # the input gradients from the stored derivatives against the fp32 evaluation, at the tolerance of the target
+                ref = cases[1].oracle.backward(X, adj, FLAG_INPUT, round_mode=0)
+                sx = max(1.0, float(np.abs(ref["adj_x"]).max()))
+                assert_close(got[1]["adj_x"] / sx, ref["adj_x"] / sx, "input gradients from stored derivatives vs fp32 oracle")
     # Points several box widths outside are extrapolated with weights far above one (the reference does not clamp the
     # fractional position either; 3 widths outside a level of resolution 128: |w| up to 5e7 in 3-D), while the
     # fixed-point sums of the slice kernel count on weights of at most one: the records kernel adds such records to
@@ -557,7 +572,7 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
         touched[far_idx.cpu().numpy().astype(np.int64).ravel() + f] = True
     largest = float(far_w.abs().max())
     assert largest > 100
-    got = {mode: c.gpu_train(X, adj, FLAG_ENC) for mode, c in cases.items()}
+    got = {mode: c.gpu_train(X, adj, FLAG_ENC) for mode, c in cases.items() if mode < 2}
     a, b = got[0]["table_grads"][1], got[1]["table_grads"][1]
     assert np.isfinite(a).all() and np.isfinite(b).all()
     scale = float(np.abs(a[~touched]).max())
@@ -566,7 +581,7 @@ def test_grid_gradients_summed_by_slices_match_the_atomic_scatter_and_the_oracle
     assert np.abs(a[touched]).max() < noise and np.abs(b[touched]).max() < noise, (np.abs(a[touched]).max(), np.abs(b[touched]).max())
     X = (lo + sz * rng.uniform(0, 1, (N, n_in))).astype(np.float32)
     X[5, 1] = np.nan
-    got = {mode: c.gpu_train(X, adj, FLAG_ENC) for mode, c in cases.items()}
+    got = {mode: c.gpu_train(X, adj, FLAG_ENC) for mode, c in cases.items() if mode < 2}
     a, b = got[0]["table_grads"][1], got[1]["table_grads"][1]
     assert np.isnan(a).any() and np.array_equal(np.isnan(a), np.isnan(b))
     ok = ~np.isnan(a)
@@ -793,7 +808,7 @@ def test_full_size_properties_cfg3_train():
                  allowed_fraction=2e-2)
     # At this size the grid gradients are summed by slices and the input gradients come from the records
     # kernel; the same network with the scatter inside the backward kernel (one atomic per contribution):
-    # outputs and input gradients bit for bit, weight and grid gradients up to the order of the fp32 additions.
+    # outputs bit for bit, weight and grid gradients up to the order of the fp32 additions.
     cfg = json.loads(json.dumps(bc.CONFIGS[3]["cfg"]))
     cfg.setdefault("options", {})["slice_gradients"] = 0
     scatter = Case(cfg, bc.ORACLE_ACTIVATIONS)
@@ -801,7 +816,10 @@ def test_full_size_properties_cfg3_train():
     scatter.set_table(0, case.tables_np[0])
     c = scatter.gpu_train(X, adj, flags)
     assert np.array_equal(c["out"], a["out"])
-    assert np.array_equal(c["adj_x"], a["adj_x"])
+    # (the input gradients of the slice path come from the position derivatives that its forward pass kept as halves,
+    # those of the scatter path from a second gather: 2^-11 relative per derivative)
+    sx = float(np.abs(c["adj_x"]).max())
+    assert np.allclose(a["adj_x"] / sx, c["adj_x"] / sx, rtol=2e-3, atol=1e-3)
     # (the backward kernel in front of the slice kernels sums the weight gradients of all layers itself, the one that
     # scatters leaves them to the weight-update kernels: the same products in another order of the fp32 sums)
     scale = float(np.abs(c["grads"]).max())
@@ -1170,3 +1188,82 @@ def test_sorted_inference_of_a_two_level_dense_grid_in_several_launches():
     sample = np.arange(0, N, 5003)
     ref = sorted_.oracle.forward(X[sample])
     assert_close(a[sample], ref, "sampled oracle check", allowed_fraction=2e-3)
+
+
+def test_position_derivatives_are_kept_when_input_gradients_are_announced():
+    """options.input_derivatives (default: when announced): a training pass whose adjoint flags ask for input and
+    grid gradients also keeps, per point and level, the derivatives of the level's features with respect to the
+    position, and the adjoint pass forms the grid's share of dL/dinput from them instead of gathering every corner
+    a second time. Which of the two ran shows in the bits: the gather repeats the operations of the atomic path
+    (bit-identical to it), the stored derivatives are halves (2^-11 relative each)."""
+    grid = {"id": "HashGrid", "start_in": 0, "n_in": 3, "n_levels": 8, "n_features_per_level": 2,
+            "log2_hashmap_size": 12, "min_resolution": 4, "max_resolution": 256, "combination_mode": "concat",
+            "bounding_box_min": [-0.5, 0.0, 0.25], "bounding_box_size": [1.0, 2.0, 0.5], "parameter_precision": "half"}
+    base = {"num_inputs": 3, "num_outputs": 2, "activation_specification": ["qmlp/builtin-activations.json"],
+            "encodings": [grid],
+            "network": [{"n_out": 32, "bias": True, "activation": "celu"}, {"n_out": 2, "bias": False, "activation": "identity"}]}
+    options = {"auto": {"slice_gradients": 1}, "never": {"slice_gradients": 1, "input_derivatives": 0},
+               "always": {"slice_gradients": 1, "input_derivatives": 1}}
+    warm_cache(*[dict(base, options=o) for o in options.values()])
+    cases = {k: Case(dict(base, options=o)) for k, o in options.items()}
+    rng = np.random.default_rng(31)
+    params = random_parameters(cases["auto"].oracle, rng)
+    table = rng.uniform(-1, 1, cases["auto"].oracle.encodings[0][1].n_params)
+    for c in cases.values():
+        c.set_parameters(params)
+        c.set_table(0, table)
+    N = 5000
+    lo, sz = np.array(grid["bounding_box_min"], np.float32), np.array(grid["bounding_box_size"], np.float32)
+    X = (lo + sz * rng.uniform(0, 1, (N, 3))).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+    x, a = torch.from_numpy(X).cuda(), torch.from_numpy(adj).cuda()
+    gathered = cases["never"].gpu_train(X, adj, 7)["adj_x"]
+    sx = float(np.abs(gathered).max())
+
+    def adjoint(case, tmp, flags=7):
+        adj_x, _, _ = case.net.adjoint_raw(x, a, flags, tmp, case.params, case.encoding_parameters())
+        torch.cuda.synchronize()
+        return adj_x.cpu().numpy()
+
+    def from_derivatives(got):
+        assert np.allclose(got / sx, gathered / sx, rtol=2e-3, atol=1e-3)
+        return not np.array_equal(got, gathered)
+
+    auto, always = cases["auto"], cases["always"]
+    # the same size of forward memory whatever the flags: 16 bytes per point and level behind the intermediates
+    assert auto.net.forward_memory(N, 6) == auto.net.forward_memory(N, 7) == cases["never"].net.forward_memory(N, 7) + 8 * 16 * 5056
+    # announced with the forward memory: stored and used
+    _, tmp7 = auto.net.forward_raw(x, auto.params, auto.encoding_parameters(), 7)
+    assert from_derivatives(adjoint(auto, tmp7))
+    # a pass that announced no input gradients keeps none; an adjoint pass that asks for them anyway gathers
+    _, tmp6 = auto.net.forward_raw(x, auto.params, auto.encoding_parameters(), 6)
+    assert not from_derivatives(adjoint(auto, tmp6))
+    # ... while the memory of the earlier pass still holds its derivatives
+    assert from_derivatives(adjoint(auto, tmp7))
+    # the flags of the last adjoint pass count as announced too: forward() of the C ABI alone
+    out = torch.empty((N, 2), device="cuda")
+    tmp = torch.empty(auto.net.forward_memory(N, 0), dtype=torch.uint8, device="cuda")
+    import ctypes
+    from qmlp import _lib
+    _lib.check(_lib.lib.qmlp_network_forward(auto.net._handle, _lib.desc(x), _lib.desc(out), ctypes.c_void_p(tmp.data_ptr()),
+                                              _lib.current_stream(x.device)))
+    assert from_derivatives(adjoint(auto, tmp))
+    # another batch into the same memory, without derivatives: those of the old batch are not taken for it
+    M = 3000
+    xs, as_ = x[:M].contiguous(), a[:M].contiguous()
+    assert auto.net.forward_memory(M, 6) <= tmp7.numel()
+    _lib.check(_lib.lib.qmlp_network_forward(auto.net._handle, _lib.desc(xs), _lib.desc(out[:M]), ctypes.c_void_p(tmp7.data_ptr()),
+                                              _lib.current_stream(x.device)))
+    small, _, _ = auto.net.adjoint_raw(xs, as_, 7, tmp7, auto.params, auto.encoding_parameters())
+    assert np.array_equal(small.cpu().numpy(), cases["never"].gpu_train(X[:M], adj[:M], 7)["adj_x"])
+    _, tmp7 = auto.net.forward_raw(x, auto.params, auto.encoding_parameters(), 7)
+    # always: also when nothing was announced
+    _, tmp6 = always.net.forward_raw(x, always.params, always.encoding_parameters(), 6)
+    assert from_derivatives(adjoint(always, tmp6))
+    # input gradients alone (no grid gradients: no records kernel) come from the backward kernel's own gathers
+    only = adjoint(auto, tmp7, flags=1)
+    assert np.array_equal(only, cases["never"].gpu_train(X, adj, 1)["adj_x"])
+    # against the fp32 oracle, at the tolerance of the target
+    ref = auto.oracle.backward(X, adj, FLAG_INPUT, round_mode=0)
+    s = max(1.0, float(np.abs(ref["adj_x"]).max()))
+    assert_close(adjoint(auto, tmp7) / s, ref["adj_x"] / s, "input gradients from stored derivatives vs fp32 oracle")

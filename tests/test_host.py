@@ -155,15 +155,23 @@ def test_temporary_memory_of_a_batch_that_trains_in_sorted_order():
     for m in (1, 1000, (1 << 19) - 1):
         assert net.forward_memory(m, 7) == given.forward_memory(m, 7)
         assert net.adjoint_memory(m, 7) == given.adjoint_memory(m, 7)
-    # a hashed grid never sorts
+    # a hashed grid never sorts (behind its intermediates: 16 bytes per point and level for the derivatives of
+    # the level's 2 features with respect to the 3 coordinates)
     hashed = qmlp.Network(json.dumps(bc.CONFIGS[3]["cfg"]))
-    assert hashed.forward_memory(n, 7) == 2 * (32 + 64 + 64 + 16) * n
+    assert hashed.forward_memory(n, 7) == (2 * (32 + 64 + 64 + 16) + 16 * 16) * n
 
 
 def test_temporary_memory_sizes():
     net = qmlp.Network(json.dumps(bc.CONFIGS[3]["cfg"]))
-    per_fwd = 2 * (32 + 64 + 64 + 16)
+    # intermediates; position derivatives of the grid (3 x 2 halves in one chunk of 16 bytes per level), whatever
+    # the flags: a caller may size the memory once for several kinds of passes
+    per_fwd = 2 * (32 + 64 + 64 + 16) + 16 * 16
     per_adj = 2 * (64 + 64 + 16)
+    plain = json.loads(json.dumps(bc.CONFIGS[3]["cfg"]))
+    plain["options"] = {"input_derivatives": 0}
+    plain = qmlp.Network(json.dumps(plain))
+    assert plain.forward_memory(1 << 18, 7) == 2 * (32 + 64 + 64 + 16) << 18
+    assert net.forward_memory(1 << 18, 2) == net.forward_memory(1 << 18, 7)
     # behind the adjoint pre-activations: fp32 partial weight gradients of up to 512 batch
     # slices (one workgroup of 4 wavefronts = 4 tiles each)
     n_params = net.num_network_parameters()
@@ -264,10 +272,11 @@ def test_kernels_compile_for_gfx950_without_a_gpu_and_are_cached(tmp_path):
         # inference and forward in four shapes (4x2, 4x1, 8x4 and 8x8 wavefronts x tiles, the last
         # with its encoded rows in registers), backward with the atomic scatter and backward for the
         # gradient slices, the records kernel of the grid for workgroups of 1024, 512, 256 and 128 points and
-        # its slice kernel, 2 weight updates + reduce
-        assert c1 - c0 == 18 and h1 == h0
+        # its slice kernel, 2 weight updates + reduce; for training passes that keep the position derivatives of
+        # the grid: forward in the four shapes once more, and the four records kernels that read them
+        assert c1 - c0 == 26 and h1 == h0
         files = os.listdir(cache)
-        assert len(files) == 18 and all(f.endswith(".co") for f in files)
+        assert len(files) == 26 and all(f.endswith(".co") for f in files)
         qmlp.Network(json.dumps(cfg)).precompile(7)
         c2, h2 = qmlp._lib.kernel_cache_stats()
         assert c2 == c1                            # nothing recompiled (memory or disk cache)
