@@ -73,6 +73,7 @@ public:
     [[nodiscard]] int parameterCount() const override;
     [[nodiscard]] int ldsGradientFloats(int maxBytes, int& levels) const override;
     [[nodiscard]] bool gradientSlices(GradientSliceLayout& layout) const override;
+    [[nodiscard]] bool gradientColumns(const kernel::PointOrderKey& key, GradientColumnLayout& layout) const override;
     [[nodiscard]] int numSweptTables() const override { return numLevels_; }
     [[nodiscard]] int gatherRegistersPerPoint() const override;
     [[nodiscard]] bool pointOrderKey(kernel::PointOrderKey& key, long long numPoints = 0) const override;
@@ -114,7 +115,7 @@ public:
 
 private:
     [[nodiscard]] std::string configName() const;
-    std::optional<KernelFunction> cornersKernel_[4];
+    std::optional<KernelFunction> cornersKernel_[5];
 };
 
 QUICKMLP_NAMESPACE_END

@@ -87,6 +87,11 @@ public:
         // 0: never (no room for them in the forward memory either); >0: every training pass.
         int inputDerivatives = -1;
 
+        // Parameter gradients of a dense single-level grid whose batch trains sorted by grid slab: summed owner by
+        // owner of the grid's nodes in LDS, without gradient records (kernels/grid_gradient_columns.h).
+        // <0 (default) and >0: wherever the encoding offers it; 0: never (records and slices as for other grids).
+        int columnGradients = -1;
+
         // Gradients of the layer weights: summed inside the backward kernel, which holds the adjoint
         // pre-activations in registers (Layer::weightGradient), instead of by one kernel per layer that reads
         // them back from memory. <0 (default): the layers with the fewest gradient tiles, up to 16 tiles (64
@@ -158,6 +163,8 @@ private:
     PointOrder pointOrder_;
     /** Smaller batches are never sorted when sortPoints < 0; larger ones if the encoding expects a gain. */
     static constexpr int SORT_POINTS_MIN_BATCH = 1 << 19;
+    /** Slabs of the sort (POINT_ORDER_MAX_SLABS of kernels/point_order.h). */
+    static constexpr int SORT_SLABS = 1024;
     /**
      * Sorts the batch by the slab key of the first encoding that offers one.
      * \return false if the batch stays as it is; else sortedInput views the sorted copy and
@@ -213,6 +220,12 @@ private:
         int channelOffset = 0;
         CompiledKernel kernel;       // GridGradientSlicesKernel
         Tensor items;                // device copy of layout.items
+        // For batches that train sorted by grid slab, where the encoding offers it: the kernels of
+        // kernels/grid_gradient_columns.h (compiled on first use), which take the place of records and slices
+        bool columnsOffered = false;
+        IEncoding::GradientColumnLayout columnLayout;
+        std::optional<CompiledKernel> columnsPlan;
+        std::optional<CompiledKernel> columns[2];   // [1]: input gradients from the position derivatives of the forward pass
     };
     struct AdjointKernel
     {
@@ -418,6 +431,12 @@ private:
     void compileBackwardKernel(int flags, bool sliceGradients = false, bool compileOnly = false);
     /** The records kernel of a batch of numel points (compiled on first use; compileOnly: all of them into the cache). */
     const CompiledKernel& recordsKernelFor(SliceGradientKernel& sk, int flags, int numel, bool fromDerivatives = false);
+    /** Compiles (compileOnly: into the cache) or loads the two kernels of kernels/grid_gradient_columns.h for sk. */
+    void compileColumnKernels(SliceGradientKernel& sk, int flags, bool compileOnly, bool fromDerivatives = false);
+    /** Bytes at the start of the slice workspace that the column kernels use: slab starts, the number of work items, the items. */
+    static size_t columnWorkspaceBytes(const IEncoding::GradientColumnLayout& layout, long long numel, int* maxItems = nullptr);
+    /** The slab totals of the sort of a training pass: behind the sorted rows and the order in the forward memory. */
+    size_t sortedTotalsOffset(int numel) const;
     void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false, bool derivatives = false) const;

@@ -161,6 +161,26 @@ public:
             return n;
         }
     };
+    /** What the host needs to run the kernels of kernels/grid_gradient_columns.h for an encoding. */
+    struct GradientColumnLayout
+    {
+        std::string configType;      // device type of the level table
+        int cellsPerSlab = 0;        // cells per slab and sorted coordinate (the kernels' CPS)
+        int owners = 0;              // owners per sorted coordinate: workgroups that share out the nodes of the grid
+        int ldsBytes = 0;            // 64-bit sums of one owner
+    };
+    /**
+     * Encodings whose parameter gradients, for a batch that is sorted by the slabs of `key` (pointOrderKey()), can
+     * be summed owner by owner in LDS without any records (see kernels/grid_gradient_columns.h) return true and
+     * fill in the layout.
+     */
+    [[nodiscard]] virtual bool gradientColumns(const kernel::PointOrderKey& key, GradientColumnLayout& layout) const
+    {
+        (void)key;
+        (void)layout;
+        return false;
+    }
+
     /**
      * Encodings whose parameter gradients can be summed slice by slice in LDS instead of being
      * scattered with global atomics (see kernels/grid_gradient.h) return true and fill in the layout.

@@ -370,6 +370,30 @@ bool EncodingHashGrid::gradientSlices(GradientSliceLayout& layout) const
     return true;
 }
 
+bool EncodingHashGrid::gradientColumns(const kernel::PointOrderKey& key, GradientColumnLayout& layout) const
+{
+    // one dense level whose batch is sorted by slabs of whole cells of its first two coordinates
+    if (numLevels_ != 1 || layers_[0].hashed || dimension_ < 2 || dimension_ > 4) return false;
+    kernel::PointOrderKey own{};
+    if (!pointOrderKey(own, 0) || own.slabs2 != 1 || own.slabs0 != own.slabs1) return false;
+    if (key.channel0 != own.channel0 || key.channel1 != own.channel1 || key.slabs0 != own.slabs0 || key.slabs1 != own.slabs1
+        || key.slabs2 != own.slabs2 || key.scale0 != own.scale0 || key.scale1 != own.scale1 || key.min0 != own.min0 || key.min1 != own.min1)
+        return false;   // sorted for another encoding
+    const int nodes = layers_[0].resolution;
+    const int cells = std::max(1, nodes - 1);
+    const int cellsPerSlab = divUp(cells, own.slabs0);
+    if (divUp(cells, cellsPerSlab) != own.slabs0) return false;
+    long long sums = static_cast<long long>(cellsPerSlab) * cellsPerSlab * numFeaturesPerLevel_;
+    for (int d = 2; d < dimension_; ++d) sums *= nodes;
+    // two workgroups of an owner's 64-bit sums per compute unit
+    if (sums * 8 > (FusedNetwork::MaxSharedMemoryBytes() - 1024) / 2) return false;
+    layout.configType = "qmlp::kernel::" + configName();
+    layout.cellsPerSlab = cellsPerSlab;
+    layout.owners = divUp(nodes, cellsPerSlab);
+    layout.ldsBytes = static_cast<int>(sums * 8);
+    return true;
+}
+
 void EncodingHashGrid::setParameter(const Tensor& tensor, Tensor::Usage usage)
 {
     if (tensor.defined()) {

@@ -85,6 +85,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         compileOptions_.directInput = options.value("direct_input", compileOptions_.directInput);
         compileOptions_.sliceGradients = options.value("slice_gradients", compileOptions_.sliceGradients);
         compileOptions_.inputDerivatives = options.value("input_derivatives", compileOptions_.inputDerivatives);
+        compileOptions_.columnGradients = options.value("column_gradients", compileOptions_.columnGradients);
         compileOptions_.fusedWeightUpdate = options.value("fused_weight_update", compileOptions_.fusedWeightUpdate);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
@@ -1369,6 +1370,16 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
                 sk.recordsFromDerivatives.emplace_back();
             }
             sk.derivativeOffset = derivativeOffsets_[i];
+            {
+                // batches that train sorted by the slabs of this grid
+                kernel::PointOrderKey key{};
+                sk.columnsOffered = compileOptions_.columnGradients != 0 && compileOptions_.sortTraining && compileOptions_.sortPoints != 0
+                    && channelsIn() <= 16 && e->pointOrderKey(key, 0) && e->gradientColumns(key, sk.columnLayout);
+                if (sk.columnsOffered && compileOnly) {
+                    compileColumnKernels(sk, flags, true);
+                    if ((flags & GRADIENTS_INPUT) && sk.derivativeOffset >= 0) compileColumnKernels(sk, flags, true, true);
+                }
+            }
             if (compileOnly)
                 for (size_t v = 0; v < sk.records.size(); ++v) {
                     compileRecordsKernel(sk, flags, v, true);
@@ -1434,6 +1445,43 @@ void FusedNetwork::compileRecordsKernel(SliceGradientKernel& sk, int flags, size
                                             sk.encoding, points, fromDerivatives ? " (stored position derivatives)" : "",
                                             ck.fun.numVgprs(), ck.fullGrid);
     (fromDerivatives ? sk.recordsFromDerivatives : sk.records)[variant] = std::move(ck);
+}
+
+void FusedNetwork::compileColumnKernels(SliceGradientKernel& sk, int flags, bool compileOnly, bool fromDerivatives)
+{
+    fromDerivatives = fromDerivatives && (flags & GRADIENTS_INPUT) && sk.derivativeOffset >= 0;
+    if (sk.columns[fromDerivatives ? 1 : 0].has_value() && !compileOnly) return;
+    auto kl = QuickMLP::Instance().kernelLoader();
+    std::stringstream source;
+    encodings_[sk.encoding]->fillCode(source);
+    source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient_columns.h");
+    const auto& layout = sk.columnLayout;
+    CompiledKernel plan, columns;
+    plan.blockSize = 1024;
+    plan.fun = kl->getKernel(format("qmlp::kernel::GridGradientColumnsPlan<%s, %d>", layout.configType.c_str(), layout.cellsPerSlab),
+                             source.str(), loaderFlags(compileOnly)).value();
+    columns.blockSize = 512;
+    columns.sharedMemorySize = layout.ldsBytes;
+    columns.fun = kl->getKernel(format("qmlp::kernel::GridGradientColumnsKernel<%s, %d, %d, %d, %d, %d>", layout.configType.c_str(),
+                                       layout.cellsPerSlab, layers_[0].channelsIn, sk.channelOffset,
+                                       !(flags & GRADIENTS_INPUT) ? 0 : fromDerivatives ? 2 : 1, columns.blockSize),
+                                source.str(), loaderFlags(compileOnly)).value();
+    if (compileOnly) return;
+    QuickMLP::Instance().getLogger()->debug("column kernel of encoding %d: %d x %d owners, LDS %d bytes, %d VGPRs, %d bytes scratch",
+                                            sk.encoding, layout.owners, layout.owners, layout.ldsBytes, columns.fun.numVgprs(),
+                                            columns.fun.scratchBytes());
+    sk.columnsPlan = std::move(plan);
+    sk.columns[fromDerivatives ? 1 : 0] = std::move(columns);
+}
+
+size_t FusedNetwork::columnWorkspaceBytes(const IEncoding::GradientColumnLayout& layout, long long numel, int* maxItems)
+{
+    // as kernels/grid_gradient_columns.h: an owner is split into parts of GRID_GRADIENT_COLUMNS_PART_POINTS points, and
+    // every point is visited by at most four owners
+    constexpr long long PART_POINTS = 24 * 1024;
+    const long long items = static_cast<long long>(layout.owners) * layout.owners + 4 * numel / PART_POINTS + 4;
+    if (maxItems) *maxItems = static_cast<int>(items);
+    return roundUp(static_cast<size_t>(SORT_SLABS + 1 + 1) * sizeof(int), size_t(256)) + static_cast<size_t>(items) * 4 * sizeof(int);
 }
 
 const FusedNetwork::CompiledKernel& FusedNetwork::recordsKernelFor(SliceGradientKernel& sk, int flags, int numel, bool fromDerivatives)
@@ -1662,7 +1710,11 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
         const bool sliceGradients = useSliceGradients(numel, adjointFlags);
         compileBackwardKernel(adjointFlags, sliceGradients);
         for (auto& sk : backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value().sliceGradients)
+        {
             (void)recordsKernelFor(sk, adjointFlags, numel, storesDerivatives(numel, adjointFlags) && sk.derivativeOffset >= 0);
+            if (sk.columnsOffered && sortsTraining(numel))
+                compileColumnKernels(sk, adjointFlags, false, storesDerivatives(numel, adjointFlags) && sk.derivativeOffset >= 0);
+        }
         // the streams and events on which the weight-update kernels of the layers run side by side
         if ((adjointFlags & GRADIENTS_NETWORK_WEIGHTS) && compileOptions_.parallelWeightUpdate && layers_.size() > 1) ensureStreams();
     }
@@ -1677,6 +1729,11 @@ bool FusedNetwork::sortsTraining(int numel) const
 size_t FusedNetwork::sortedRowsOffset(int numel) const
 {
     return roundUp(forwardBytesPerPoint() * static_cast<size_t>(roundUp(numel, WARP_SIZE)), size_t(256));
+}
+
+size_t FusedNetwork::sortedTotalsOffset(int numel) const
+{
+    return sortedRowsOffset(numel) + roundUp(static_cast<size_t>(numel) * (channelsIn() + 1) * sizeof(float), size_t(256));
 }
 
 bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
@@ -1733,6 +1790,9 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     // the histograms are a multiple of 4 KiB: the sorted rows behind them stay 16-byte aligned
     float* sortedData = destination ? static_cast<float*>(destination) : reinterpret_cast<float*>(totals + histogramWords);
     int* orderData = reinterpret_cast<int*>(sortedData + static_cast<long long>(numel) * channels);
+    // a training pass keeps the points per slab with its sorted rows: the adjoint pass may walk the batch slab by slab
+    static_assert(SLABS == SORT_SLABS, "the slabs of kernels/point_order.h");
+    if (destination) totals = reinterpret_cast<int*>(static_cast<char*>(destination) + (sortedTotalsOffset(numel) - sortedRowsOffset(numel)));
 
     int count = numel;
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
@@ -1765,7 +1825,7 @@ size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlag
     if (adjointFlags > 0 && adjointFlags < ADJOINT_MODE_MAX_COMBINATIONS) announcedFlags_ = adjointFlags;
     // a batch that trains in sorted order: its sorted rows and the order, behind the intermediates and the derivatives
     if (sortsTraining(numElements))
-        return sortedRowsOffset(numElements) + roundUp(static_cast<size_t>(numElements) * (channelsIn() + 1) * sizeof(float), size_t(256));
+        return sortedTotalsOffset(numElements) + SORT_SLABS * sizeof(int);
     numElements = roundUp(numElements, WARP_SIZE);
     return forwardBytesPerPoint() * static_cast<size_t>(numElements);
 }
@@ -1995,6 +2055,46 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         auto inputAcc = sortedInput;
         for (auto& sk : ak.sliceGradients) {
             const auto& layout = sk.layout;
+            kernel::PointOrderKey sortKey{};
+            if (sortedPoints && sk.columnsOffered && pointOrderFor(numel, sortKey)) {
+                IEncoding::GradientColumnLayout sortedFor;
+                if (encodings_[sk.encoding]->gradientColumns(sortKey, sortedFor)
+                    && columnWorkspaceBytes(sk.columnLayout, numel) <= sliceGradientWorkspaceBytes(numel64)) {
+                    // the batch is sorted by the slabs of this grid: its gradients owner by owner, without records
+                    const bool fromDerivatives = derivativesStored && sk.derivativeOffset >= 0;
+                    compileColumnKernels(sk, adjointFlags, false, fromDerivatives);
+                    int maxItems = 0;
+                    (void)columnWorkspaceBytes(sk.columnLayout, numel, &maxItems);
+                    int* starts = reinterpret_cast<int*>(workspace);
+                    int* itemCount = starts + SORT_SLABS + 1;
+                    void* items = workspace + roundUp(static_cast<size_t>(SORT_SLABS + 1 + 1) * sizeof(int), size_t(256));
+                    const int* totals = reinterpret_cast<const int*>(static_cast<const char*>(tmpMemoryForward) + sortedTotalsOffset(numel));
+                    int slabs0 = sortKey.slabs0, slabs1 = sortKey.slabs1;
+                    std::vector<char> params(1024);
+                    int n = encodings_[sk.encoding]->fillParameterMemory(params.data(), static_cast<int>(params.size()));
+                    (void)n;
+                    {
+                        void* args[] = {&numel, &totals, &slabs0, &slabs1, &starts, &items, &itemCount, &maxItems};
+                        sk.columnsPlan.value().fun.launch(1, sk.columnsPlan.value().blockSize, 0, stream, args);
+                    }
+                    {
+                        const int* startsRead = starts;
+                        const void* itemsRead = items;
+                        const int* itemCountRead = itemCount;
+                        auto adjInputAcc = sortedAdjInput;
+                        const void* derivatives = static_cast<const char*>(tmpMemoryForward)
+                            + (static_cast<long long>(perEntryForwardMemoryBytes_) + std::max(0ll, sk.derivativeOffset)) * numel64;
+                        void* args[] = {&numel, &inputAcc, &adjEncoded, params.data(), &startsRead, &slabs0, &slabs1, &itemsRead, &itemCountRead,
+                                        &adjInputAcc, &derivatives};
+                        const auto& ck = sk.columns[fromDerivatives ? 1 : 0].value();
+                        ck.fun.launch(maxItems, ck.blockSize, ck.sharedMemorySize, stream, args);
+                    }
+                    // (the room of this encoding's cursors and records stays where it is for the encodings behind it)
+                    workspace += roundUp(static_cast<size_t>(layout.numBuckets() + 1) * sizeof(int), size_t(256))
+                        + roundUp(static_cast<size_t>(layout.totalRecords(numel64)) * layout.recordWords * sizeof(uint32_t), size_t(256));
+                    continue;
+                }
+            }
             int* cursors = reinterpret_cast<int*>(workspace);
             const size_t cursorBytes = roundUp(static_cast<size_t>(layout.numBuckets() + 1) * sizeof(int), size_t(256));
             uint32_t* records = reinterpret_cast<uint32_t*>(workspace + cursorBytes);

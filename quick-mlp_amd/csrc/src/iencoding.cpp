@@ -178,8 +178,8 @@ void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* we
     CHECK_DIM(input, 2);
     CHECK_DTYPE(input, Tensor::FLOAT);
     CHECK_ERROR(input.size(1) > maxInputChannel());
-    CHECK_ERROR(mode >= 0 && mode <= 3, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter, "
-                                        "3: the gradient records of the slice kernels");
+    CHECK_ERROR(mode >= 0 && mode <= 4, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter, "
+                                        "3: the gradient records of the slice kernels, 4: the sums of the column kernel");
     CHECK_ERROR(mode != 2 || (numFeaturesPerLevel_ & (numFeaturesPerLevel_ - 1)) == 0 && numFeaturesPerLevel_ <= 32,
                 "the tile-wide gradient scatter exists for 1, 2, 4 .. 32 features per level");
     CHECK_ERROR(mode == 0 || hasParameterTensor(Tensor::INFERENCE), "the traces read the table: bind one first");
@@ -195,7 +195,7 @@ void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* we
     const int grid = static_cast<int>(std::min<long long>(divUp<long long>(numel, block), fun.fullGridSize(block, 0)));
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
     int perPoint = numLevels() * (1 << ndim());
-    if (mode == 3) {
+    if (mode == 3 || mode == 4) {
         void* args[] = {&numel, &inputAcc, &indices, &weights, paramBytes.data()};
         fun.launch(grid, block, 0, stream, args);
         return;
@@ -206,8 +206,8 @@ void EncodingHashGrid::corners(const Tensor& input, unsigned* indices, float* we
 
 void EncodingHashGrid::precompileCorners(int mode, bool compileOnly)
 {
-    CHECK_ERROR(mode >= 0 && mode <= 3, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter, "
-                                        "3: the gradient records of the slice kernels");
+    CHECK_ERROR(mode >= 0 && mode <= 4, "mode 0: the index function, 1: the gathers of the forward pass, 2: the gradient scatter, "
+                                        "3: the gradient records of the slice kernels, 4: the sums of the column kernel");
     if (mode == 3) {
         // the record building of kernels/grid_gradient.h with the slice size the fused network uses for this grid
         GradientSliceLayout layout;
@@ -218,6 +218,21 @@ void EncodingHashGrid::precompileCorners(int mode, bool compileOnly)
         const int flags = QuickMLP::Instance().getCompileFlags() | (compileOnly ? KernelLoader::CompileOnly : 0);
         auto kernel = QuickMLP::Instance().kernelLoader()->getKernel(
             "qmlp::kernel::GridGradientTraceKernel<" + layout.configType + ", " + std::to_string(layout.sliceFloats) + ">",
+            source.str(), flags);
+        if (!compileOnly) cornersKernel_[mode] = kernel.value();
+        return;
+    }
+    if (mode == 4) {
+        // the index arithmetic of kernels/grid_gradient_columns.h for the slabs by which the fused network sorts for this grid
+        kernel::PointOrderKey key{};
+        GradientColumnLayout layout;
+        CHECK_ERROR(pointOrderKey(key, 0) && gradientColumns(key, layout), "this grid has no gradient columns");
+        std::stringstream source;
+        fillCode(source);
+        source << "\n" << KernelLoader::MainFile("qmlp/kernels/grid_gradient_columns.h");
+        const int flags = QuickMLP::Instance().getCompileFlags() | (compileOnly ? KernelLoader::CompileOnly : 0);
+        auto kernel = QuickMLP::Instance().kernelLoader()->getKernel(
+            "qmlp::kernel::GridGradientColumnsTraceKernel<" + layout.configType + ", " + std::to_string(layout.cellsPerSlab) + ">",
             source.str(), flags);
         if (!compileOnly) cornersKernel_[mode] = kernel.value();
         return;

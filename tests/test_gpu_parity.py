@@ -306,8 +306,17 @@ def _per_point_sets(idx, w):
     return idx, np.where(last, acc, 0.0)
 
 
+# single dense levels of 4 MB and more: their batches can be sorted by slab, and their gradients summed by columns
+COLUMN_GRIDS = [
+    ({"n_in": 3, "n_levels": 1, "n_features_per_level": 2, "log2_hashmap_size": -1, "min_resolution": 128, "max_resolution": 128}, "half"),
+    ({"n_in": 2, "n_levels": 1, "n_features_per_level": 4, "log2_hashmap_size": -1, "min_resolution": 1000, "max_resolution": 1000}, "float"),
+    ({"n_in": 4, "n_levels": 1, "n_features_per_level": 8, "log2_hashmap_size": -1, "min_resolution": 32, "max_resolution": 32}, "half"),
+]
+COLUMN_GRID_CFGS = [_grid_cfg(s, p) for s, p in COLUMN_GRIDS] + [bc.densegrid4d("half")]
+
+
 @pytest.mark.parametrize("spec", GRID_SPECS + [bc.hashgrid3d("float"), bc.hashgrid3d("half"), bc.densegrid4d("half")]
-                         + [dict(s, parameter_precision=p) for s, p in SLICE_GRIDS[1:4] + SLICE_GRIDS[6:]])
+                         + [dict(s, parameter_precision=p) for s, p in SLICE_GRIDS[1:4] + SLICE_GRIDS[6:] + COLUMN_GRIDS[:2]])
 def test_grid_indices_are_bit_exact(spec):
     """The table entries the device code touches, against the oracle's restatement of the
     reference's index arithmetic (encoding_hashgrid.cuh:17-60,279-287): the index function on its
@@ -318,7 +327,9 @@ def test_grid_indices_are_bit_exact(spec):
     Mode 3, for grids of up to four dimensions: what the gradient records of large batches stand
     for (kernels/grid_gradient.h: the slice of the record's bucket plus the two 16-bit offsets
     as the slice kernel decodes them, and the entries of other slices that the records kernel adds
-    itself)."""
+    itself). Mode 4, for single dense levels whose batches are sorted by slab: the elements behind the sums
+    of the column kernel (kernels/grid_gradient_columns.h: the place in the LDS of the owner of the corner's
+    node, and back to the table as the kernel writes its sums)."""
     import json
     import qmlp
     cfg = _grid_cfg(spec, spec.get("parameter_precision", "float")) if "id" not in spec else spec
@@ -331,6 +342,12 @@ def test_grid_indices_are_bit_exact(spec):
     except qmlp.QmlpError as e:
         # more than four dimensions, or a level of more than 512 slices
         assert "no gradient slices" in str(e) and (cfg["n_in"] > 4 or cfg["max_resolution"] == 2048)
+    try:
+        enc.hashgrid_corners(None, 4)       # compiles the kernel of mode 4, or says that the grid has no columns
+        modes.append(4)
+    except qmlp.QmlpError as e:
+        # several levels, hashed levels, or a dense level below the 4 MB from which batches are sorted by slab
+        assert "no gradient columns" in str(e) and (cfg["n_levels"] > 1 or cfg not in [dict(c) for c in COLUMN_GRID_CFGS])
     if os.environ.get("QMLP_WARM_CACHE"):
         for m in modes:
             enc.hashgrid_corners(None, m)
@@ -1267,3 +1284,95 @@ def test_position_derivatives_are_kept_when_input_gradients_are_announced():
     ref = auto.oracle.backward(X, adj, FLAG_INPUT, round_mode=0)
     s = max(1.0, float(np.abs(ref["adj_x"]).max()))
     assert_close(adjoint(auto, tmp7) / s, ref["adj_x"] / s, "input gradients from stored derivatives vs fp32 oracle")
+
+
+@pytest.mark.parametrize("spec,precision", COLUMN_GRIDS)
+def test_grid_gradients_summed_by_columns_match_the_records_the_atomic_scatter_and_the_oracle(spec, precision):
+    """A single dense level whose batch trains sorted by grid slab (options.sort_points = 1 here, so that small
+    batches sort too): the gradients of the table are summed owner by owner of the grid's nodes in LDS, without
+    records (kernels/grid_gradient_columns.h; options.column_gradients = 0: records and slices on the same sorted
+    batch; options.slice_gradients = 0, sort_points = 0: float atomics on the batch as given). Same entries, same
+    weights, another order of the additions; all against the fp32 oracle. Batches: fewer points than slabs; a
+    ragged last tile with points outside the box; all points in one small region (one owner, split into parts);
+    far outside points and a NaN coordinate (added with atomics by the workgroup of their slab)."""
+    d = spec["n_in"]
+    grid = _grid_cfg(spec, precision, start=1)
+    n_in = d + 1
+    base = {"num_inputs": n_in, "num_outputs": 2, "activation_specification": ["qmlp/builtin-activations.json"],
+            "encodings": [{"id": "Identity", "start_in": 0, "n_in": 2}, grid],
+            "network": [{"n_out": 32, "bias": True, "activation": "celu"},
+                        {"n_out": 2, "bias": False, "activation": "identity"}]}
+    options = {"columns": {"sort_points": 1, "slice_gradients": 1},
+               "records": {"sort_points": 1, "slice_gradients": 1, "column_gradients": 0},
+               "atomics": {"sort_points": 0, "slice_gradients": 0}}
+    warm_cache(*[dict(base, options=o) for o in options.values()])
+    cases = {k: Case(dict(base, options=o)) for k, o in options.items()}
+    rng = np.random.default_rng(23)
+    params = random_parameters(cases["columns"].oracle, rng)
+    table = rng.uniform(-1, 1, cases["columns"].oracle.encodings[1][1].n_params)
+    for c in cases.values():
+        c.set_parameters(params)
+        c.set_table(1, table)
+    lo = np.array([0.0] + grid["bounding_box_min"], np.float32)
+    sz = np.array([1.0] + grid["bounding_box_size"], np.float32)
+    flags = FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC
+    for N, clustered in [(500, False), (70001, False), (70001, True)]:
+        # (up to one and a half cells outside the box: weights up to 2.5^D; further out the cancelling terms of the
+        # extrapolation leave rounding noise in either mode, see below)
+        margin = 1.5 / spec["max_resolution"]
+        u = rng.uniform(-margin, 1 + margin, (N, n_in)) if not clustered else 0.37 + 2e-3 * rng.uniform(0, 1, (N, n_in))
+        X = (lo + sz * u).astype(np.float32)
+        if not clustered:
+            X[:16, 1:] = lo[1:] + sz[1:] * rng.integers(0, 2, (16, d))        # exact box corners and borders
+        adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+        for f in (FLAG_ENC, flags):
+            got = {k: c.gpu_train(X, adj, f) for k, c in cases.items()}
+            a, b, c = (got[k]["table_grads"][1] for k in ("columns", "records", "atomics"))
+            scale = max(1.0, float(np.abs(c).max()))
+            what = "N=%d clustered=%s flags=%d" % (N, clustered, f)
+            assert np.allclose(a / scale, c / scale, rtol=1e-4, atol=2e-6), what + ": %g" % np.abs(a - c).max()
+            assert np.allclose(a / scale, b / scale, rtol=1e-4, atol=2e-6), what + ": %g" % np.abs(a - b).max()
+            assert np.array_equal(got["columns"]["out"], got["atomics"]["out"])
+            if f & FLAG_INPUT:
+                # the same arithmetic for the input gradients in both sorted modes
+                assert np.array_equal(got["columns"]["adj_x"], got["records"]["adj_x"]), what
+                # (the order of the points inside a slab differs from sort to sort: another order of the fp32 sums)
+                sg = float(np.abs(got["records"]["grads"]).max())
+                assert np.allclose(got["columns"]["grads"] / sg, got["records"]["grads"] / sg, rtol=1e-4, atol=1e-6), what
+                sx = max(1e-30, float(np.abs(got["atomics"]["adj_x"]).max()))
+                assert np.allclose(got["columns"]["adj_x"] / sx, got["atomics"]["adj_x"] / sx, rtol=2e-3, atol=1e-3), what
+            check_gradients(cases["columns"], X, adj, FLAG_ENC, got["columns"], what="columns, " + what + ": ")
+            if N == 500 and f & FLAG_INPUT:
+                ref = cases["columns"].oracle.backward(X, adj, FLAG_INPUT, round_mode=0)
+                sx = max(1.0, float(np.abs(ref["adj_x"]).max()))
+                assert_close(got["columns"]["adj_x"] / sx, ref["adj_x"] / sx, "input gradients vs fp32 oracle")
+    # far outside points (weights far above one) and a NaN coordinate: as in the slice kernels' test
+    N = 70001
+    X = (lo + sz * rng.uniform(0, 1, (N, n_in))).astype(np.float32)
+    far = np.arange(7, N, 1000)
+    X[far] = (lo + sz * rng.uniform(-3.0, 4.0, (len(far), n_in))).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 2)) * 0.05).astype(np.float32)
+    probe = qmlp.Encoding(json.dumps(grid))
+    probe.set_parameter(torch.zeros(probe.num_parameters(), device="cuda", dtype=probe.parameter_dtype()))
+    far_idx, far_w = probe.hashgrid_corners(torch.from_numpy(X[far]).cuda())
+    touched = np.zeros(probe.num_parameters(), bool)
+    for f in range(spec["n_features_per_level"]):
+        touched[far_idx.cpu().numpy().astype(np.int64).ravel() + f] = True
+    largest = float(far_w.abs().max())
+    assert largest > 100
+    got = {k: cases[k].gpu_train(X, adj, FLAG_ENC) for k in ("columns", "atomics")}
+    a, b = got["atomics"]["table_grads"][1], got["columns"]["table_grads"][1]
+    assert np.isfinite(a).all() and np.isfinite(b).all()
+    scale = float(np.abs(a[~touched]).max())
+    bad = np.where(~np.isclose(a / scale, b / scale, rtol=1e-4, atol=2e-5) & ~touched)[0]
+    assert scale > 0 and len(bad) == 0, (len(bad), bad[:8], a[bad[:8]], b[bad[:8]])
+    noise = 1.0 + len(far) * largest * 2.0 ** -20
+    assert np.abs(a[touched]).max() < noise and np.abs(b[touched]).max() < noise
+    X = (lo + sz * rng.uniform(0, 1, (N, n_in))).astype(np.float32)
+    X[5, 1] = np.nan
+    got = {k: cases[k].gpu_train(X, adj, FLAG_ENC) for k in ("columns", "atomics")}
+    a, b = got["atomics"]["table_grads"][1], got["columns"]["table_grads"][1]
+    assert np.isnan(a).any() and np.array_equal(np.isnan(a), np.isnan(b))
+    ok = ~np.isnan(a)
+    scale = float(np.abs(a[ok]).max())
+    assert np.allclose(a[ok] / scale, b[ok] / scale, rtol=1e-4, atol=2e-5)
