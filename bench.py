@@ -173,6 +173,9 @@ def ordered_batch_report(cfg_id, n, device, steps, warmup):
     return out
 
 
+LOSS_SCALE = 65536.0
+
+
 def run_train(case, steps, warmup, input_gradients=True, warmup_seconds=0.0):
     import torch
     import baseline_configs as bc
@@ -194,7 +197,10 @@ def run_train(case, steps, warmup, input_gradients=True, warmup_seconds=0.0):
             if g is not None:
                 g.zero_()
         out, tmp = net.forward_raw(x, params, enc, flags)
-        adj_out = (out - target) * (2.0 / out.numel())
+        # (mean squared error with the loss scaled by 2^16, as fp16 training does: 2 / numel alone is 5e-7 for 2^21
+        # points with two outputs, and the adjoints of the layers, which are halves, underflow to zero -- a step whose
+        # gradients vanish is not the work of a train step: kernels that skip zeros would look faster than they are)
+        adj_out = (out - target) * (2.0 * LOSS_SCALE / out.numel())
         net.adjoint_raw(x, adj_out, flags, tmp, params, enc, grad_network=grad_net, grad_encodings=grad_enc,
                         adj_input=adj_in if input_gradients else None)
 

@@ -534,6 +534,15 @@ struct GridGradientRecords
         float adjFeat[F];
 #pragma unroll
         for (int i = 0; i < F; ++i) adjFeat[i] = static_cast<float>(adjRow[i * TILE_POINTS]);
+        positionGradient<LEVEL>(s, held, adjFeat, adjPos);
+    }
+
+    /** The same from the adjoint of the level's features as floats. */
+    template <int LEVEL>
+    __device__ __forceinline__ static void positionGradient(const typename Grid::LevelSetup& s,
+                                                            const detail::HeldFeatures<F, typename Cfg::table_t> (&held)[Grid::NC],
+                                                            const float (&adjFeat)[F], float (&adjPos)[D])
+    {
         float lvl[D];
 #pragma unroll
         for (int d = 0; d < D; ++d) lvl[d] = 0.f;

@@ -79,6 +79,38 @@ struct GridGradientColumns
             + static_cast<unsigned>(within);
     }
 
+    /** Entries of the table around one slab: the nodes (a * CPS .. (a + 1) * CPS) in both sorted coordinates, all others. */
+    static constexpr int REGION_NODES = CPS + 1;
+    static constexpr int REGION_ENTRIES = REGION_NODES * REGION_NODES * REST;
+    static constexpr int REGION_BYTES = REGION_ENTRIES * F * static_cast<int>(sizeof(typename Cfg::table_t));
+    static constexpr int LDS_BYTES = ((LOCAL_FLOATS * 8 > REGION_BYTES ? LOCAL_FLOATS * 8 : REGION_BYTES) + 15) / 16 * 16;
+
+    /** Place of node (n0, n1, rest) in the staged region of slab (a0, a1), in entries; valid: the node lies inside it. */
+    __device__ __forceinline__ static int regionEntry(int n0, int n1, unsigned rest, int a0, int a1, bool& valid)
+    {
+        const int l0 = n0 - a0 * CPS, l1 = n1 - a1 * CPS;
+        valid = l0 >= 0 && l0 < REGION_NODES && l1 >= 0 && l1 < REGION_NODES;
+        return (l0 * REGION_NODES + l1) * REST + static_cast<int>(rest);
+    }
+
+    /** The position of point p in the unit box, as every kernel of the grid computes it. */
+    __device__ __forceinline__ static void loadPosition(const Tensor2Read<float>& inputs, int p, const param_t& params,
+                                                        bool rowsOfFloat4, float (&pos)[D])
+    {
+#pragma clang fp contract(off)
+        float in[D];
+        if (D == 4 && rowsOfFloat4) {
+            const float4 v = *reinterpret_cast<const float4*>(inputs.data_ + static_cast<long long>(p) * inputs.strides_[0] + Cfg::Start);
+            in[0] = v.x, in[1 % D] = v.y, in[2 % D] = v.z, in[3 % D] = v.w;
+        } else {
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                in[d] = inputs.data_[static_cast<long long>(p) * inputs.strides_[0] + static_cast<long long>(d + Cfg::Start) * inputs.strides_[1]];
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) pos[d] = (in[d] - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
+    }
+
     /** Node indices of corner c (bit d: upper in dimension d) in the two sorted coordinates, and the rest of its index. */
     __device__ __forceinline__ static void cornerNode(const typename Grid::LevelSetup& s, int c, int& n0, int& n1, unsigned& rest)
     {
@@ -188,7 +220,7 @@ __global__ void __launch_bounds__(1024) GridGradientColumnsPlan(
  * \tparam INPUT_GRADIENTS 0: none; 1: from a gather of all corners; 2: from the position derivatives of the forward pass
  * inputs: the rows of the batch in sorted order; starts, items, itemCount: as GridGradientColumnsPlan wrote them.
  * Launched with as many workgroups as there can be work items; those beyond itemCount leave at once.
- * Dynamic LDS: LOCAL_FLOATS * 8 bytes.
+ * Dynamic LDS: GridGradientColumns::LDS_BYTES (the sums of an owner, then the entries of the table around its slab).
  */
 template <typename Cfg, int CPS, int ROW_CHANNELS, int CHANNEL_OFFSET, int INPUT_GRADIENTS, int BLOCK>
 __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
@@ -232,6 +264,7 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
         unsigned maxBits = 0u;
 #pragma unroll
         for (int r = 0; r < 2; ++r)
+#pragma unroll 4
             for (int p = begin[r] + tid; p < end[r]; p += BLOCK) {
                 const f16* adjRow = adjEncoded + static_cast<long long>(p / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
                     + CHANNEL_OFFSET * TILE_POINTS + (p % TILE_POINTS);
@@ -249,31 +282,48 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
     const int maxExponent = static_cast<int>(maxBits >> 10) - 14;   // |adjoint| < 2^maxExponent
     const long long terms = static_cast<long long>(NC) * max(1, (end[0] - begin[0]) + (end[1] - begin[1]));
     const int termsLog2 = 64 - __builtin_clzll(static_cast<unsigned long long>(terms));
-    const int scaleExponent = 61 - maxExponent - termsLog2;
+    // A term is the product of two integers: the adjoint in units of 2^-adjointShift (below 2^adjointBits in
+    // magnitude) and the weight of the corner in units of 2^-WEIGHT_BITS (at most one): one multiply-add instruction
+    // per term instead of the nine of a float product split into two words. The sum of all terms that can meet in
+    // one element stays below 2^62.
+    constexpr int WEIGHT_BITS = 22;
+    const int adjointBits = min(30, 62 - WEIGHT_BITS - termsLog2);
+    const int adjointShift = adjointBits - maxExponent;
+    const int scaleExponent = adjointShift + WEIGHT_BITS;
     float* __restrict__ gradients = params.parametersBackward;
+    // rows of four floats that lie side by side: one load
+    const bool rowsOfFloat4 = D == 4 && Cfg::Start % 4 == 0 && inputs.strides_[1] == 1 && inputs.strides_[0] % 4 == 0
+        && reinterpret_cast<unsigned long long>(inputs.data_) % 16 == 0;
 
 #pragma unroll 1
     for (int r = 0; r < 2; ++r) {
         const int a0 = item.owner0 - 1 + r;
+        // (the position and the adjoints of a lane's next point are loaded before it works on this one: with four
+        // wavefronts per SIMD nothing else hides the latency of the loads)
+        float nextPos[D];
+        f16 nextAdj[F];
+        auto loadPoint = [&](int q) {
+            Impl::loadPosition(inputs, q, params, rowsOfFloat4, nextPos);
+            const f16* row = adjEncoded + static_cast<long long>(q / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
+                + CHANNEL_OFFSET * TILE_POINTS + (q % TILE_POINTS);
+#pragma unroll
+            for (int i = 0; i < F; ++i) nextAdj[i] = row[i * TILE_POINTS];
+        };
+        if (begin[r] + tid < end[r]) loadPoint(begin[r] + tid);
 #pragma unroll 1
         for (int p = begin[r] + tid; p < end[r]; p += BLOCK) {
             const int a1 = p < runs.middle[r] ? item.owner1 - 1 : item.owner1;
             const bool home = a0 == item.owner0 && a1 == item.owner1;
             float pos[D];
-            {
-#pragma clang fp contract(off)
+            f16 adjHalf[F];
 #pragma unroll
-                for (int d = 0; d < D; ++d) {
-                    const float in = inputs.data_[static_cast<long long>(p) * inputs.strides_[0]
-                                                  + static_cast<long long>(d + Cfg::Start) * inputs.strides_[1]];
-                    pos[d] = (in - params.boundingBoxMin[d]) * params.boundingBoxInvSize[d];
-                }
-            }
+            for (int d = 0; d < D; ++d) pos[d] = nextPos[d];
+#pragma unroll
+            for (int i = 0; i < F; ++i) adjHalf[i] = nextAdj[i];
+            if (p + BLOCK < end[r]) loadPoint(p + BLOCK);
             const typename Grid::LevelSetup s = Grid::setupLevel(0, pos);
             int c0, c1;
             Impl::cell(s, c0, c1);
-            const f16* adjRow = adjEncoded + static_cast<long long>(p / TILE_POINTS) * (ROW_CHANNELS * TILE_POINTS)
-                + CHANNEL_OFFSET * TILE_POINTS + (p % TILE_POINTS);
             // Points that do not fit the scheme -- the same verdict in every workgroup that visits the point: outside
             // the box, in a cell of another slab than the sort's, or with an adjoint that is not finite (NaN and
             // infinity have no fixed-point form and reach the gradients through the atomics of the point's home).
@@ -281,7 +331,7 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
             bool finite = true;
 #pragma unroll
             for (int i = 0; i < F; ++i) {
-                const f16 h = adjRow[i * TILE_POINTS];
+                const f16 h = adjHalf[i];
                 finite = finite && (static_cast<unsigned>(__builtin_bit_cast(unsigned short, h)) & 0x7c00u) != 0x7c00u;
                 adj[i] = static_cast<float>(h);
             }
@@ -291,13 +341,14 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
                 if (maxBits != 0u) {
                     // neighbouring lanes take the features in rotated order (an entry starts at a multiple of
                     // 8 F bytes: lanes that all add the same feature would meet on a few LDS banks)
-                    float rotated[F];
+                    int rotated[F];
 #pragma unroll
                     for (int step = 0; step < F; ++step) {
                         const int i = (F & (F - 1)) == 0 ? ((step + tid) & (F - 1)) : ((step + tid % F) % F);
-                        rotated[step] = adj[0];
+                        float a = adj[0];
 #pragma unroll
-                        for (int k = 1; k < F; ++k) rotated[step] = i == k ? adj[k] : rotated[step];
+                        for (int k = 1; k < F; ++k) a = i == k ? adj[k] : a;
+                        rotated[step] = static_cast<int>(rintf(ldexpf(a, adjointShift)));
                     }
 #pragma unroll
                     for (int c = 0; c < NC; ++c) {
@@ -305,12 +356,12 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
                         unsigned rest;
                         Impl::cornerNode(s, c, n0, n1, rest);
                         if (n0 / CPS != item.owner0 || n1 / CPS != item.owner1) continue;
-                        const float w = Grid::cornerWeight(s, c);
+                        const int w = static_cast<int>(rintf(ldexpf(Grid::cornerWeight(s, c), WEIGHT_BITS)));
                         long long* sums = sSums + Impl::localElement(n0, n1, rest, item.owner0, item.owner1);
 #pragma unroll
                         for (int step = 0; step < F; ++step) {
                             const int i = (F & (F - 1)) == 0 ? ((step + tid) & (F - 1)) : ((step + tid % F) % F);
-                            Fixed::ldsAddFixed(sums + i, Fixed::toFixed(w * rotated[step], scaleExponent));
+                            Fixed::ldsAddFixed(sums + i, static_cast<long long>(w) * static_cast<long long>(rotated[step]));
                         }
                     }
                 }
@@ -321,27 +372,7 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
                     const float w = Grid::cornerWeight(s, c);
                     const unsigned element = Grid::cornerOffset(0, s, c);
 #pragma unroll 1
-                    for (int i = 0; i < F; ++i) unsafeAtomicAdd(gradients + element + i, w * static_cast<float>(adjRow[i * TILE_POINTS]));
-                }
-            }
-            if constexpr (INPUT_GRADIENTS != 0) {
-                if (home) {
-                    float adjPos[D];
-#pragma unroll
-                    for (int d = 0; d < D; ++d) adjPos[d] = 0.f;
-                    if constexpr (INPUT_GRADIENTS == 2) {
-                        Records::template positionGradientFromDerivatives<0>(
-                            p, static_cast<const typename Records::DerivativeChunk*>(derivativesV), adjEncoded, adjPos);
-                    } else {
-                        detail::HeldFeatures<F, typename Cfg::table_t> held[NC];
-                        Records::template loadHeld<0>(s, params, held);
-                        Records::template positionGradient<0>(p, s, held, adjEncoded, adjPos);
-                    }
-                    // every point has one home: a plain read-modify-write
-#pragma unroll
-                    for (int d = 0; d < D; ++d)
-                        adjInputs.data_[static_cast<long long>(p) * adjInputs.strides_[0]
-                                        + static_cast<long long>(d + Cfg::Start) * adjInputs.strides_[1]] += adjPos[d] * params.boundingBoxInvSize[d];
+                    for (int i = 0; i < F; ++i) unsafeAtomicAdd(gradients + element + i, w * adj[i]);
                 }
             }
         }
@@ -351,15 +382,89 @@ __global__ void __launch_bounds__(BLOCK) GridGradientColumnsKernel(
     // The sums of this owner, added with atomics (16 neighbouring floats per request): other workgroups may be adding
     // the corners of points that do not fit the scheme to the same elements at this moment, and the parts of a
     // split owner hold sums for the same elements.
-    if (maxBits == 0u) return;
-    for (int i = tid; i < Impl::LOCAL_FLOATS; i += BLOCK) {
-        const long long fixed = sSums[i];
-        if (fixed == 0) continue;
-        bool valid;
-        const unsigned element = Impl::globalElement(i, item.owner0, item.owner1, valid);
-        if (!valid) continue;
-        const float v = static_cast<float>(ldexp(static_cast<double>(fixed), -scaleExponent));
-        unsafeAtomicAdd(gradients + element, v);
+    if (maxBits != 0u) {
+        for (int i = tid; i < Impl::LOCAL_FLOATS; i += BLOCK) {
+            const long long fixed = sSums[i];
+            if (fixed == 0) continue;
+            bool valid;
+            const unsigned element = Impl::globalElement(i, item.owner0, item.owner1, valid);
+            if (!valid) continue;
+            const float v = static_cast<float>(ldexp(static_cast<double>(fixed), -scaleExponent));
+            unsafeAtomicAdd(gradients + element, v);
+        }
+    }
+
+    if constexpr (INPUT_GRADIENTS != 0) {
+        // The grid's share of the gradient with respect to the input, for the points whose slab has the indices of
+        // this owner (every point has one such home: a plain read-modify-write of its row). From the position
+        // derivatives of the forward pass where it kept them; else from the entries of all corners, as the records
+        // kernel gathers them -- but out of the LDS, which the sums have left: the entries around one slab are as
+        // many bytes as an owner's sums (half tables) and are copied in with coalesced loads once, instead of
+        // 2^D gathers of one entry per point (dense 4-D grid with 8 features, 2^21 points: 96 of 180 us).
+        const int a0 = item.owner0, a1 = item.owner1;
+        if (a0 >= slabs0 || a1 >= slabs1) return;   // an owner of border nodes only: no slab of its own
+        const int homeBegin = max(begin[1], min(runs.middle[1], end[1])), homeEnd = end[1];
+        if (homeBegin >= homeEnd) return;           // (the same for the whole workgroup)
+        typedef typename Cfg::table_t table_t;
+        table_t* sRegion = reinterpret_cast<table_t*>(sMemory);
+        if constexpr (INPUT_GRADIENTS == 1) {
+            __syncthreads();   // the sums have been read
+            // 16 bytes per load: the entries of one (n0, n1) are REST * F values side by side in the table and in the region
+            constexpr int COLUMN_VALUES = Impl::REST * F;
+            constexpr int WIDEST = 16 / static_cast<int>(sizeof(table_t));
+            constexpr int PER_LOAD = COLUMN_VALUES % WIDEST == 0 ? WIDEST : COLUMN_VALUES % (WIDEST / 2) == 0 ? WIDEST / 2
+                : COLUMN_VALUES % (WIDEST / 4) == 0 ? WIDEST / 4 : 1;
+            typedef table_t load_t __attribute__((ext_vector_type(PER_LOAD)));
+            for (int i = tid; i < Impl::REGION_NODES * Impl::REGION_NODES * (COLUMN_VALUES / PER_LOAD); i += BLOCK) {
+                const int column = i / (COLUMN_VALUES / PER_LOAD), within = i % (COLUMN_VALUES / PER_LOAD);
+                const int n0 = a0 * CPS + column / Impl::REGION_NODES, n1 = a1 * CPS + column % Impl::REGION_NODES;
+                if (n0 < Impl::R && n1 < Impl::R) {
+                    const table_t* src = params.parametersForward + Cfg::memoryOffset[0]
+                        + (static_cast<long long>(n0) * Impl::R + n1) * COLUMN_VALUES + within * PER_LOAD;
+                    *reinterpret_cast<load_t*>(sRegion + column * COLUMN_VALUES + within * PER_LOAD) = *reinterpret_cast<const load_t*>(src);
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll 1
+        for (int p = homeBegin + tid; p < homeEnd; p += BLOCK) {
+            float pos[D];
+            Impl::loadPosition(inputs, p, params, rowsOfFloat4, pos);
+            float adjPos[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d) adjPos[d] = 0.f;
+            if constexpr (INPUT_GRADIENTS == 2) {
+                Records::template positionGradientFromDerivatives<0>(
+                    p, static_cast<const typename Records::DerivativeChunk*>(derivativesV), adjEncoded, adjPos);
+            } else {
+                const typename Grid::LevelSetup s = Grid::setupLevel(0, pos);
+                detail::HeldFeatures<F, table_t> held[NC];
+                // (a point in a cell of another slab than the sort's -- within rounding of a slab boundary, on the upper
+                // border -- may have corners outside the region: it gathers from the table)
+                bool staged = true;
+                int entry[NC];
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    int n0, n1;
+                    unsigned rest;
+                    Impl::cornerNode(s, c, n0, n1, rest);
+                    bool valid;
+                    entry[c] = Impl::regionEntry(n0, n1, rest, a0, a1, valid);
+                    staged = staged && valid;
+                }
+                if (staged) {
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) held[c].load(sRegion + entry[c] * F);
+                } else {
+                    Records::template loadHeld<0>(s, params, held);
+                }
+                Records::template positionGradient<0>(p, s, held, adjEncoded, adjPos);
+            }
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                adjInputs.data_[static_cast<long long>(p) * adjInputs.strides_[0]
+                                + static_cast<long long>(d + Cfg::Start) * adjInputs.strides_[1]] += adjPos[d] * params.boundingBoxInvSize[d];
+        }
     }
 }
 

@@ -384,13 +384,19 @@ bool EncodingHashGrid::gradientColumns(const kernel::PointOrderKey& key, Gradien
     const int cellsPerSlab = divUp(cells, own.slabs0);
     if (divUp(cells, cellsPerSlab) != own.slabs0) return false;
     long long sums = static_cast<long long>(cellsPerSlab) * cellsPerSlab * numFeaturesPerLevel_;
-    for (int d = 2; d < dimension_; ++d) sums *= nodes;
-    // two workgroups of an owner's 64-bit sums per compute unit
-    if (sums * 8 > (FusedNetwork::MaxSharedMemoryBytes() - 1024) / 2) return false;
+    long long region = static_cast<long long>(cellsPerSlab + 1) * (cellsPerSlab + 1) * numFeaturesPerLevel_;
+    for (int d = 2; d < dimension_; ++d) {
+        sums *= nodes;
+        region *= nodes;
+    }
+    // as GridGradientColumns::LDS_BYTES: the 64-bit sums of an owner, later the entries of the table around its slab;
+    // two workgroups per compute unit
+    const long long ldsBytes = roundUp<long long>(std::max(sums * 8, region * (parameterPrecision_ == Tensor::HALF ? 2 : 4)), 16);
+    if (ldsBytes > (FusedNetwork::MaxSharedMemoryBytes() - 1024) / 2) return false;
     layout.configType = "qmlp::kernel::" + configName();
     layout.cellsPerSlab = cellsPerSlab;
     layout.owners = divUp(nodes, cellsPerSlab);
-    layout.ldsBytes = static_cast<int>(sums * 8);
+    layout.ldsBytes = static_cast<int>(ldsBytes);
     return true;
 }
 
