@@ -176,7 +176,9 @@ int qmlp_encoding_hashgrid_corners(qmlp_encoding_t encoding, const qmlp_tensor* 
  * adds to (encoding_hashgrid.cuh:345-369; nothing is added); mode 3: the entries and weights that
  * the gradient records of large batches stand for (slice of the record's bucket + 16-bit offsets,
  * and the entries of other slices that the records kernel adds itself; grids that offer gradient
- * slices only); mode 0 = qmlp_encoding_hashgrid_corners.
+ * slices only); mode 4: the entries behind the sums of the column kernel of sorted batches (the place of
+ * each corner in the LDS of the owner of its node, and back to the table as the kernel writes its sums;
+ * single dense levels that offer gradient columns only); mode 0 = qmlp_encoding_hashgrid_corners.
  * The order of the 2^dim corners of a level is the order the code visits them. input = NULL only
  * compiles the kernel of that mode into the kernel cache (needs no GPU). */
 int qmlp_encoding_hashgrid_trace(qmlp_encoding_t encoding, const qmlp_tensor* input, int mode, uint32_t* indices,

@@ -225,7 +225,8 @@ class Encoding:
         """Device-computed table offsets and weights, shape (N, levels, 2^dim). mode 0: the index
         function; 1: what the gathers of the fused forward kernels use (bind a table first);
         2: what the gradient scatter of the fused backward kernel adds to; 3: what the gradient
-        records of large batches (sums per slice of the table) stand for."""
+        records of large batches (sums per slice of the table) stand for; 4: the elements behind the
+        sums of the column kernel (single dense levels whose batches train sorted by slab)."""
         if input is None:      # compile the kernel of this mode into the kernel cache, nothing runs
             check(lib.qmlp_encoding_hashgrid_trace(self._handle, None, int(mode), None, None, None))
             return None
