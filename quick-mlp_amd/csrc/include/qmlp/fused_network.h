@@ -92,6 +92,14 @@ public:
         // <0 (default) and >0: wherever the encoding offers it; 0: never (records and slices as for other grids).
         int columnGradients = -1;
 
+        // Networks whose backward kernel sums the weight gradients of all layers: a training pass keeps the encoded
+        // input only (2 C_in0 bytes per point instead of 2 (C_in0 + sum C_out)) and the backward kernel runs the layers
+        // forward again per tile, the pre-activations staying in registers. <0 (default): when the adjoint flags
+        // announced last (forwardMemory(), prepare(), adjoint()) lead to such a backward kernel; 0: never; >0: as <0.
+        // An adjoint pass with other flags than announced, whose kernels need the stored intermediates, first runs
+        // the forward pass again into the same forward memory.
+        int recomputeIntermediates = -1;
+
         // Gradients of the layer weights: summed inside the backward kernel, which holds the adjoint
         // pre-activations in registers (Layer::weightGradient), instead of by one kernel per layer that reads
         // them back from memory. <0 (default): the layers with the fewest gradient tiles, up to 16 tiles (64
@@ -148,9 +156,10 @@ private:
     };
     // [store intermediates][variant], see ForwardVariant
     // [0]: inference, [1]: forward (stores the intermediates), [2]: forward that also stores position derivatives
-    std::optional<CompiledKernel> forwardKernels_[3][4];
+    // ([3], [4]: as [1], [2], but of the intermediates only the encoded input is stored)
+    std::optional<CompiledKernel> forwardKernels_[5][4];
     // set once the compiled REGISTERS shape turned out to spill heavily: it is not used then
-    bool registerShapeSpills_[3] = {false, false, false};
+    bool registerShapeSpills_[5] = {false, false, false, false, false};
 
     // counting sort of the batch by grid slab in front of the inference kernel
     struct PointOrder
@@ -238,8 +247,8 @@ private:
         std::vector<bool> fusedLayers;    // layers whose weight gradients the adjoint kernel sums (no kernel in 'layers')
         bool fusedWeightUpdate = false;   // any of them
     };
-    // [adjoint flags][grid gradients by slices instead of atomics]
-    std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2];
+    // [adjoint flags][grid gradients by slices instead of atomics][the layers run again instead of reading their intermediates]
+    std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2][2];
     // Below this the two slice kernels cost more than the atomics they save (their work items zero and write
     // back whole slices whatever the batch): a train step of a 16-level hash grid at 2^14 / 2^15 / 2^16 / 2^17
     // points 0.18 / 0.24 / 0.37 / 0.63 ms with atomics, 0.18 / 0.19 / 0.22 / 0.30 ms by slices; of one dense
@@ -267,8 +276,25 @@ private:
     int derivativeBytesPerPoint_ = 0;
     /** The adjoint flags that the caller announced last: forwardMemory(n, flags), adjoint(..., flags, ...). */
     int announcedFlags_ = 0;
-    /** Forward memories whose last training pass stored position derivatives, with the size of that batch. */
-    std::unordered_map<const void*, int> derivativesStored_;
+    /** What the last training pass left in a forward memory. */
+    struct ForwardRecord
+    {
+        int numel = 0;
+        bool derivatives = false;   // position derivatives of the grids
+        bool inputOnly = false;     // of the intermediates only the encoded input
+    };
+    std::unordered_map<const void*, ForwardRecord> forwardRecords_;
+    /** Whether adjoint(flags) over numel points runs the layers again in its backward kernel instead of reading
+     *  their intermediates: a training pass that is followed by it keeps the encoded input only. */
+    bool recomputesFor(int numel, int flags) const;
+    /**
+     * recomputesFor(), and the backward kernel that runs the layers again holds its registers: loaded on the first
+     * call for these flags (it is the kernel that adjoint() will run), and not used if it spills more than a few
+     * words (16 -> 64 -> 64 -> 16 with biases: 27 gradient tiles and 72 registers of pre-activations, 316 bytes).
+     */
+    bool recomputes(int numel, int flags);
+    int recomputeVerdict_[ADJOINT_MODE_MAX_COMBINATIONS][2];   // -1: not known yet
+    static constexpr int MAX_RECOMPUTE_SCRATCH = 64;
     /** Bytes per point of the forward memory: intermediates and, where kept, position derivatives. */
     size_t forwardBytesPerPoint() const { return static_cast<size_t>(perEntryForwardMemoryBytes_) + static_cast<size_t>(derivativeBytesPerPoint_); }
     /** Whether a training pass over numel points that is followed by adjoint(flags) stores position derivatives. */
@@ -410,13 +436,13 @@ private:
     int registerVariantTiles(bool store) const;
     /** Workgroup size and tiles per wavefront of a shape of the forward kernel. */
     void forwardShape(bool store, int variant, int& blockSize, int& pointsPerLane) const;
-    void compileForwardKernel(bool store, int variant, bool compileOnly = false, bool derivatives = false);
+    void compileForwardKernel(bool store, int variant, bool compileOnly = false, bool derivatives = false, bool inputOnly = false);
     /**
      * The kernel shape for the next launch over a batch of numTiles tiles and, in launchTiles,
      * how many of them that launch should take (whole steps of a large shape first; the caller
      * asks again for the rest).
      */
-    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr, bool noAlloc = false, bool derivatives = false);
+    const CompiledKernel& forwardKernelFor(bool store, int numTiles, int* launchTiles = nullptr, bool noAlloc = false, bool derivatives = false, bool inputOnly = false);
     /** Points per launch of a forward kernel: the whole batch, or two passes of the grid for networks that gather. */
     int gatherChunkPoints(const CompiledKernel& ck) const;
     /** inference (store = false) or forward with stored intermediates, in one or several launches. */
@@ -427,8 +453,8 @@ private:
     int directInputStart() const;
     /** Throws unless every encoding with parameters has a tensor bound for 'usage'. */
     void checkEncodingParameters(Tensor::Usage usage) const;
-    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false, bool derivatives = false);
-    void compileBackwardKernel(int flags, bool sliceGradients = false, bool compileOnly = false);
+    void launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc = false, bool derivatives = false, bool inputOnly = false);
+    void compileBackwardKernel(int flags, bool sliceGradients = false, bool compileOnly = false, bool recompute = false);
     /** The records kernel of a batch of numel points (compiled on first use; compileOnly: all of them into the cache). */
     const CompiledKernel& recordsKernelFor(SliceGradientKernel& sk, int flags, int numel, bool fromDerivatives = false);
     /** Compiles (compileOnly: into the cache) or loads the two kernels of kernels/grid_gradient_columns.h for sk. */
@@ -439,8 +465,8 @@ private:
     size_t sortedTotalsOffset(int numel) const;
     void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives = false);
 
-    std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false, bool derivatives = false) const;
-    std::string backwardSource(int flags, int blockSize, bool sliceGradients = false) const;
+    std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false, bool derivatives = false, bool inputOnly = false) const;
+    std::string backwardSource(int flags, int blockSize, bool sliceGradients = false, bool recompute = false) const;
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const;
     void fillEncodingsAndActivations(std::string& codeTemplate) const;
@@ -453,7 +479,7 @@ private:
      *  tiles of all layers in its accumulation registers). */
     std::vector<bool> fusedWeightUpdateLayers(int adjointFlags, bool sliceGradients, bool* wideRegisters = nullptr) const;
     /** LDS halves per wavefront of the backward kernel for the tile that Layer::weightGradient transposes. */
-    int fusedWeightUpdateTransposeHalves() const;
+    int fusedWeightUpdateTransposeHalves(bool recompute = false) const;
     /** Channels of adjoint pre-activations that the backward kernel stores per point for the weight-update kernels. */
     int storedAdjointChannels(int adjointFlags, bool sliceGradients) const;
     // Where a kernel finds the weights of a layer. RESIDENT: in LDS for the whole kernel.
@@ -484,7 +510,7 @@ private:
         int byteOffset = 0;  // of the region in the kernel's dynamic LDS
     };
     /** One entry per encoding; returns the LDS bytes of the backward kernel including these regions. */
-    int ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients = false) const;
+    int ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients = false, bool recompute = false) const;
     std::vector<char> encodingArguments(std::vector<void*>& args, std::vector<std::vector<char>>& storage);
     void ensureStreams();
 };

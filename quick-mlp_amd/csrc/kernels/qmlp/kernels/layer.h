@@ -229,6 +229,47 @@ struct Layer
     }
 
     /**
+     * forward<false> that also hands out the pre-activations, in the layout in which forward<true> stores them and
+     * adjoint reads them (lane: channels 16m + 4g + i of the points 4r + nt): the adjoint kernel of a network whose
+     * training pass kept the encoded input only runs the layers again (the same operations: the same bits) instead
+     * of reading 2 C_out bytes per point and layer back from memory.
+     */
+    __device__ __forceinline__ static void forwardKeep(const f16* __restrict__ w, const f16* __restrict__ bias,
+                                                       const f16x4 (&x)[NT][KT], f16x4 (&pre)[NT][MT], f16x4 (&y)[NT][MT], int lane)
+    {
+        const int g = lane >> 4;
+        const f16x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            f32x4 acc[NT];
+            if constexpr (BIAS) {
+                const f16x4 b = *reinterpret_cast<const f16x4*>(bias + 16 * m + 4 * g);
+                const f32x4 bf = {static_cast<float>(b[0]), static_cast<float>(b[1]),
+                                  static_cast<float>(b[2]), static_cast<float>(b[3])};
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = bf;
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int kb = 0; kb < F_KB; ++kb) {
+                const f16x8 a = forwardOperand<false>(w, m, kb, lane);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const f16x4 hi = (2 * kb + 1 < KT) ? x[nt][(2 * kb + 1 < KT) ? 2 * kb + 1 : 0] : zero4;
+                    acc[nt] = mfma32(a, concat(x[nt][2 * kb], hi), acc[nt]);
+                }
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                pre[nt][m] = toF16(acc[nt]);
+                y[nt][m] = activationForwardChannels<Activation>(pre[nt][m], 16 * m + 4 * g);
+            }
+        }
+    }
+
+    /**
      * Adjoint pass of the layer for one 64-point tile.
      * \param wT transposed weights: LDS copy in adjoint operand order, or (GLOBAL_W) the
      *        row-major (CIN, COUT) matrix in global memory
@@ -284,6 +325,65 @@ struct Layer
         }
     }
 
+    /**
+     * adjoint<true, COMPUTE_DX, false, false, T_STRIDE> with the pre-activations in registers (forwardKeep) instead of
+     * in memory: the adjoint pre-activations go to the wavefront's LDS tile for weightGradient.
+     */
+    template <bool COMPUTE_DX>
+    __device__ __forceinline__ static void adjointKept(const f16* __restrict__ wT, f16x4 (&dy)[NT][MT], f16x4 (&dx)[NT][KT],
+                                                       const f16x4 (&pre)[NT][MT], f16* __restrict__ dpreTile, int validMask, int lane)
+    {
+        const int g = lane >> 4, r = lane & 15;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f16x4 d;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const half a = activationAdjointChannel<Activation>(toHalf(pre[nt][m][i]), toHalf(dy[nt][m][i]), 16 * m + 4 * g + i);
+                    d[nt] = ((validMask >> nt) & 1) ? fromHalf(a) : static_cast<f16>(0);
+                    dy[nt][m][i] = d[nt];
+                }
+                *reinterpret_cast<f16x4*>(dpreTile + (16 * m + 4 * g + i) * (TILE_POINTS + 8) + 4 * r) = d;
+            }
+        }
+        if constexpr (COMPUTE_DX) {
+            const f16x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+            for (int mi = 0; mi < KT; ++mi) {
+                f32x4 acc[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kb = 0; kb < A_KB; ++kb) {
+                    const f16x8 a = adjointOperand<false>(wT, mi, kb, lane);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const f16x4 hi = (2 * kb + 1 < MT) ? dy[nt][(2 * kb + 1 < MT) ? 2 * kb + 1 : 0] : zero4;
+                        acc[nt] = mfma32(a, concat(dy[nt][2 * kb], hi), acc[nt]);
+                    }
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) dx[nt][mi] = toF16(acc[nt]);
+            }
+        }
+    }
+
+    /** The input of the layer (before the activation of the layer in front of it), from registers into the
+     *  wavefront's LDS tile of CIN rows of T_STRIDE halves that weightGradient<.., T_STRIDE> reads. */
+    __device__ __forceinline__ static void stageInput(const f16x4 (&x)[NT][KT], f16* __restrict__ inTile, int lane)
+    {
+        const int g = lane >> 4, r = lane & 15;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16x4 v = {x[0][t][i], x[1][t][i], x[2][t][i], x[3][t][i]};
+                *reinterpret_cast<f16x4*>(inTile + (16 * t + 4 * g + i) * (TILE_POINTS + 8) + 4 * r) = v;
+            }
+    }
+
     // halves between the channel rows of the tile that weightGradient transposes in LDS: 64 points and 16 bytes,
     // so that the sixteen rows a 16-byte operand read touches start in different banks
     static constexpr int T_STRIDE = TILE_POINTS + 8;
@@ -301,9 +401,10 @@ struct Layer
      * applied again (as WeightUpdateKernel does, which this replaces for networks whose gradient tiles fit into
      * the registers of a wavefront; replaces network_weight_update_block.cuh:356-494 of the reference).
      * \param sTile T_HALVES halves of LDS of this wavefront: the adjoint pre-activations (zero for points outside the batch)
-     * \param inTile (CIN, 64) halves: the stored input of the layer before InputActivation
+     * \param inTile CIN rows of IN_STRIDE halves (64 points each): the input of the layer before InputActivation, as
+     *        the forward kernel stored it, or (IN_STRIDE = T_STRIDE) as stageInput put it into LDS
      */
-    template <typename InputActivation>
+    template <typename InputActivation, int IN_STRIDE = TILE_POINTS>
     __device__ __forceinline__ static void weightGradient(const f16* sTile, const f16* __restrict__ inTile,
                                                           f32x4 (&accW)[MT][KT], f32x4& accB, int lane)
     {
@@ -319,7 +420,7 @@ struct Layer
 #pragma unroll
             for (int k = 0; k < KT; ++k) {
                 const int channel = 16 * k + r;
-                const f16x8 raw = *reinterpret_cast<const f16x8*>(inTile + channel * TILE_POINTS + 32 * kb + 8 * g);
+                const f16x8 raw = *reinterpret_cast<const f16x8*>(inTile + channel * IN_STRIDE + 32 * kb + 8 * g);
                 b[k] = activationForwardChannel<InputActivation>(raw, channel);
             }
 #pragma unroll

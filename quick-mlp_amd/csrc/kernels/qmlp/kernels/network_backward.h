@@ -8,7 +8,9 @@
 // staged transposed). For the weight gradients dpre is either stored for the weight-update
 // kernels or, where the gradient tiles of all layers fit into the registers of a wavefront,
 // contracted with the layer input right here (Layer::weightGradient), the workgroup storing
-// its partial sums after its last tile. The adjoint of
+// its partial sums after its last tile. Where all layers are summed here, the training pass may
+// have kept the encoded input only: the kernel then runs the layers forward once more per tile
+// (Layer::forwardKeep) instead of reading their pre-activations back. The adjoint of
 // the encoded input finally goes through the LDS staging rows to one lane per point,
 // which accumulates input gradients and scatter-adds grid gradients with hardware
 // fp32 atomics.
@@ -116,6 +118,9 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     // FUSED_WEIGHT_UPDATE: this wavefront's tile of adjoint pre-activations, a row of 64 points per channel
     f16* sTranspose = reinterpret_cast<f16*>(sMemory + $$OFFSET_TRANSPOSE$$) + wave * $$TRANSPOSE_HALVES$$;
     (void)sTranspose;
+    // RECOMPUTE: behind it, this wavefront's tile of the input of the layer whose weight gradients are being summed
+    f16* sLayerInput = sTranspose + $$LAYER_INPUT_OFFSET$$;
+    (void)sLayerInput;
 
     // stage the transposed weights in operand order
 $$STAGE_PARAMETERS$$
@@ -185,6 +190,8 @@ $$ZERO_LDS_GRADIENTS$$
             }
         }
 
+        // RECOMPUTE: the training pass kept the encoded input only; the layers run again, their pre-activations stay in registers
+$$RECOMPUTE_FORWARD$$
         // layers, last to first
 $$CALL_NETWORK_LAYERS$$
 

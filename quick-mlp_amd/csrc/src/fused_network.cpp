@@ -86,6 +86,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
         compileOptions_.sliceGradients = options.value("slice_gradients", compileOptions_.sliceGradients);
         compileOptions_.inputDerivatives = options.value("input_derivatives", compileOptions_.inputDerivatives);
         compileOptions_.columnGradients = options.value("column_gradients", compileOptions_.columnGradients);
+        compileOptions_.recomputeIntermediates = options.value("recompute_intermediates", compileOptions_.recomputeIntermediates);
         compileOptions_.fusedWeightUpdate = options.value("fused_weight_update", compileOptions_.fusedWeightUpdate);
         compileOptions_.skewSharedMemory = options.value("skew_shared_memory", compileOptions_.skewSharedMemory);
         compileOptions_.parallelWeightUpdate =
@@ -219,6 +220,7 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
     }
     perEntryForwardMemoryBytes_ = offsetFwd * static_cast<int>(sizeof(half));
 
+    for (auto& perFlags : recomputeVerdict_) perFlags[0] = perFlags[1] = -1;
     // behind the intermediates: the position derivatives of the grids whose gradients take the slice kernels
     derivativeOffsets_.assign(encodings_.size(), -1);
     derivativeBytesPerPoint_ = 0;
@@ -230,6 +232,40 @@ FusedNetwork::FusedNetwork(const json& cfg, const std::filesystem::path& parent)
             derivativeBytesPerPoint_ += layout.derivativeBytesPerPoint;
         }
     }
+}
+
+bool FusedNetwork::recomputesFor(int numel, int flags) const
+{
+    if (compileOptions_.recomputeIntermediates == 0 || flags <= 0 || flags >= ADJOINT_MODE_MAX_COMBINATIONS) return false;
+    if (!(flags & GRADIENTS_NETWORK_WEIGHTS)) return false;
+    // the backward kernel of these flags sums the weight gradients of every layer itself ...
+    const bool sliceGradients = useSliceGradients(numel, flags);
+    for (bool fused : fusedWeightUpdateLayers(flags, sliceGradients))
+        if (!fused) return false;
+    // ... and has room for the weights in both operand orders and for a second tile per wavefront
+    for (int p : weightPlacement(false))
+        if (p != WEIGHTS_RESIDENT) return false;
+    const int blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
+    std::vector<LdsGradients> unused;
+    const int lds = roundUp(ldsGradientLayout(flags, blockSize, unused, sliceGradients, true), 16)
+        + (blockSize / WARP_SIZE) * fusedWeightUpdateTransposeHalves(true) * static_cast<int>(sizeof(half));
+    return lds <= MaxSharedMemoryBytes();
+}
+
+bool FusedNetwork::recomputes(int numel, int flags)
+{
+    if (!recomputesFor(numel, flags)) return false;
+    const bool sliceGradients = useSliceGradients(numel, flags);
+    int& verdict = recomputeVerdict_[flags][sliceGradients ? 1 : 0];
+    if (verdict < 0) {
+        compileBackwardKernel(flags, sliceGradients, false, true);
+        const auto& kernel = backwardKernel_[flags][sliceGradients ? 1 : 0][1].value().adjoint;
+        verdict = kernel.fun.scratchBytes() <= MAX_RECOMPUTE_SCRATCH ? 1 : 0;
+        if (!verdict)
+            QuickMLP::Instance().getLogger()->debug("the backward kernel that runs the layers again (flags %d) spills %d bytes per lane, not used",
+                                                    flags, kernel.fun.scratchBytes());
+    }
+    return verdict == 1;
 }
 
 bool FusedNetwork::storesDerivatives(int numel, int flags) const
@@ -688,11 +724,15 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
     return fused;
 }
 
-int FusedNetwork::fusedWeightUpdateTransposeHalves() const
+int FusedNetwork::fusedWeightUpdateTransposeHalves(bool recompute) const
 {
-    int widest = 0;
-    for (const auto& l : layers_) widest = std::max(widest, l.channelsOut);
-    return widest * (TILE_POINTS + 8);   // Layer::T_HALVES
+    int widest = 0, widestIn = 0;
+    for (const auto& l : layers_) {
+        widest = std::max(widest, l.channelsOut);
+        widestIn = std::max(widestIn, l.channelsIn);
+    }
+    // Layer::T_HALVES; behind it, where the layers run again in the backward kernel, the tile of a layer's input
+    return (widest + (recompute ? widestIn : 0)) * (TILE_POINTS + 8);
 }
 
 int FusedNetwork::storedAdjointChannels(int adjointFlags, bool sliceGradients) const
@@ -714,7 +754,7 @@ static std::string layerTypedefs(const std::vector<std::string>& layerTypes)
     return ss.str();
 }
 
-std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool registerStaging, bool derivatives) const
+std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool registerStaging, bool derivatives, bool inputOnly) const
 {
     auto kl = QuickMLP::Instance().kernelLoader();
     std::string code = kl->findFile("qmlp/kernels/network_forward.h").value();
@@ -795,10 +835,12 @@ std::string FusedNetwork::forwardSource(int blockSize, int pointsPerLane, bool r
             callLayers << "        materialize(x" << i << ");\n        __syncthreads();   // the stream buffer is free\n        Layer" << i
                        << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + " << ldsW[i]
                        << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
+        // (inputOnly: of the intermediates a training pass keeps the encoded input only; the backward kernel runs the layers again)
+        const char* storeLayer = inputOnly ? "false" : "STORE";
         if (placement[i] != WEIGHTS_GLOBAL)
-            callLayers << "        Layer" << i << "::template forward<STORE, false, HAS_STREAMED_LAYERS>(sParams + " << ldsW[i] << ", ";
+            callLayers << "        Layer" << i << "::template forward<" << storeLayer << ", false, HAS_STREAMED_LAYERS>(sParams + " << ldsW[i] << ", ";
         else
-            callLayers << "        Layer" << i << "::template forward<STORE, true, HAS_STREAMED_LAYERS>(networkParameters + " << l.weightsStart
+            callLayers << "        Layer" << i << "::template forward<" << storeLayer << ", true, HAS_STREAMED_LAYERS>(networkParameters + " << l.weightsStart
                        << ", ";
         if (l.useBias)
             callLayers << "sParams + " << ldsB[i];
@@ -852,10 +894,13 @@ bool FusedNetwork::useSliceGradients(int numel, int flags) const
     return false;
 }
 
-int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients) const
+int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector<LdsGradients>& perEncoding, bool sliceGradients,
+                                    bool recompute) const
 {
     perEncoding.assign(encodings_.size(), LdsGradients{});
-    int bytes = ldsParamHalves(true) * static_cast<int>(sizeof(half)) + (blockSize / WARP_SIZE) * stageBytesPerWave(true);
+    // (recompute: the weights in forward operand order and the biases behind the transposed weights)
+    int bytes = (ldsParamHalves(true) + (recompute ? ldsParamHalves(false) : 0)) * static_cast<int>(sizeof(half))
+        + (blockSize / WARP_SIZE) * stageBytesPerWave(true);
     if (!(adjointFlags & GRADIENTS_INPUT_ENCODINGS)) return bytes;
     // Up to 96 KiB of LDS per workgroup in total: a coarse level of a grid fits (16^3 cells with
     // 2 features: 32 KiB), and a second workgroup per compute unit stays possible.
@@ -874,7 +919,7 @@ int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector
     return bytes;
 }
 
-std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGradients) const
+std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGradients, bool recompute) const
 {
     const bool hasInputGradients = flags & GRADIENTS_INPUT;
     const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
@@ -886,13 +931,20 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
     bool wideRegisters = false;
     (void)fusedWeightUpdateLayers(flags, sliceGradients, &wideRegisters);
+    // (the pre-activations of all layers stay in registers beside the gradient tiles: 256 registers spilled 404 bytes
+    // per lane for 16 -> 32 -> 32 -> 32 -> 16)
+    wideRegisters = wideRegisters || recompute;
     replaceAll(code, "$$KERNEL_ATTRIBUTES$$", wideRegisters ? std::string("__attribute__((amdgpu_waves_per_eu(1, 1)))") : kernelAttributes(blockSize));
     // (set below: input gradients that the kernels of the gradient slices compute are none of this kernel's)
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
     replaceAll(code, "$$HAS_ENCODING_GRADIENTS$$", hasEncodingGradients ? "true" : "false");
     std::vector<int> ldsW, ldsB;
     int streamOffset = -1;
-    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(ldsLayout(true, ldsW, ldsB, &streamOffset)));
+    const int adjointParamHalves = ldsLayout(true, ldsW, ldsB, &streamOffset);
+    // recompute: the weights in forward operand order and the biases, behind the transposed weights
+    std::vector<int> ldsWForward, ldsBForward;
+    const int forwardParamHalves = recompute ? ldsLayout(false, ldsWForward, ldsBForward) : 0;
+    replaceAll(code, "$$LDS_PARAM_HALVES$$", std::to_string(adjointParamHalves + forwardParamHalves));
     const auto placement = weightPlacement(true);
 
     std::vector<std::string> layerTypes;
@@ -911,6 +963,16 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
         const auto& l = layers_[i];
         stage << "    Layer" << i << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + "
               << ldsW[i] << ", threadIdx.x, blockDim.x);\n";
+    }
+    if (recompute) {
+        for (size_t i = 0; i < layers_.size(); ++i) {
+            const auto& l = layers_[i];
+            stage << "    Layer" << i << "::stageForward(networkParameters + " << l.weightsStart << ", sParams + "
+                  << (adjointParamHalves + ldsWForward[i]) << ", threadIdx.x, blockDim.x);\n";
+            if (l.useBias)
+                stage << "    for (int i = threadIdx.x; i < " << l.channelsOut << "; i += blockDim.x) sParams["
+                      << (adjointParamHalves + ldsBForward[i]) << " + i] = networkParameters[" << l.biasStart << " + i];\n";
+        }
     }
     replaceAll(code, "$$STAGE_PARAMETERS$$", stage.str());
 
@@ -936,6 +998,23 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
             callLayers << "        materialize(" << dy << ");\n        __syncthreads();   // the stream buffer is free\n        Layer" << i
                        << "::stageAdjoint(networkParameters + " << l.weightsStart << ", sParams + " << ldsW[i]
                        << ", threadIdx.x, blockDim.x);\n        __syncthreads();\n";
+        }
+        if (recompute) {
+            // (every layer is summed here: recomputesFor())
+            const std::string inputActivation = i > 0 ? "activations::" + activationTypeName(i - 1) : std::string("activations::passthrough_");
+            callLayers << "        Layer" << i << "::template adjointKept<" << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << ">(" << weights << ", "
+                       << dy << ", dx" << i << ", pre" << i << ", sTranspose, validMask, lane);\n"
+                       << "        Layer" << i << "::stageInput(" << (i == 0 ? std::string("x0Kept") : "pre" + std::to_string(i - 1))
+                       << ", sLayerInput, lane);\n"
+                       << "        Layer" << i << "::template weightGradient<" << inputActivation << ", Layer" << i
+                       << "::T_STRIDE>(sTranspose, sLayerInput, accW" << i << ", accB" << i << ", lane);\n";
+            declareGradients << "    f32x4 accW" << i << "[Layer" << i << "::MT][Layer" << i << "::KT], accB" << i << " = {0.f, 0.f, 0.f, 0.f};\n"
+                             << "    zeroTiles(accW" << i << ");\n";
+            storeGradients << "    Layer" << i << "::template storeWeightGradient<WAVES>(accW" << i << ", accB" << i
+                           << ", reinterpret_cast<float*>(sMemory),\n        partialGradients + (static_cast<long long>(blockIdx.x) * NUM_PARAMETERS + "
+                           << l.weightsStart << "), partialGradients + (static_cast<long long>(blockIdx.x) * NUM_PARAMETERS + "
+                           << (l.useBias ? l.biasStart : 0) << "), partialSlices, NUM_PARAMETERS, wave, lane);\n";
+            continue;
         }
         callLayers << "        Layer" << i << "::template adjoint<" << (fused ? "true" : "STORE_DPRE") << ", "
                    << (i == 0 ? "NEEDS_ENCODING_ADJOINT" : "true") << (placement[i] == WEIGHTS_GLOBAL ? ", true" : ", false")
@@ -967,8 +1046,31 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     replaceAll(code, "$$STORE_WEIGHT_GRADIENTS$$", storeGradients.str());
     {
         std::vector<LdsGradients> unused;
-        replaceAll(code, "$$OFFSET_TRANSPOSE$$", std::to_string(roundUp(ldsGradientLayout(flags, blockSize, unused, sliceGradients), 16)));
-        replaceAll(code, "$$TRANSPOSE_HALVES$$", std::to_string(anyFused ? fusedWeightUpdateTransposeHalves() : 0));
+        replaceAll(code, "$$OFFSET_TRANSPOSE$$", std::to_string(roundUp(ldsGradientLayout(flags, blockSize, unused, sliceGradients, recompute), 16)));
+        replaceAll(code, "$$TRANSPOSE_HALVES$$", std::to_string(anyFused ? fusedWeightUpdateTransposeHalves(recompute) : 0));
+        replaceAll(code, "$$LAYER_INPUT_OFFSET$$", std::to_string(fusedWeightUpdateTransposeHalves(false)));
+    }
+    {
+        // recompute: the encoded input of the tile as the forward kernel stored it (channel-major, four points per
+        // load: the layout of the matrix-core operands of the first layer), then the layers, first to last
+        std::stringstream forward;
+        if (recompute) {
+            forward << "        f16x4 x0Kept[NT][Layer0::KT];\n        {\n"
+                    << "            const f16* encTile = forwardTmpMemory + static_cast<long long>(tileRead) * (CHANNELS_IN * TILE_POINTS);\n"
+                    << "#pragma unroll\n            for (int t = 0; t < KT0; ++t)\n#pragma unroll\n                for (int i = 0; i < 4; ++i) {\n"
+                    << "                    const f16x4 v = *reinterpret_cast<const f16x4*>(encTile + (16 * t + 4 * g + i) * TILE_POINTS + 4 * r);\n"
+                    << "#pragma unroll\n                    for (int nt = 0; nt < NT; ++nt) x0Kept[nt][t][i] = v[nt];\n                }\n        }\n";
+            for (int i = 0; i < L; ++i) {
+                const auto& l = layers_[i];
+                const std::string in = i == 0 ? std::string("x0Kept") : "act" + std::to_string(i);
+                forward << "        f16x4 pre" << i << "[NT][Layer" << i << "::MT], act" << (i + 1) << "[NT][Layer" << i << "::MT];\n"
+                        << "        Layer" << i << "::forwardKeep(sParams + " << (adjointParamHalves + ldsWForward[i]) << ", "
+                        << (l.useBias ? "sParams + " + std::to_string(adjointParamHalves + ldsBForward[i]) : std::string("nullptr")) << ", " << in
+                        << ", pre" << i << ", act" << (i + 1) << ", lane);\n";
+            }
+            forward << "        (void)act" << L << ";\n";
+        }
+        replaceAll(code, "$$RECOMPUTE_FORWARD$$", forward.str());
     }
     callLayers << "        auto& dxIn = dx0;\n        (void)dxIn;\n";
     replaceAll(code, "$$CALL_NETWORK_LAYERS$$", callLayers.str());
@@ -1114,15 +1216,20 @@ std::string FusedNetwork::generatedSource(const std::string& kind, int adjointFl
     // the shape with the encoded rows in registers, whether or not the network would get it
     if (kind == "forward_registers") return forwardSource(2 * DEFAULT_BLOCK_SIZE, std::min(8, 256 / layers_[0].channelsIn), true);
     if (kind == "backward") return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true));
+    if (kind == "backward_recompute")   // the variant that runs the layers again, for networks that have one at these flags
+        return backwardSource(adjointFlags, forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true),
+                              useSliceGradients(1 << 30, adjointFlags), true);
     if (kind == "weight_update") return weightUpdateSource(weightUpdateBlockSize());
     if (kind == "backward_resources" || kind == "backward_slices_resources") {
         // what the loaded backward kernel takes (needs a device): for tests of the register budget
         const bool slices = kind == "backward_slices_resources";
-        compileBackwardKernel(adjointFlags, slices);
-        const auto& ak = backwardKernel_[adjointFlags][slices ? 1 : 0].value();
-        return format("{\"block\": %d, \"lds_bytes\": %d, \"registers\": %d, \"scratch_bytes\": %d, \"full_grid\": %d}",
+        // ("recompute": the kernel of a batch of that kind runs the layers again instead of reading their intermediates)
+        const bool recompute = useSliceGradients(slices ? (1 << 30) : 1, adjointFlags) == slices && recomputes(slices ? (1 << 30) : 1, adjointFlags);
+        compileBackwardKernel(adjointFlags, slices, false, recompute);
+        const auto& ak = backwardKernel_[adjointFlags][slices ? 1 : 0][recompute ? 1 : 0].value();
+        return format("{\"block\": %d, \"lds_bytes\": %d, \"registers\": %d, \"scratch_bytes\": %d, \"full_grid\": %d, \"recompute\": %s}",
                       ak.adjoint.blockSize, ak.adjoint.sharedMemorySize, ak.adjoint.fun.numVgprs(), ak.adjoint.fun.scratchBytes(),
-                      ak.adjoint.fullGrid);
+                      ak.adjoint.fullGrid, recompute ? "true" : "false");
     }
     throw std::runtime_error("unknown kernel kind '" + kind + "'");
 }
@@ -1197,10 +1304,11 @@ void FusedNetwork::forwardShape(bool store, int variant, int& blockSize, int& po
     }
 }
 
-void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnly, bool derivatives)
+void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnly, bool derivatives, bool inputOnly)
 {
     derivatives = derivatives && store;
-    auto& slot = forwardKernels_[derivatives ? 2 : store ? 1 : 0][variant];
+    inputOnly = inputOnly && store;
+    auto& slot = forwardKernels_[(derivatives ? 2 : store ? 1 : 0) + (inputOnly ? 2 : 0)][variant];
     if (slot.has_value() && !compileOnly) return;
     auto kl = QuickMLP::Instance().kernelLoader();
     CompiledKernel ck;
@@ -1211,26 +1319,29 @@ void FusedNetwork::compileForwardKernel(bool store, int variant, bool compileOnl
     ck.fun = kl->getKernel(derivatives ? "qmlp::kernel::NetworkKernelInferenceAndForward<true, true>"
                            : store     ? "qmlp::kernel::NetworkKernelInferenceAndForward<true>"
                                        : "qmlp::kernel::NetworkKernelInferenceAndForward<false>",
-                           forwardSource(ck.blockSize, ck.pointsPerLane, registerStaging, derivatives), loaderFlags(compileOnly)).value();
+                           forwardSource(ck.blockSize, ck.pointsPerLane, registerStaging, derivatives, inputOnly), loaderFlags(compileOnly)).value();
     if (compileOnly) return;
     ck.fullGrid = ck.fun.fullGridSize(ck.blockSize, ck.sharedMemorySize);
     QuickMLP::Instance().getLogger()->debug(
         "%s kernel, %d tile(s) per wave: block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d",
-        derivatives ? "forward (with position derivatives)" : store ? "forward" : "inference", ck.pointsPerLane, ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(),
+        inputOnly ? (derivatives ? "forward (encoded input and position derivatives only)" : "forward (encoded input only)")
+                  : derivatives ? "forward (with position derivatives)" : store ? "forward" : "inference", ck.pointsPerLane, ck.blockSize, ck.sharedMemorySize, ck.fun.numVgprs(),
         ck.fun.scratchBytes(), ck.fullGrid);
     slot = std::move(ck);
 }
 
-const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles, bool noAlloc, bool derivatives)
+const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, int numTiles, int* launchTiles, bool noAlloc, bool derivatives,
+                                                                  bool inputOnly)
 {
     derivatives = derivatives && store;
-    const int s = derivatives ? 2 : store ? 1 : 0;
+    inputOnly = inputOnly && store;
+    const int s = (derivatives ? 2 : store ? 1 : 0) + (inputOnly ? 2 : 0);
     // loading a kernel allocates device memory: a call that must not allocate only takes what is loaded
     auto loaded = [&](int variant) -> const CompiledKernel& {
         if (noAlloc && !forwardKernels_[s][variant].has_value())
             throw std::runtime_error("The kernel for a batch of this size is not loaded yet, and loading allocates: run "
                                      "inference() once on a batch of the same size first");
-        compileForwardKernel(store, variant, false, derivatives);
+        compileForwardKernel(store, variant, false, derivatives, inputOnly);
         return forwardKernels_[s][variant].value();
     };
     if (launchTiles) *launchTiles = numTiles;
@@ -1294,16 +1405,16 @@ const FusedNetwork::CompiledKernel& FusedNetwork::forwardKernelFor(bool store, i
         QuickMLP::Instance().getLogger()->debug("the forward kernel with rows in registers spills %d bytes per lane, not used",
                                                 forwardKernels_[s][best].value().fun.scratchBytes());
         registerShapeSpills_[s] = true;
-        return forwardKernelFor(store, numTiles, launchTiles, noAlloc, derivatives);
+        return forwardKernelFor(store, numTiles, launchTiles, noAlloc, derivatives, inputOnly);
     }
     return forwardKernels_[s][best].value();
 }
 
-void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool compileOnly)
+void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool compileOnly, bool recompute)
 {
     if (flags <= 0 || flags >= ADJOINT_MODE_MAX_COMBINATIONS) throw std::runtime_error("At least one derivative must be enabled");
     const int variant = sliceGradients ? 1 : 0;
-    if (backwardKernel_[flags][variant].has_value() && !compileOnly) return;
+    if (backwardKernel_[flags][variant][recompute ? 1 : 0].has_value() && !compileOnly) return;
     const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
     auto kl = QuickMLP::Instance().kernelLoader();
     auto logger = QuickMLP::Instance().getLogger();
@@ -1312,7 +1423,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
     ak.adjoint.blockSize = forwardBlockSize(compileOptions_.overwriteBlocksizeBackward, true);
     {
         std::vector<LdsGradients> ldsGradients;
-        ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients, sliceGradients);
+        ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients, sliceGradients, recompute);
     }
     ak.fusedLayers = fusedWeightUpdateLayers(flags, sliceGradients);
     ak.fusedWeightUpdate = false;
@@ -1327,10 +1438,10 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
             if (ak.fusedLayers[i]) widestTiles = std::max(widestTiles, mt * kt + (l.useBias ? 1 : 0));
         }
         ak.adjoint.sharedMemorySize = std::max(roundUp(ak.adjoint.sharedMemorySize, 16) + (ak.adjoint.blockSize / WARP_SIZE)
-                                                   * fusedWeightUpdateTransposeHalves() * static_cast<int>(sizeof(half)),
+                                                   * fusedWeightUpdateTransposeHalves(recompute) * static_cast<int>(sizeof(half)),
                                                widestTiles * 256 * static_cast<int>(sizeof(float)));
     }
-    const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients);
+    const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients, recompute);
     ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
     {
         std::vector<long long> transposed;
@@ -1342,7 +1453,8 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
     }
     if (!compileOnly) {
         ak.adjoint.fullGrid = ak.adjoint.fun.fullGridSize(ak.adjoint.blockSize, ak.adjoint.sharedMemorySize);
-        logger->debug("backward kernel (flags %d): block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d", flags,
+        logger->debug("backward kernel (flags %d%s): block %d, LDS %d bytes, %d VGPRs, %d bytes scratch, full grid %d", flags,
+                      recompute ? ", the layers run again" : "",
                       ak.adjoint.blockSize, ak.adjoint.sharedMemorySize, ak.adjoint.fun.numVgprs(),
                       ak.adjoint.fun.scratchBytes(), ak.adjoint.fullGrid);
     }
@@ -1424,7 +1536,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
             }
         }
     }
-    if (!compileOnly) backwardKernel_[flags][variant] = std::move(ak);
+    if (!compileOnly) backwardKernel_[flags][variant][recompute ? 1 : 0] = std::move(ak);
 }
 
 void FusedNetwork::compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives)
@@ -1507,6 +1619,24 @@ void FusedNetwork::precompile(int adjointFlags)
         if (ppl > 1) compileForwardKernel(store, VARIANT_NARROW, true);
         if (hasLargeVariant(store)) compileForwardKernel(store, VARIANT_LARGE, true);
         if (registerVariantTiles(store) > 0) compileForwardKernel(store, VARIANT_REGISTERS, true);
+    }
+    if (adjointFlags > 0) {
+        // training passes that keep the encoded input only, and the backward kernels that run the layers again
+        bool any = false;
+        for (int numel : {1, 1 << 30}) {
+            if (!recomputesFor(numel, adjointFlags)) continue;
+            any = true;
+            compileBackwardKernel(adjointFlags, useSliceGradients(numel, adjointFlags), true, true);
+        }
+        if (any)
+            for (int derivatives = 0; derivatives <= (storesDerivatives(1 << 30, adjointFlags) ? 1 : 0); ++derivatives) {
+                compileForwardKernel(true, VARIANT_DEFAULT, true, derivatives != 0, true);
+                int ppl = 1;
+                forwardBlockSize(-1, false, &ppl);
+                if (ppl > 1) compileForwardKernel(true, VARIANT_NARROW, true, derivatives != 0, true);
+                if (hasLargeVariant(true)) compileForwardKernel(true, VARIANT_LARGE, true, derivatives != 0, true);
+                if (registerVariantTiles(true) > 0) compileForwardKernel(true, VARIANT_REGISTERS, true, derivatives != 0, true);
+            }
     }
     if (adjointFlags > 0 && storesDerivatives(1 << 30, adjointFlags)) {
         // training passes that keep the position derivatives of their grids
@@ -1614,7 +1744,8 @@ void FusedNetwork::inferenceNoAlloc(const Tensor& input, Tensor& output, stream_
     launchForward(false, input, output, nullptr, stream, true);
 }
 
-void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc, bool derivatives)
+void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output, half* tmpMemory, stream_t stream, bool noAlloc, bool derivatives,
+                                 bool inputOnly)
 {
     const int numel = input.size(0);
     int tmpNumTiles = divUp(numel, TILE_POINTS);
@@ -1630,7 +1761,8 @@ void FusedNetwork::launchForward(bool store, const Tensor& input, Tensor& output
     for (long long start = 0; start < numel;) {
         // the kernel shape for what is left; a network that gathers gets at most two steps of it per launch
         int launchTiles = 0;
-        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, noAlloc, derivatives);
+        const auto& ck = forwardKernelFor(store, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, noAlloc, derivatives,
+                                          inputOnly);
         int count = static_cast<int>(std::min<long long>(
             {static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS, numel - start}));
         auto inputAcc = inputAll;
@@ -1687,7 +1819,7 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
         for (long long start = 0; start < numel;) {
             int launchTiles = 0;
             const auto& ck = forwardKernelFor(store != 0, static_cast<int>(divUp<long long>(numel - start, TILE_POINTS)), &launchTiles, false,
-                                              store != 0 && storesDerivatives(numel, adjointFlags));
+                                              store != 0 && storesDerivatives(numel, adjointFlags), store != 0 && recomputes(numel, adjointFlags));
             start += std::min<long long>({static_cast<long long>(gatherChunkPoints(ck)), static_cast<long long>(launchTiles) * TILE_POINTS,
                                           numel - start});
         }
@@ -1708,8 +1840,9 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
     }
     if (adjointFlags > 0) {
         const bool sliceGradients = useSliceGradients(numel, adjointFlags);
-        compileBackwardKernel(adjointFlags, sliceGradients);
-        for (auto& sk : backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value().sliceGradients)
+        const bool recompute = recomputes(numel, adjointFlags);
+        compileBackwardKernel(adjointFlags, sliceGradients, false, recompute);
+        for (auto& sk : backwardKernel_[adjointFlags][sliceGradients ? 1 : 0][recompute ? 1 : 0].value().sliceGradients)
         {
             (void)recordsKernelFor(sk, adjointFlags, numel, storesDerivatives(numel, adjointFlags) && sk.derivativeOffset >= 0);
             if (sk.columnsOffered && sortsTraining(numel))
@@ -1854,9 +1987,10 @@ void FusedNetwork::forward(const Tensor& input, Tensor& output, void* tmpMemory,
     CHECK_ERROR(reinterpret_cast<uintptr_t>(tmpMemory) % 16 == 0, "The temporary memory must be aligned to 16 bytes");
 
     const bool derivatives = storesDerivatives(numel, announcedFlags_);
-    if (derivatives) derivativesStored_[tmpMemory] = numel;
-    else derivativesStored_.erase(tmpMemory);
-    launchForward(true, input, output, static_cast<half*>(tmpMemory), stream, false, derivatives);
+    const bool inputOnly = recomputes(numel, announcedFlags_);
+    if (derivatives || inputOnly) forwardRecords_[tmpMemory] = ForwardRecord{numel, derivatives, inputOnly};
+    else forwardRecords_.erase(tmpMemory);
+    launchForward(true, input, output, static_cast<half*>(tmpMemory), stream, false, derivatives, inputOnly);
 }
 
 void FusedNetwork::zeroGradients()
@@ -1954,15 +2088,32 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     const bool sliceGradients = useSliceGradients(numel, adjointFlags);
     CHECK_ERROR(!sliceGradients || numel < (1 << 27), "batches of 2^27 points or more: set options.slice_gradients to 0");
     announcedFlags_ = adjointFlags;
-    // whether the forward pass that wrote this forward memory kept the position derivatives of the grids
-    bool derivativesStored = false;
+    // what the forward pass that wrote this forward memory left there: the position derivatives of the grids? Of the
+    // intermediates the encoded input only?
+    bool derivativesStored = false, recompute = false;
     {
-        const auto it = derivativesStored_.find(tmpMemoryForward);
-        derivativesStored = hasInputGradients && sliceGradients && it != derivativesStored_.end() && it->second == numel;
+        const auto it = forwardRecords_.find(tmpMemoryForward);
+        if (it != forwardRecords_.end() && it->second.numel == numel) {
+            derivativesStored = hasInputGradients && sliceGradients && it->second.derivatives;
+            if (it->second.inputOnly) {
+                if (recomputes(numel, adjointFlags)) {
+                    recompute = true;
+                } else {
+                    // Announced otherwise: the kernels of these flags read intermediates that the training pass did not
+                    // keep. The forward pass runs again into the same memory, this time storing them (a batch that
+                    // trains in sorted order is sorted again: rows, order and slab totals are rewritten together).
+                    QuickMLP::Instance().getLogger()->debug("adjoint(flags %d): the forward pass kept the encoded input only; it runs again", adjointFlags);
+                    Tensor scratchOutput(precisionOut(), {numel, channelsOut()});
+                    const bool derivatives = it->second.derivatives;
+                    it->second.inputOnly = false;
+                    launchForward(true, input, scratchOutput, static_cast<half*>(const_cast<void*>(tmpMemoryForward)), stream, false, derivatives, false);
+                }
+            }
+        }
     }
     const bool sortedPoints = sortsTraining(numel);
-    compileBackwardKernel(adjointFlags, sliceGradients);
-    auto& ak = backwardKernel_[adjointFlags][sliceGradients ? 1 : 0].value();
+    compileBackwardKernel(adjointFlags, sliceGradients, false, recompute);
+    auto& ak = backwardKernel_[adjointFlags][sliceGradients ? 1 : 0][recompute ? 1 : 0].value();
 
     const int numTiles = divUp(numel, TILE_POINTS);
     const long long numel64 = static_cast<long long>(numTiles) * TILE_POINTS;
@@ -2184,7 +2335,9 @@ void FusedNetwork::clearCachedKernels()
     for (auto& perStore : forwardKernels_)
         for (auto& k : perStore) k = {};
     for (int i = 0; i < ADJOINT_MODE_MAX_COMBINATIONS; ++i)
-        for (auto& k : backwardKernel_[i]) k = {};
+        for (auto& perSlices : backwardKernel_[i])
+            for (auto& k : perSlices) k = {};
+    for (auto& perFlags : recomputeVerdict_) perFlags[0] = perFlags[1] = -1;
     pointOrder_.scan = {};
     pointOrder_.count = {};
     pointOrder_.scatter = {};

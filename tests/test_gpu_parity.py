@@ -1376,3 +1376,78 @@ def test_grid_gradients_summed_by_columns_match_the_records_the_atomic_scatter_a
     ok = ~np.isnan(a)
     scale = float(np.abs(a[ok]).max())
     assert np.allclose(a[ok] / scale, b[ok] / scale, rtol=1e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("which", ["hashgrid", "identity"])
+def test_backward_kernel_that_runs_the_layers_again_gives_the_same_bits(which):
+    """options.recompute_intermediates (default: when announced): where the backward kernel sums the weight gradients
+    of all layers, the training pass keeps the encoded input only and the backward kernel runs the layers again per
+    tile (Layer::forwardKeep: the same operations as the forward kernel, so the same pre-activations bit for bit)
+    instead of reading 2 x sum(C_out) bytes per point back. Against the same network with the option off: outputs,
+    input and weight gradients bit for bit, grid gradients up to the order of their float atomics. An adjoint pass
+    with other flags than announced, whose kernels need the stored intermediates, makes the forward pass run again."""
+    if which == "hashgrid":
+        grid = {"id": "HashGrid", "start_in": 0, "n_in": 3, "n_levels": 8, "n_features_per_level": 2,
+                "log2_hashmap_size": 12, "min_resolution": 4, "max_resolution": 256, "combination_mode": "concat",
+                "bounding_box_min": [-0.5, 0.0, 0.25], "bounding_box_size": [1.0, 2.0, 0.5], "parameter_precision": "half"}
+        base = {"num_inputs": 3, "num_outputs": 3, "activation_specification": ["qmlp/builtin-activations.json"],
+                "encodings": [grid],
+                "network": [{"n_out": 64, "bias": True, "activation": "celu"}, {"n_out": 48, "bias": False, "activation": "sine"},
+                            {"n_out": 3, "bias": True, "activation": "identity"}]}
+        options, n_in = {"slice_gradients": 1}, 3
+    else:
+        base = identity_cfg(7, [32, 64, 5], ["sine", "celu", "identity"], [True, True, False])
+        options, n_in = {}, 7
+    on, off = dict(base, options=options), dict(base, options=dict(options, recompute_intermediates=0))
+    warm_cache(on, off)
+    cases = {"on": Case(on), "off": Case(off)}
+    rng = np.random.default_rng(41)
+    params = random_parameters(cases["on"].oracle, rng)
+    for c in cases.values():
+        c.set_parameters(params)
+        if which == "hashgrid":
+            c.set_table(0, rng.uniform(-1, 1, c.oracle.encodings[0][1].n_params) if c is cases["on"] else cases["on"].tables_np[0])
+    N = 5003
+    if which == "hashgrid":
+        lo, sz = np.array(grid["bounding_box_min"], np.float32), np.array(grid["bounding_box_size"], np.float32)
+        X = (lo + sz * rng.uniform(0, 1, (N, 3))).astype(np.float32)
+    else:
+        X = rng.uniform(-1, 1, (N, n_in)).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, base["num_outputs"])) / 16).astype(np.float32)
+    full = (FLAG_INPUT | FLAG_WEIGHTS | FLAG_ENC) if which == "hashgrid" else (FLAG_INPUT | FLAG_WEIGHTS)
+    # the kernel that runs for these flags
+    kind = "backward_slices_resources" if which == "hashgrid" else "backward_resources"
+    assert json.loads(cases["on"].net.generated_source(kind, full))["recompute"] is True
+    assert json.loads(cases["off"].net.generated_source(kind, full))["recompute"] is False
+    assert "forwardKeep" in cases["on"].net.generated_source("backward_recompute", full)
+    got = {k: c.gpu_train(X, adj, full) for k, c in cases.items()}
+    assert np.array_equal(got["on"]["out"], got["off"]["out"])
+    assert np.array_equal(got["on"]["adj_x"], got["off"]["adj_x"])
+    assert np.array_equal(got["on"]["grads"], got["off"]["grads"])
+    if which == "hashgrid":
+        a, b = got["on"]["table_grads"][0], got["off"]["table_grads"][0]
+        s = float(np.abs(b).max())
+        assert np.allclose(a / s, b / s, rtol=1e-4, atol=2e-6)
+    check_gradients(cases["on"], X, adj, full, got["on"])
+    # announced with all gradients, asked for others: input gradients alone, weight gradients alone, ...
+    x, a = torch.from_numpy(X).cuda(), torch.from_numpy(adj).cuda()
+    on_case, off_case = cases["on"], cases["off"]
+    for flags in ([FLAG_INPUT, FLAG_WEIGHTS, FLAG_INPUT | FLAG_WEIGHTS] + ([FLAG_ENC, FLAG_WEIGHTS | FLAG_ENC] if which == "hashgrid" else [])):
+        _, tmp = on_case.net.forward_raw(x, on_case.params, on_case.encoding_parameters(), full)
+        adj_x, gnet, genc = on_case.net.adjoint_raw(x, a, flags, tmp, on_case.params, on_case.encoding_parameters())
+        want = off_case.gpu_train(X, adj, flags)
+        torch.cuda.synchronize()
+        if flags & FLAG_INPUT:
+            assert np.array_equal(adj_x.cpu().numpy(), want["adj_x"]), flags
+        if flags & FLAG_WEIGHTS:
+            assert np.array_equal(gnet.cpu().numpy(), want["grads"]), flags
+        if flags & FLAG_ENC:
+            s = float(np.abs(want["table_grads"][0]).max())
+            assert np.allclose(genc[0].cpu().numpy() / s, want["table_grads"][0] / s, rtol=1e-4, atol=2e-6), flags
+        # ... and once more with the same memory: whatever ran the first time left it complete
+        adj_x2, gnet2, _ = on_case.net.adjoint_raw(x, a, flags, tmp, on_case.params, on_case.encoding_parameters())
+        torch.cuda.synchronize()
+        if flags & FLAG_INPUT:
+            assert np.array_equal(adj_x2.cpu().numpy(), want["adj_x"]), flags
+        if flags & FLAG_WEIGHTS:
+            assert np.array_equal(gnet2.cpu().numpy(), want["grads"]), flags
