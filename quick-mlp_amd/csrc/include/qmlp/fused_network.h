@@ -165,7 +165,7 @@ private:
     struct PointOrder
     {
         std::optional<KernelFunction> count, scan, scatter;
-        std::optional<KernelFunction> gatherRows, scatterAddRows;   // rows of dL/dy into, rows of the input gradients out of the sorted order
+        std::optional<KernelFunction> gatherRows, gatherAddRows;   // rows of dL/dy into, rows of the input gradients out of the sorted order
         Tensor workspace;           // slab totals and per-chunk histograms (ints), sorted inputs (floats), order (ints)
         long long capacityWords = 0;   // 32-bit words the workspace holds
     };
@@ -463,6 +463,8 @@ private:
     static size_t columnWorkspaceBytes(const IEncoding::GradientColumnLayout& layout, long long numel, int* maxItems = nullptr);
     /** The slab totals of the sort of a training pass: behind the sorted rows and the order in the forward memory. */
     size_t sortedTotalsOffset(int numel) const;
+    /** Behind them: per point of the batch its place in the sorted order. */
+    size_t sortedPlacementOffset(int numel) const;
     void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false, bool derivatives = false, bool inputOnly = false) const;

@@ -1660,7 +1660,7 @@ void FusedNetwork::precompile(int adjointFlags)
             const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
             const std::string scatter = "PointOrderScatter<" + std::to_string(channelsIn_ <= 4 ? 4 : channelsIn_ <= 8 ? 8 : 16) + ">";
             for (const std::string& name : {std::string("PointOrderCount"), std::string("PointOrderScan"), scatter,
-                                            std::string("PointOrderGatherRows"), std::string("PointOrderScatterAddRows")})
+                                            std::string("PointOrderGatherRows"), std::string("PointOrderGatherAddRows")})
                 kl->getKernel("qmlp::kernel::" + name, source, loaderFlags(true));
             break;
         }
@@ -1804,7 +1804,7 @@ void FusedNetwork::loadPointOrderKernels(bool rowMoves)
     }
     if (rowMoves && !po.gatherRows.has_value()) {
         po.gatherRows = kl->getKernel("qmlp::kernel::PointOrderGatherRows", source, loaderFlags(false)).value();
-        po.scatterAddRows = kl->getKernel("qmlp::kernel::PointOrderScatterAddRows", source, loaderFlags(false)).value();
+        po.gatherAddRows = kl->getKernel("qmlp::kernel::PointOrderGatherAddRows", source, loaderFlags(false)).value();
     }
 }
 
@@ -1869,6 +1869,11 @@ size_t FusedNetwork::sortedTotalsOffset(int numel) const
     return sortedRowsOffset(numel) + roundUp(static_cast<size_t>(numel) * (channelsIn() + 1) * sizeof(float), size_t(256));
 }
 
+size_t FusedNetwork::sortedPlacementOffset(int numel) const
+{
+    return sortedTotalsOffset(numel) + SORT_SLABS * sizeof(int);
+}
+
 bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
                               bool noAlloc, void* destination)
 {
@@ -1926,6 +1931,9 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
     // a training pass keeps the points per slab with its sorted rows: the adjoint pass may walk the batch slab by slab
     static_assert(SLABS == SORT_SLABS, "the slabs of kernels/point_order.h");
     if (destination) totals = reinterpret_cast<int*>(static_cast<char*>(destination) + (sortedTotalsOffset(numel) - sortedRowsOffset(numel)));
+    // ... and for every point its place in the sorted order: rows computed in that order are gathered back with it
+    int* placement = destination ? reinterpret_cast<int*>(static_cast<char*>(destination) + (sortedPlacementOffset(numel) - sortedRowsOffset(numel)))
+                                 : nullptr;
 
     int count = numel;
     auto inputAcc = input.accessor<kernel::Tensor2Read<float>>();
@@ -1939,7 +1947,7 @@ bool FusedNetwork::sortPoints(const Tensor& input, kernel::Tensor2Read<float>& s
         po.scan.value().launch(SLABS / 16, BLOCK, 0, stream, args);   // 16 slabs per workgroup (POINT_ORDER_SCAN_SLABS)
     }
     {
-        void* args[] = {&count, &inputAcc, &key, &histogram, &totals, &sortedData, &orderData};
+        void* args[] = {&count, &inputAcc, &key, &histogram, &totals, &sortedData, &orderData, &placement};
         po.scatter.value().launch(chunks, BLOCK, 0, stream, args);
     }
     sortedInput.data_ = sortedData;
@@ -1958,7 +1966,7 @@ size_t FusedNetwork::forwardMemory(int numElements, AdjointModeFlags adjointFlag
     if (adjointFlags > 0 && adjointFlags < ADJOINT_MODE_MAX_COMBINATIONS) announcedFlags_ = adjointFlags;
     // a batch that trains in sorted order: its sorted rows and the order, behind the intermediates and the derivatives
     if (sortsTraining(numElements))
-        return sortedTotalsOffset(numElements) + SORT_SLABS * sizeof(int);
+        return sortedPlacementOffset(numElements) + roundUp(static_cast<size_t>(numElements) * sizeof(int), size_t(256));
     numElements = roundUp(numElements, WARP_SIZE);
     return forwardBytesPerPoint() * static_cast<size_t>(numElements);
 }
@@ -2281,8 +2289,9 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         int channels = channelsIn();
         const float* src = sortedAdjInput.data_;
         auto dst = adjInput.accessor<kernel::Tensor2RW<float>>();
-        void* args[] = {&elements, &channels, &src, &pointOrder, &dst};
-        pointOrder_.scatterAddRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0,
+        const int* placement = reinterpret_cast<const int*>(static_cast<const char*>(tmpMemoryForward) + sortedPlacementOffset(numel));
+        void* args[] = {&elements, &channels, &src, &placement, &dst};
+        pointOrder_.gatherAddRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0,
                                                   stream, args);
     }
 
@@ -2342,7 +2351,7 @@ void FusedNetwork::clearCachedKernels()
     pointOrder_.count = {};
     pointOrder_.scatter = {};
     pointOrder_.gatherRows = {};
-    pointOrder_.scatterAddRows = {};
+    pointOrder_.gatherAddRows = {};
 }
 
 QUICKMLP_NAMESPACE_END
