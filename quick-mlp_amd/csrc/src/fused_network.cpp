@@ -703,7 +703,9 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
     // 64 -> 64 -> 64 -> 16 (36 tiles) on 10^6 points 530 -> 505 us. Networks that 16 tiles fuse completely lose
     // 8-14 % with one wavefront per SIMD, 64 x 4 hidden layers (68 tiles, partly fused) gain nothing, and where 16
     // tiles leave out only a small layer (32 x 4 hidden layers: 16 of 18 tiles) the smaller kernel stays ahead
-    // (forward + backward 300 against 317 us).
+    // (forward + backward 300 against 317 us) -- unless the kernel that holds every tile may also run the layers
+    // again, so that the training pass stores the encoded input only (layers of up to 32 channels, whose
+    // pre-activations fit beside the tiles: 32 x 4 hidden layers 300 -> 230 us).
     std::sort(byTiles.begin(), byTiles.end());
     int within = 0;
     for (const auto& [count, layer] : byTiles) {
@@ -711,7 +713,10 @@ std::vector<bool> FusedNetwork::fusedWeightUpdateLayers(int adjointFlags, bool s
         within += count;
     }
     if (wideRegisters) *wideRegisters = false;
-    if (compileOptions_.fusedWeightUpdate < 0 && allTiles <= 48 && allTiles - within >= 12) {
+    int widest = 0;
+    for (const auto& l : layers_) widest = std::max(widest, std::max(l.channelsIn, l.channelsOut));
+    const bool runsLayersAgain = compileOptions_.recomputeIntermediates != 0 && widest <= 32 && allTiles > within;
+    if (compileOptions_.fusedWeightUpdate < 0 && allTiles <= 48 && (allTiles - within >= 12 || runsLayersAgain)) {
         budget = allTiles;
         if (wideRegisters) *wideRegisters = true;
     }
