@@ -33,8 +33,8 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, published
 # code: "kernels" is device_code_hash() at the time of the counter runs, and a workload whose
 # device code has changed since (or that has no counter run) reports traffic null.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2-inference": {"points": 1 << 20, "fetch": 105169.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
-                       "kernels": "4ad4add129c4ab5d"},
+    "cfg2-inference": {"points": 1 << 20, "fetch": 105163.0 * 1024 * 2.0, "write": 4096.0 * 1024 * 1.0,
+                       "kernels": "6abc8c19b03aa50d"},
 }
 
 
