@@ -62,6 +62,11 @@ int qmlp_is_compile_debug_mode(int* enabled);               /* isCompileDebugMod
 int qmlp_set_kernel_cache_dir(const char* directory);
 /* Number of runtime compilations / disk-cache hits so far (diagnostics). */
 int qmlp_kernel_cache_stats(int* compilations, int* disk_hits);
+/* Whether kernels without template arguments that ask for it are compiled by the offline compiler of the installed
+ * ROCm (<ROCM_PATH>/bin/hipcc as a child process; QMLP_COMPILER=hiprtc in the environment switches it off) instead of
+ * the run-time compiler that the process has loaded, and how many were so far. No counterpart in the reference
+ * (its loader only has NVRTC); diagnostics for tests and logs. */
+int qmlp_kernel_compiler_stats(int* has_offline_compiler, int* offline_compilations);
 
 /* ---- qmlp::FusedNetwork (src_cpp/include/qmlp/fused_network.h:16-338) ---- */
 /* FusedNetwork(cfg, parent), fused_network.h:157 / src_cpp/src/fused_network.cpp:33-223 */

@@ -468,7 +468,7 @@ private:
     void compileRecordsKernel(SliceGradientKernel& sk, int flags, size_t variant, bool compileOnly, bool fromDerivatives = false);
 
     std::string forwardSource(int blockSize, int pointsPerLane, bool registerStaging = false, bool derivatives = false, bool inputOnly = false) const;
-    std::string backwardSource(int flags, int blockSize, bool sliceGradients = false, bool recompute = false) const;
+    std::string backwardSource(int flags, int blockSize, bool sliceGradients = false, bool recompute = false, bool twoWavefrontsPerSimd = false) const;
     std::string weightUpdateSource(int blockSize) const;
     std::string weightUpdateKernelName(int layer, int& numChunks, int& tilesPerBlock) const;
     void fillEncodingsAndActivations(std::string& codeTemplate) const;

@@ -72,7 +72,8 @@ public:
     {
         CompileDebugMode = 1,      // -g, reduced optimization
         CompileThrowOnError = 2,   // throw instead of returning an empty optional
-        CompileOnly = 4            // compile (and cache) without loading onto a device
+        CompileOnly = 4,           // compile (and cache) without loading onto a device
+        CompileOffline = 8         // with the offline compiler of the installed ROCm where there is one (see hasOfflineCompiler)
     };
     static const std::filesystem::path DEFAULT_CACHE_DIR;
 
@@ -98,8 +99,22 @@ public:
      * Compiles 'source' (or fetches it from the caches) and returns the function with
      * the C++ name 'kernelName' (template arguments allowed).
      * With CompileOnly the returned function is undefined but the code object is cached.
+     * offlineOptions: further options for the offline compiler where CompileOffline takes effect (the run-time
+     * compiler, which may not know them, never sees them).
      */
-    std::optional<KernelFunction> getKernel(const std::string& kernelName, const std::string& source, int flags);
+    std::optional<KernelFunction> getKernel(const std::string& kernelName, const std::string& source, int flags,
+                                            const std::vector<std::string>& offlineOptions = {});
+
+    /**
+     * True if kernels can be compiled by the offline compiler of the installed ROCm (`<ROCM_PATH>/bin/hipcc`, run as
+     * a child process) instead of the run-time compiler of the process. The run-time compiler is whatever
+     * `libhiprtc` the process has loaded: a Python process that imported torch first compiles with the one that torch
+     * ships, which can be older than the installed ROCm (register allocation of kernels that hold many matrix-core
+     * accumulators differs a lot between them). `QMLP_COMPILER=hiprtc` in the environment switches it off. Only
+     * kernels without template arguments can take this path (their symbol is found by its mangled qualified name);
+     * a failure of the child process falls back to the run-time compiler.
+     */
+    [[nodiscard]] static bool hasOfflineCompiler();
 
     /** Drops all in-memory modules (kernels already handed out stay valid). */
     void clearMemoryCache();
@@ -107,6 +122,7 @@ public:
     /** Statistics for tests and logs. */
     [[nodiscard]] int numCompilations() const { return numCompilations_; }
     [[nodiscard]] int numDiskHits() const { return numDiskHits_; }
+    [[nodiscard]] int numOfflineCompilations() const { return numOfflineCompilations_; }
 
 private:
     struct Entry
@@ -124,6 +140,7 @@ private:
     std::mutex mutex_;
     int numCompilations_ = 0;
     int numDiskHits_ = 0;
+    int numOfflineCompilations_ = 0;
 
     void loadHeaders();
     /** Digest of the device headers that 'source' includes, directly or through other headers. */
@@ -132,6 +149,9 @@ private:
                          const std::vector<std::string>& options) const;
     bool loadFromDisk(const std::string& key, Entry& entry);
     void saveToDisk(const std::string& key, const Entry& entry);
+    /** The code object of `source` from the offline compiler and the symbol of the kernel in it; false (with the reason in `log`) if anything fails. */
+    bool compileOffline(const std::string& kernelName, const std::string& source, const std::vector<std::string>& options,
+                        Entry& entry, std::string& log) const;
 };
 typedef std::shared_ptr<KernelLoader> KernelLoader_ptr;
 

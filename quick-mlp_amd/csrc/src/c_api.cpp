@@ -173,6 +173,15 @@ int qmlp_kernel_cache_stats(int* compilations, int* disk_hits)
     QMLP_API_END
 }
 
+int qmlp_kernel_compiler_stats(int* has_offline_compiler, int* offline_compilations)
+{
+    QMLP_API_BEGIN
+    auto kl = QuickMLP::Instance().kernelLoader();
+    if (has_offline_compiler) *has_offline_compiler = KernelLoader::hasOfflineCompiler() ? 1 : 0;
+    if (offline_compilations) *offline_compilations = kl->numOfflineCompilations();
+    QMLP_API_END
+}
+
 // ---------------------------------------------------------------- network
 
 int qmlp_network_create(const char* cfg_json, const char* parent_directory, qmlp_network_t* network)

@@ -924,7 +924,7 @@ int FusedNetwork::ldsGradientLayout(int adjointFlags, int blockSize, std::vector
     return bytes;
 }
 
-std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGradients, bool recompute) const
+std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGradients, bool recompute, bool twoWavefrontsPerSimd) const
 {
     const bool hasInputGradients = flags & GRADIENTS_INPUT;
     const bool hasNetworkGradients = flags & GRADIENTS_NETWORK_WEIGHTS;
@@ -937,8 +937,9 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     bool wideRegisters = false;
     (void)fusedWeightUpdateLayers(flags, sliceGradients, &wideRegisters);
     // (the pre-activations of all layers stay in registers beside the gradient tiles: 256 registers spilled 404 bytes
-    // per lane for 16 -> 32 -> 32 -> 32 -> 16)
-    wideRegisters = wideRegisters || recompute;
+    // per lane for 16 -> 32 -> 32 -> 32 -> 16 with the run-time compiler that ships with torch 2.10; the offline compiler of
+    // ROCm 7.2 needs 232 registers and no scratch for the same source, see compileBackwardKernel)
+    wideRegisters = (wideRegisters || recompute) && !twoWavefrontsPerSimd;
     replaceAll(code, "$$KERNEL_ATTRIBUTES$$", wideRegisters ? std::string("__attribute__((amdgpu_waves_per_eu(1, 1)))") : kernelAttributes(blockSize));
     // (set below: input gradients that the kernels of the gradient slices compute are none of this kernel's)
     replaceAll(code, "$$HAS_NETWORK_GRADIENTS$$", hasNetworkGradients ? "true" : "false");
@@ -1446,14 +1447,49 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
                                                    * fusedWeightUpdateTransposeHalves(recompute) * static_cast<int>(sizeof(half)),
                                                widestTiles * 256 * static_cast<int>(sizeof(float)));
     }
-    const std::string adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients, recompute);
-    ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, loaderFlags(compileOnly)).value();
+    // Which compiler and how many registers. The run-time compiler is the one of the process (a Python process that
+    // imported torch compiles with the libamd_comgr that torch ships, ROCm 7.0's under torch 2.10); where the installed
+    // ROCm has an offline compiler, the kernels that hold gradient tiles are given to it:
+    //  - the kernel that runs the layers again, within the 256 registers of two wavefronts per SIMD: BASELINE config 5
+    //    needs 232 registers and no scratch there against 404 bytes of scratch from the run-time compiler, and takes
+    //    135 instead of 233 us, also because no matrix result passes through accumulation registers. Taken if it does
+    //    not spill; a pass that only fills the cache cannot know and compiles the next form as well.
+    //  - kernels of one wavefront per SIMD with the matrix instructions in their vector-register form: a kernel that may
+    //    use more than 256 registers otherwise gets every matrix result in an accumulation register and copies each
+    //    value out (a quarter of the instructions of such a kernel's loop).
+    std::string adjointSource;
+    int adjointLoaderFlags = loaderFlags(compileOnly);
+    std::vector<std::string> offlineOptions;
+    bool wideByTiles = false;
+    (void)fusedWeightUpdateLayers(flags, sliceGradients, &wideByTiles);
+    const bool offlineCompiler = KernelLoader::hasOfflineCompiler() && (recompute || wideByTiles);
+    bool chosen = false;
+    if (recompute && offlineCompiler) {
+        adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients, true, true);
+        auto fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, adjointLoaderFlags | KernelLoader::CompileOffline);
+        if (fun.has_value() && !compileOnly && fun.value().scratchBytes() <= MAX_RECOMPUTE_SCRATCH) {
+            ak.adjoint.fun = fun.value();
+            adjointLoaderFlags |= KernelLoader::CompileOffline;
+            chosen = true;
+        } else if (fun.has_value() && !compileOnly) {
+            logger->debug("the backward kernel that runs the layers again (flags %d) spills %d bytes per lane with two wavefronts per SIMD",
+                          flags, fun.value().scratchBytes());
+        }
+    }
+    if (!chosen) {
+        adjointSource = backwardSource(flags, ak.adjoint.blockSize, sliceGradients, recompute);
+        if (offlineCompiler) {
+            adjointLoaderFlags |= KernelLoader::CompileOffline;
+            offlineOptions = {"-mllvm", "-amdgpu-mfma-vgpr-form"};
+        }
+        ak.adjoint.fun = kl->getKernel("qmlp::kernel::NetworkKernelBackward", adjointSource, adjointLoaderFlags, offlineOptions).value();
+    }
     {
         std::vector<long long> transposed;
         if (transposedWeightLayout(flags, transposed) > 0) {
             ak.transpose.blockSize = 256;
             ak.transpose.fun =
-                kl->getKernel("qmlp::kernel::TransposeWeightsKernel", adjointSource, loaderFlags(compileOnly)).value();
+                kl->getKernel("qmlp::kernel::TransposeWeightsKernel", adjointSource, adjointLoaderFlags, offlineOptions).value();
         }
     }
     if (!compileOnly) {

@@ -8,7 +8,12 @@
 #include <cstring>
 #include <fstream>
 #include <sstream>
+#include <fcntl.h>
+#include <spawn.h>
+#include <sys/wait.h>
 #include <unistd.h>
+
+extern char** environ;
 
 QUICKMLP_NAMESPACE_BEGIN
 
@@ -50,6 +55,71 @@ std::string rocmIncludeDir()
 }
 
 const char CACHE_MAGIC[8] = {'Q', 'M', 'L', 'P', 'C', 'O', '0', '1'};
+
+std::string rocmRoot()
+{
+    const char* env = std::getenv("ROCM_PATH");
+    return env && *env ? env : "/opt/rocm";
+}
+
+// The offline compiler of the installed ROCm: its path (empty: none, or switched off) and what identifies its
+// version in a cache key, read from a file so that no process has to be started to look a kernel up.
+struct OfflineCompiler
+{
+    std::string path, id;
+};
+const OfflineCompiler& offlineCompiler()
+{
+    static const OfflineCompiler compiler = [] {
+        OfflineCompiler c;
+        const char* choice = std::getenv("QMLP_COMPILER");
+        if (choice && std::string(choice) == "hiprtc") return c;
+        const std::string path = rocmRoot() + "/bin/hipcc";
+        if (::access(path.c_str(), X_OK) != 0) return c;
+        std::string version = readFile(rocmRoot() + "/.info/version");
+        version = version.substr(0, version.find_first_of("\r\n"));
+        if (version.empty()) return c;   // nothing to tell two installations apart by
+        c.path = path;
+        c.id = "hipcc " + version;
+        return c;
+    }();
+    return compiler;
+}
+
+// Symbols of the kernels in a code object (ELF64, little endian): every kernel has a descriptor "<symbol>.kd".
+std::vector<std::string> kernelSymbols(const std::string& elf)
+{
+    std::vector<std::string> symbols;
+    auto u16 = [&](size_t at) { uint16_t v = 0; if (at + 2 <= elf.size()) std::memcpy(&v, elf.data() + at, 2); return v; };
+    auto u32 = [&](size_t at) { uint32_t v = 0; if (at + 4 <= elf.size()) std::memcpy(&v, elf.data() + at, 4); return v; };
+    auto u64 = [&](size_t at) { uint64_t v = 0; if (at + 8 <= elf.size()) std::memcpy(&v, elf.data() + at, 8); return v; };
+    if (elf.size() < 64 || std::memcmp(elf.data(), "\177ELF", 4) != 0 || elf[4] != 2 || elf[5] != 1) return symbols;
+    const uint64_t shoff = u64(0x28);
+    const uint16_t shentsize = u16(0x3A), shnum = u16(0x3C);
+    auto section = [&](uint32_t i) { return shoff + static_cast<uint64_t>(i) * shentsize; };
+    for (uint32_t i = 0; i < shnum; ++i) {
+        const uint64_t sh = section(i);
+        if (sh + 64 > elf.size()) return symbols;
+        const uint32_t type = u32(sh + 4);
+        if (type != 2 && type != 11) continue;   // SHT_SYMTAB, SHT_DYNSYM
+        const uint64_t offset = u64(sh + 24), size = u64(sh + 32), entsize = u64(sh + 56);
+        const uint32_t link = u32(sh + 40);
+        if (link >= shnum || entsize < 24) continue;
+        const uint64_t strOffset = u64(section(link) + 24), strSize = u64(section(link) + 32);
+        if (strOffset + strSize > elf.size() || offset + size > elf.size()) continue;
+        for (uint64_t at = offset; at + entsize <= offset + size; at += entsize) {
+            const uint32_t name = u32(at);
+            if (name >= strSize) continue;
+            const char* text = elf.data() + strOffset + name;
+            const size_t length = ::strnlen(text, strSize - name);
+            if (length > 3 && std::memcmp(text + length - 3, ".kd", 3) == 0) {
+                std::string symbol(text, length - 3);
+                if (std::find(symbols.begin(), symbols.end(), symbol) == symbols.end()) symbols.push_back(std::move(symbol));
+            }
+        }
+    }
+    return symbols;
+}
 
 } // namespace
 
@@ -322,7 +392,7 @@ void KernelLoader::saveToDisk(const std::string& key, const Entry& entry)
 }
 
 std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelName, const std::string& source,
-                                                      int flags)
+                                                      int flags, const std::vector<std::string>& offlineOptions)
 {
     std::lock_guard<std::mutex> lock(mutex_);
     const bool debug = (flags & CompileDebugMode) != 0;
@@ -344,8 +414,16 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
         while (ss >> tok) options.push_back(tok);
     }
 
+    // (part of the key, not of the command line: a cache filled by one compiler is not taken for the other's)
+    const bool offline = (flags & CompileOffline) != 0 && hasOfflineCompiler() && kernelName.find('<') == std::string::npos;
+    std::vector<std::string> keyOptions = options;
+    if (offline) {
+        keyOptions.push_back("compiler: " + offlineCompiler().id);
+        keyOptions.insert(keyOptions.end(), offlineOptions.begin(), offlineOptions.end());
+    }
+
     try {
-        const std::string key = cacheKey(kernelName, source, options);
+        const std::string key = cacheKey(kernelName, source, keyOptions);
         auto it = modules_.find(key);
         if (it == modules_.end()) {
             Entry entry;
@@ -355,6 +433,23 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
             } else {
                 logger_->info("compiling kernel %s", kernelName.c_str());
                 if (logger_->should_log(Logger::DEBUG)) logger_->debug("source:\n%s", source.c_str());
+                bool compiled = false;
+                if (offline) {
+                    std::string offlineLog;
+                    std::vector<std::string> allOptions = options;
+                    allOptions.insert(allOptions.end(), offlineOptions.begin(), offlineOptions.end());
+                    compiled = compileOffline(kernelName, source, allOptions, entry, offlineLog);
+                    if (compiled) {
+                        ++numCompilations_;
+                        ++numOfflineCompilations_;
+                        if (!offlineLog.empty()) logger_->debug("compiler log of %s:\n%s", kernelName.c_str(), offlineLog.c_str());
+                        saveToDisk(key, entry);
+                    } else {
+                        logger_->warn("offline compilation of %s failed, the run-time compiler takes it: %s", kernelName.c_str(), offlineLog.c_str());
+                        entry = Entry();
+                    }
+                }
+                if (!compiled) {
                 std::vector<const char*> hn, hc, opts;
                 for (const auto& n : headerNames_) hn.push_back(n.c_str());
                 for (const auto& c : headerContents_) hc.push_back(c.c_str());
@@ -380,6 +475,7 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
                 QMLP_HIP_CALL(qmlp_hip_module_lowered_name(m, kernelName.c_str(), &lowered));
                 entry.lowered[kernelName] = lowered;
                 saveToDisk(key, entry);
+                }
             }
             it = modules_.emplace(key, std::move(entry)).first;
         }
@@ -397,6 +493,102 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
         if (throwOnError) throw;
         return {};
     }
+}
+
+bool KernelLoader::hasOfflineCompiler()
+{
+    return !offlineCompiler().path.empty();
+}
+
+bool KernelLoader::compileOffline(const std::string& kernelName, const std::string& source, const std::vector<std::string>& options,
+                                  Entry& entry, std::string& log) const
+{
+    namespace fs = std::filesystem;
+    const OfflineCompiler& compiler = offlineCompiler();
+    if (compiler.path.empty()) { log = "no offline compiler"; return false; }
+    if (kernelName.find('<') != std::string::npos) { log = "kernels with template arguments are left to the run-time compiler"; return false; }
+    std::string processor;
+    {
+        char* target = nullptr;
+        if (qmlp_hip_compile_target(std::getenv("QMLP_OFFLOAD_ARCH"), &target) != 0 || !target) { log = "no compile target"; return false; }
+        processor = target;
+        qmlp_hip_free_string(target);
+        processor = processor.substr(0, processor.find(';'));
+    }
+    std::error_code ec;
+    std::string pattern = (fs::temp_directory_path(ec) / "qmlp-offline-XXXXXX").string();
+    if (ec || !::mkdtemp(&pattern[0])) { log = "cannot create a temporary directory"; return false; }
+    const fs::path dir = pattern;
+    struct Cleanup { fs::path dir; ~Cleanup() { std::error_code e; fs::remove_all(dir, e); } } cleanup{dir};
+    // the same headers the run-time compiler is given, from memory: what is on disk may have changed since they were read
+    for (size_t i = 0; i < headerNames_.size(); ++i) {
+        const fs::path file = dir / "include" / headerNames_[i];
+        fs::create_directories(file.parent_path(), ec);
+        std::ofstream(file, std::ios::binary) << headerContents_[i];
+    }
+    std::ofstream(dir / "kernel.hip", std::ios::binary) << source;
+    const std::string output = (dir / "kernel.co").string(), messages = (dir / "messages.txt").string();
+    std::vector<std::string> arguments = {compiler.path, "--genco", "--no-gpu-bundle-output", "--offload-arch=" + processor};
+    for (const auto& o : options) arguments.push_back(o);
+    arguments.push_back("-I" + (dir / "include").string());
+    arguments.push_back("-o");
+    arguments.push_back(output);
+    arguments.push_back((dir / "kernel.hip").string());
+    std::vector<char*> argv;
+    for (auto& a : arguments) argv.push_back(&a[0]);
+    argv.push_back(nullptr);
+    posix_spawn_file_actions_t actions;
+    posix_spawn_file_actions_init(&actions);
+    posix_spawn_file_actions_addopen(&actions, 0, "/dev/null", O_RDONLY, 0);
+    posix_spawn_file_actions_addopen(&actions, 1, messages.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0600);
+    posix_spawn_file_actions_adddup2(&actions, 1, 2);
+    pid_t child = 0;
+    const int spawned = posix_spawn(&child, compiler.path.c_str(), &actions, nullptr, argv.data(), environ);
+    posix_spawn_file_actions_destroy(&actions);
+    if (spawned != 0) { log = std::string("cannot start ") + compiler.path + ": " + std::strerror(spawned); return false; }
+    int status = 0;
+    while (::waitpid(child, &status, 0) < 0) {
+        if (errno != EINTR) { log = "waiting for the compiler failed"; return false; }
+    }
+    log = readFile(messages);
+    if (!WIFEXITED(status) || WEXITSTATUS(status) != 0) {
+        log = compiler.path + " failed:\n" + log;
+        return false;
+    }
+    const std::string code = readFile(output);
+    // The symbol of a function without template arguments starts with its mangled qualified name, the parameter types
+    // follow: _ZN <length><component>... E for a name in namespaces, _Z <length><name> for one outside (or the plain name
+    // of an extern "C" function). Two overloads of one name are not told apart: left to the run-time compiler.
+    std::string prefix, plain;
+    {
+        std::vector<std::string> components;
+        size_t from = 0;
+        for (size_t at; (at = kernelName.find("::", from)) != std::string::npos; from = at + 2) components.push_back(kernelName.substr(from, at - from));
+        components.push_back(kernelName.substr(from));
+        if (components.size() == 1) {
+            plain = components[0];
+            prefix = "_Z" + std::to_string(plain.size()) + plain;
+        } else {
+            prefix = "_ZN";
+            for (const auto& c : components) prefix += std::to_string(c.size()) + c;
+            prefix += "E";
+        }
+    }
+    std::string symbol;
+    int matches = 0;
+    for (const std::string& candidate : kernelSymbols(code)) {
+        if (candidate.compare(0, prefix.size(), prefix) == 0 || (!plain.empty() && candidate == plain)) {
+            symbol = candidate;
+            ++matches;
+        }
+    }
+    if (matches > 1) symbol.clear();
+    if (symbol.empty()) { log = "the code object of the offline compiler has no kernel " + kernelName + "\n" + log; return false; }
+    qmlp_hip_module m = nullptr;
+    if (qmlp_hip_module_from_code(code.data(), code.size(), &m) != 0) { log = "cannot keep the code object"; return false; }
+    entry.module = std::shared_ptr<qmlp_hip_module_s>(m, ModuleDeleter());
+    entry.lowered[kernelName] = symbol;
+    return true;
 }
 
 void KernelLoader::clearMemoryCache()

@@ -53,6 +53,7 @@ _SIGNATURES = {
     "qmlp_is_compile_debug_mode": [_pi],
     "qmlp_set_kernel_cache_dir": [ctypes.c_char_p],
     "qmlp_kernel_cache_stats": [_pi, _pi],
+    "qmlp_kernel_compiler_stats": [_pi, _pi],
     "qmlp_network_create": [ctypes.c_char_p, ctypes.c_char_p, _P(_vp)],
     "qmlp_network_destroy": [_vp],
     "qmlp_network_channels_in": [_vp, _pi],
@@ -177,6 +178,13 @@ def kernel_cache_stats():
     a, b = ctypes.c_int(), ctypes.c_int()
     check(lib.qmlp_kernel_cache_stats(ctypes.byref(a), ctypes.byref(b)))
     return a.value, b.value
+
+
+def kernel_compiler_stats():
+    """(whether the offline compiler of the installed ROCm takes the kernels that ask for it, how many it compiled so far)"""
+    a, b = ctypes.c_int(), ctypes.c_int()
+    check(lib.qmlp_kernel_compiler_stats(ctypes.byref(a), ctypes.byref(b)))
+    return bool(a.value), b.value
 
 
 set_kernel_cache_dir(os.environ.get("QMLP_CACHE_DIR", DEFAULT_CACHE_DIR))

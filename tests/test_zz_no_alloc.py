@@ -3,6 +3,7 @@ qmlp_network_inference on the same inputs: bit for bit (every point is evaluated
 whatever the order of the batch), on two calls in a row, the second on a smaller batch, with a
 network whose batches are ordered by grid slab in the library's static device buffer; then networks
 that never use the buffer, and the hand-over of the buffer between streams."""
+import gc
 import json
 import os
 
@@ -182,6 +183,7 @@ def test_prepare_leaves_nothing_to_load_or_allocate_for_a_train_step():
     del plain, spare                     # torch's allocator keeps the blocks of one more step for the results below
     net = qmlp.Network(json.dumps(cfg))
     net.prepare(n, flags)
+    gc.collect()                         # networks of earlier tests that wait for the collector would unload their kernels below
     torch.cuda.synchronize()
     stats = qmlp._lib.kernel_cache_stats()
     free_before = torch.cuda.mem_get_info()[0]
