@@ -433,6 +433,13 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
             } else {
                 logger_->info("compiling kernel %s", kernelName.c_str());
                 if (logger_->should_log(Logger::DEBUG)) logger_->debug("source:\n%s", source.c_str());
+                if (const char* dump = std::getenv("QMLP_DUMP_SOURCES")) {
+                    // debugging aid: the source and the name of every kernel that is compiled, by cache key
+                    std::error_code dumpError;
+                    std::filesystem::create_directories(dump, dumpError);
+                    std::ofstream(std::filesystem::path(dump) / (key + ".hip"), std::ios::binary) << source;
+                    std::ofstream(std::filesystem::path(dump) / (key + ".name"), std::ios::binary) << kernelName;
+                }
                 bool compiled = false;
                 if (offline) {
                     std::string offlineLog;
