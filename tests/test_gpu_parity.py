@@ -1378,6 +1378,40 @@ def test_grid_gradients_summed_by_columns_match_the_records_the_atomic_scatter_a
     assert np.allclose(a[ok] / scale, b[ok] / scale, rtol=1e-4, atol=2e-5)
 
 
+def test_backward_kernel_from_the_offline_compiler_runs_two_wavefronts_per_simd():
+    """Where the installed ROCm has an offline compiler (KernelLoader::CompileOffline), the backward kernel that runs
+    the layers again is compiled by it for 256 registers and taken if it does not spill: workgroups of four wavefronts,
+    two of them resident per compute unit. Its gradients are checked against the oracle like any other kernel's, and
+    bit for bit against the kernels that read stored intermediates (from the run-time compiler of the process)."""
+    base = identity_cfg(16, [32, 32, 4], ["sine", "celu", "identity"], [False, True, False])
+    off = dict(base, options={"recompute_intermediates": 0})
+    warm_cache(base, off)
+    offline, _ = qmlp._lib.kernel_compiler_stats()
+    if not offline:
+        pytest.skip("no offline compiler in this installation (or QMLP_COMPILER=hiprtc)")
+    cases = {"on": Case(base), "off": Case(off)}
+    rng = np.random.default_rng(43)
+    params = random_parameters(cases["on"].oracle, rng)
+    for c in cases.values():
+        c.set_parameters(params)
+    full = FLAG_INPUT | FLAG_WEIGHTS
+    res = json.loads(cases["on"].net.generated_source("backward_resources", full))
+    assert res["recompute"] is True and res["block"] == 256 and res["scratch_bytes"] <= 64 and res["registers"] <= 256
+    assert res["full_grid"] == 2 * torch.cuda.get_device_properties(0).multi_processor_count
+    N = 4099
+    X = rng.uniform(-1, 1, (N, 16)).astype(np.float32)
+    adj = (rng.uniform(-1, 1, (N, 4)) / 16).astype(np.float32)
+    got = {k: c.gpu_train(X, adj, full) for k, c in cases.items()}
+    for key in ("out", "adj_x", "grads"):
+        assert np.array_equal(got["on"][key], got["off"][key]), key
+    # (against the fp32 oracle at rel 1e-2 / abs 1e-3 of the largest entry; the oracle that rounds where the device
+    # rounds is matched by the kernels this one equals bit for bit in the tests of the stored intermediates)
+    ref = cases["on"].oracle.backward(X, adj, full, round_mode=0)
+    for key in ("adj_x", "grads"):
+        scale = max(1.0, float(np.abs(ref[key]).max()))
+        assert_close(got["on"][key] / scale, ref[key] / scale, key + " vs fp32 oracle")
+
+
 @pytest.mark.parametrize("which", ["hashgrid", "identity"])
 def test_backward_kernel_that_runs_the_layers_again_gives_the_same_bits(which):
     """options.recompute_intermediates (default: when announced): where the backward kernel sums the weight gradients
