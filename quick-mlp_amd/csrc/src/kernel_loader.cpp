@@ -456,6 +456,7 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
                         entry = Entry();
                     }
                 }
+                const bool fallback = offline && !compiled;   // stays in memory: the key on disk names the offline compiler
                 if (!compiled) {
                 std::vector<const char*> hn, hc, opts;
                 for (const auto& n : headerNames_) hn.push_back(n.c_str());
@@ -481,7 +482,7 @@ std::optional<KernelFunction> KernelLoader::getKernel(const std::string& kernelN
                 const char* lowered = nullptr;
                 QMLP_HIP_CALL(qmlp_hip_module_lowered_name(m, kernelName.c_str(), &lowered));
                 entry.lowered[kernelName] = lowered;
-                saveToDisk(key, entry);
+                if (!fallback) saveToDisk(key, entry);
                 }
             }
             it = modules_.emplace(key, std::move(entry)).first;
@@ -514,6 +515,11 @@ bool KernelLoader::compileOffline(const std::string& kernelName, const std::stri
     const OfflineCompiler& compiler = offlineCompiler();
     if (compiler.path.empty()) { log = "no offline compiler"; return false; }
     if (kernelName.find('<') != std::string::npos) { log = "kernels with template arguments are left to the run-time compiler"; return false; }
+    // A preloaded profiler library would be loaded into the compiler's processes as well and set up the device in each
+    // of them before they start their own children: no child processes under a profiler.
+    if (const char* preload = std::getenv("LD_PRELOAD")) {
+        if (std::strstr(preload, "rocprof") || std::strstr(preload, "roctracer")) { log = "a profiler is preloaded into this process"; return false; }
+    }
     std::string processor;
     {
         char* target = nullptr;
