@@ -165,7 +165,7 @@ private:
     struct PointOrder
     {
         std::optional<KernelFunction> count, scan, scatter;
-        std::optional<KernelFunction> gatherRows, gatherAddRows;   // rows of dL/dy into, rows of the input gradients out of the sorted order
+        std::optional<KernelFunction> gatherAddRows;   // rows of the input gradients out of the sorted order
         Tensor workspace;           // slab totals and per-chunk histograms (ints), sorted inputs (floats), order (ints)
         long long capacityWords = 0;   // 32-bit words the workspace holds
     };

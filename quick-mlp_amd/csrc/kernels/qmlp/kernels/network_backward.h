@@ -67,7 +67,8 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     half* __restrict__ adjointTmpMemoryH,        //receives dpre if weight gradients are requested
     const half* __restrict__ transposedWeightsH, //W^T of the layers whose weights do not stay in LDS, or nullptr
     float* __restrict__ partialGradients,        //FUSED_WEIGHT_UPDATE: partialSlices x the layout of the parameters; workgroup b
-    int partialSlices                            //stores the sums of its tiles into slice b (and zeroes slices b + k * gridDim.x)
+    int partialSlices,                           //stores the sums of its tiles into slice b (and zeroes slices b + k * gridDim.x)
+    const int* __restrict__ adjOutputOrder       //nullptr, or (numel): the row of adjOutputs that belongs to point p (a batch that trains in sorted order)
     $$ENCODING_PARAMETERS$$)
 {
     constexpr int NUM_INPUTS = $$NUM_INPUTS$$;
@@ -153,10 +154,11 @@ $$ZERO_LDS_GRADIENTS$$
             const int p = tile * TILE_POINTS + 4 * r + nt;
             const bool pv = p < numel;
             validMask |= pv ? (1 << nt) : 0;
+            const long long adjRow = (adjOutputOrder && pv) ? adjOutputOrder[p] : p;
             if (adjOutputRowsOfFloat2 || adjOutputRowsOfFloat4) {
                 // channels side by side in memory: four per load (a lane holds channels
                 // 16m+4g .. +3 of its points), a row of two channels as one 8-byte load
-                const float* row = adjOutputs.data_ + static_cast<long long>(p) * adjOutputs.strides_[0];
+                const float* row = adjOutputs.data_ + adjRow * adjOutputs.strides_[0];
 #pragma unroll
                 for (int m = 0; m < MTL; ++m) {
 #pragma unroll
@@ -183,7 +185,7 @@ $$ZERO_LDS_GRADIENTS$$
                         const int c = 16 * m + 4 * g + i;
                         float v = 0.f;
                         if (pv && c < actualChannelsOut)
-                            v = adjOutputs.data_[static_cast<long long>(p) * adjOutputs.strides_[0]
+                            v = adjOutputs.data_[adjRow * adjOutputs.strides_[0]
                                                  + static_cast<long long>(c) * adjOutputs.strides_[1]];
                         dyOut[nt][m][i] = static_cast<f16>(v);
                     }

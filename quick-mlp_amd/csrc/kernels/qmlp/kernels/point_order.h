@@ -292,21 +292,6 @@ __global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderScatter(
 }
 
 /**
- * Rows of a caller's tensor in the sorted order: dst[i, c] = src[order[i], c] (dst dense). One
- * lane per element, so a wavefront writes consecutive words and reads short runs.
- */
-__global__ void __launch_bounds__(POINT_ORDER_BLOCK) PointOrderGatherRows(
-    long long elements, int channels, const Tensor2Read<float> src, const int* __restrict__ order, float* __restrict__ dst)
-{
-    for (long long e = static_cast<long long>(blockIdx.x) * POINT_ORDER_BLOCK + threadIdx.x; e < elements;
-         e += static_cast<long long>(gridDim.x) * POINT_ORDER_BLOCK) {
-        const long long row = e / channels;
-        const int c = static_cast<int>(e - row * channels);
-        dst[e] = src.data_[static_cast<long long>(order[row]) * src.strides_[0] + static_cast<long long>(c) * src.strides_[1]];
-    }
-}
-
-/**
  * Rows that were computed in the sorted order, added to the caller's tensor: dst[j, c] += src[placement[j], c]
  * (src dense). The rows of dst are walked in their own order, so the read-modify-write is coalesced and only the
  * reads of src are scattered (2^21 rows of 16 bytes: 76 us as a scatter through `order`, whose rows of 16 bytes

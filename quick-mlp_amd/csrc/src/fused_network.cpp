@@ -1701,7 +1701,7 @@ void FusedNetwork::precompile(int adjointFlags)
             const std::string source = KernelLoader::MainFile("qmlp/kernels/point_order.h");
             const std::string scatter = "PointOrderScatter<" + std::to_string(channelsIn_ <= 4 ? 4 : channelsIn_ <= 8 ? 8 : 16) + ">";
             for (const std::string& name : {std::string("PointOrderCount"), std::string("PointOrderScan"), scatter,
-                                            std::string("PointOrderGatherRows"), std::string("PointOrderGatherAddRows")})
+                                            std::string("PointOrderGatherAddRows")})
                 kl->getKernel("qmlp::kernel::" + name, source, loaderFlags(true));
             break;
         }
@@ -1843,10 +1843,8 @@ void FusedNetwork::loadPointOrderKernels(bool rowMoves)
         po.count = kl->getKernel("qmlp::kernel::PointOrderCount", source, loaderFlags(false)).value();
         po.scatter = kl->getKernel("qmlp::kernel::PointOrderScatter<" + std::to_string(maxChannels) + ">", source, loaderFlags(false)).value();
     }
-    if (rowMoves && !po.gatherRows.has_value()) {
-        po.gatherRows = kl->getKernel("qmlp::kernel::PointOrderGatherRows", source, loaderFlags(false)).value();
+    if (rowMoves && !po.gatherAddRows.has_value())
         po.gatherAddRows = kl->getKernel("qmlp::kernel::PointOrderGatherAddRows", source, loaderFlags(false)).value();
-    }
 }
 
 void FusedNetwork::prepare(int numel, int adjointFlags)
@@ -2077,12 +2075,11 @@ size_t FusedNetwork::adjointMemoryAsGiven(int numElements, AdjointModeFlags adjo
 
 size_t FusedNetwork::sortedAdjointBytes(int numElements, AdjointModeFlags adjointFlags, size_t bytesInFront) const
 {
-    // A batch that trains in sorted order: dL/dy gathered into that order, and the input gradients in that order
-    // before they are added to the caller's rows (each dense, 256-byte aligned, behind everything else).
-    if (!sortsTraining(numElements)) return 0;
+    // A batch that trains in sorted order: the input gradients in that order before they are added to the caller's
+    // rows (dense, 256-byte aligned, behind everything else).
+    if (!sortsTraining(numElements) || !(adjointFlags & GRADIENTS_INPUT)) return 0;
     size_t bytes = roundUp(bytesInFront, size_t(256)) - bytesInFront;
-    bytes += roundUp(static_cast<size_t>(numElements) * channelsOut() * sizeof(float), size_t(256));
-    if (adjointFlags & GRADIENTS_INPUT) bytes += roundUp(static_cast<size_t>(numElements) * channelsIn() * sizeof(float), size_t(256));
+    bytes += roundUp(static_cast<size_t>(numElements) * channelsIn() * sizeof(float), size_t(256));
     return bytes;
 }
 
@@ -2174,29 +2171,20 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
     std::memset(&sortedAdjInput, 0, sizeof(sortedAdjInput));
     if (hasInputGradients) sortedAdjInput = adjInput.accessor<kernel::Tensor2RW<float>>();
     const int* pointOrder = nullptr;
+    const int* adjOutputOrder = nullptr;
     if (sortedPoints) {
         const float* rows = reinterpret_cast<const float*>(static_cast<const char*>(tmpMemoryForward) + sortedRowsOffset(numel));
         sortedInput.data_ = rows;
         sortedInput.strides_[0] = channelsIn();
         sortedInput.strides_[1] = 1;
         pointOrder = reinterpret_cast<const int*>(rows + static_cast<long long>(numel) * channelsIn());
-        // Scattered 8- and 16-byte accesses from inside the adjoint kernel cost a third of its time (cfg5: 577 us
-        // against 389 us on a batch the caller had sorted); two streaming kernels move the rows instead.
-        auto& po = pointOrder_;
+        // The backward kernel reads its rows of dL/dy through the order (one index and one row of C_out floats per point
+        // and tile: BASELINE config 5, rows of 8 bytes, kernel 135 -> 151 us against a gather kernel of 34 us in front
+        // of it). The input gradients go the other way through dense rows behind the adjoint memory and one streaming
+        // kernel: scattered 16-byte read-modify-writes from inside the kernels cost more than that kernel's 44 us.
+        adjOutputOrder = pointOrder;
         loadPointOrderKernels(true);
         char* staging = static_cast<char*>(tmpMemoryAdjoint) + roundUp(adjointMemoryAsGiven(numel, adjointFlags), size_t(256));
-        float* adjOutputRows = reinterpret_cast<float*>(staging);
-        staging += roundUp(static_cast<size_t>(numel) * channelsOut() * sizeof(float), size_t(256));
-        {
-            long long elements = static_cast<long long>(numel) * channelsOut();
-            int channels = channelsOut();
-            auto src = adjOutput.accessor<kernel::Tensor2Read<float>>();
-            void* args[] = {&elements, &channels, &src, &pointOrder, &adjOutputRows};
-            po.gatherRows.value().launch(static_cast<int>(std::min<long long>(divUp<long long>(elements, 1024), 1 << 16)), 1024, 0, stream, args);
-        }
-        sortedAdjOutput.data_ = adjOutputRows;
-        sortedAdjOutput.strides_[0] = channelsOut();
-        sortedAdjOutput.strides_[1] = 1;
         if (hasInputGradients) {
             float* adjInputRows = reinterpret_cast<float*>(staging);
             QMLP_HIP_CALL(qmlp_hip_memset_async(adjInputRows, 0, static_cast<size_t>(numel) * channelsIn() * sizeof(float), stream));
@@ -2239,7 +2227,7 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         float* partialGradients = reinterpret_cast<float*>(static_cast<char*>(tmpMemoryAdjoint)
                                                            + static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64));
         std::vector<void*> args = {&numel, &inputAcc, &adjOutputAcc, &adjInputAcc, &networkParams,
-                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights, &partialGradients, &partialSlices};
+                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights, &partialGradients, &partialSlices, &adjOutputOrder};
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
@@ -2391,7 +2379,6 @@ void FusedNetwork::clearCachedKernels()
     pointOrder_.scan = {};
     pointOrder_.count = {};
     pointOrder_.scatter = {};
-    pointOrder_.gatherRows = {};
     pointOrder_.gatherAddRows = {};
 }
 
