@@ -139,6 +139,13 @@ $$ZERO_LDS_GRADIENTS$$
         && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 8 == 0;
     const bool adjOutputRowsOfFloat4 = actualChannelsOut % 4 == 0 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 4 == 0
         && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 16 == 0;
+    // a batch that trains in sorted order: the rows of dL/dy of this wavefront's next tile, asked for one tile ahead
+    int adjRowAhead[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int p = (static_cast<int>(blockIdx.x) * WAVES + wave) * TILE_POINTS + 4 * r + nt;
+        adjRowAhead[nt] = (adjOutputOrder && p < numel) ? adjOutputOrder[p] : p;
+    }
     for (int tileBase = blockIdx.x * WAVES; tileBase < numTiles; tileBase += gridDim.x * WAVES)
     {
         const int tile = tileBase + wave;
@@ -154,7 +161,11 @@ $$ZERO_LDS_GRADIENTS$$
             const int p = tile * TILE_POINTS + 4 * r + nt;
             const bool pv = p < numel;
             validMask |= pv ? (1 << nt) : 0;
-            const long long adjRow = (adjOutputOrder && pv) ? adjOutputOrder[p] : p;
+            const long long adjRow = adjRowAhead[nt];
+            {
+                const long long ahead = static_cast<long long>(p) + static_cast<long long>(gridDim.x) * (WAVES * TILE_POINTS);
+                adjRowAhead[nt] = (adjOutputOrder && ahead < numel) ? adjOutputOrder[ahead] : static_cast<int>(ahead < numel ? ahead : 0);
+            }
             if (adjOutputRowsOfFloat2 || adjOutputRowsOfFloat4) {
                 // channels side by side in memory: four per load (a lane holds channels
                 // 16m+4g .. +3 of its points), a row of two channels as one 8-byte load
