@@ -182,6 +182,8 @@ private:
     bool sortPoints(const Tensor& input, kernel::Tensor2Read<float>& sortedInput, const int*& order, stream_t stream,
                     bool noAlloc = false, void* destination = nullptr);
     void loadPointOrderKernels(bool rowMoves);
+    /** True if some batch size makes this network train in sorted order (its backward kernels then take the order). */
+    bool trainsSortedBatches() const;
     /** The slab key of the encoding that orders a batch of numel points, if such a batch is ordered at all
      *  (a function of the specification and numel alone). */
     bool pointOrderFor(int numel, kernel::PointOrderKey& key) const;
@@ -246,6 +248,7 @@ private:
         int perEntryAdjointMemoryBytes = 0;
         std::vector<bool> fusedLayers;    // layers whose weight gradients the adjoint kernel sums (no kernel in 'layers')
         bool fusedWeightUpdate = false;   // any of them
+        bool outputOrder = false;         // the kernel takes the order of a sorted batch for its rows of dL/dy
     };
     // [adjoint flags][grid gradients by slices instead of atomics][the layers run again instead of reading their intermediates]
     std::optional<AdjointKernel> backwardKernel_[ADJOINT_MODE_MAX_COMBINATIONS][2][2];

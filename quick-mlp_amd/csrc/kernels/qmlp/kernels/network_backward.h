@@ -67,8 +67,13 @@ __global__ void __launch_bounds__($$BLOCK_SIZE$$) $$KERNEL_ATTRIBUTES$$ NetworkK
     half* __restrict__ adjointTmpMemoryH,        //receives dpre if weight gradients are requested
     const half* __restrict__ transposedWeightsH, //W^T of the layers whose weights do not stay in LDS, or nullptr
     float* __restrict__ partialGradients,        //FUSED_WEIGHT_UPDATE: partialSlices x the layout of the parameters; workgroup b
-    int partialSlices,                           //stores the sums of its tiles into slice b (and zeroes slices b + k * gridDim.x)
-    const int* __restrict__ adjOutputOrder       //nullptr, or (numel): the row of adjOutputs that belongs to point p (a batch that trains in sorted order)
+    int partialSlices                            //stores the sums of its tiles into slice b (and zeroes slices b + k * gridDim.x)
+#if $$HAS_OUTPUT_ORDER$$
+    // Networks whose batches may train in sorted order: nullptr, or (numel) the row of adjOutputs that belongs to
+    // point p. The parameter and its code exist only in the kernels of such networks: with them the run-time compiler
+    // scheduled the kernel of 64 -> 64 x 4 -> 4 (which never sorts) so that it took 689 instead of 372 us.
+    , const int* __restrict__ adjOutputOrder
+#endif
     $$ENCODING_PARAMETERS$$)
 {
     constexpr int NUM_INPUTS = $$NUM_INPUTS$$;
@@ -139,6 +144,7 @@ $$ZERO_LDS_GRADIENTS$$
         && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 8 == 0;
     const bool adjOutputRowsOfFloat4 = actualChannelsOut % 4 == 0 && adjOutputs.strides_[1] == 1 && adjOutputs.strides_[0] % 4 == 0
         && reinterpret_cast<unsigned long long>(adjOutputs.data_) % 16 == 0;
+#if $$HAS_OUTPUT_ORDER$$
     // a batch that trains in sorted order: the rows of dL/dy of this wavefront's next tile, asked for one tile ahead
     int adjRowAhead[NT];
 #pragma unroll
@@ -146,6 +152,7 @@ $$ZERO_LDS_GRADIENTS$$
         const int p = (static_cast<int>(blockIdx.x) * WAVES + wave) * TILE_POINTS + 4 * r + nt;
         adjRowAhead[nt] = (adjOutputOrder && p < numel) ? adjOutputOrder[p] : p;
     }
+#endif
     for (int tileBase = blockIdx.x * WAVES; tileBase < numTiles; tileBase += gridDim.x * WAVES)
     {
         const int tile = tileBase + wave;
@@ -161,11 +168,15 @@ $$ZERO_LDS_GRADIENTS$$
             const int p = tile * TILE_POINTS + 4 * r + nt;
             const bool pv = p < numel;
             validMask |= pv ? (1 << nt) : 0;
+#if $$HAS_OUTPUT_ORDER$$
             const long long adjRow = adjRowAhead[nt];
             {
                 const long long ahead = static_cast<long long>(p) + static_cast<long long>(gridDim.x) * (WAVES * TILE_POINTS);
                 adjRowAhead[nt] = (adjOutputOrder && ahead < numel) ? adjOutputOrder[ahead] : static_cast<int>(ahead < numel ? ahead : 0);
             }
+#else
+            const long long adjRow = p;
+#endif
             if (adjOutputRowsOfFloat2 || adjOutputRowsOfFloat4) {
                 // channels side by side in memory: four per load (a lane holds channels
                 // 16m+4g .. +3 of its points), a row of two channels as one 8-byte load

@@ -934,6 +934,7 @@ std::string FusedNetwork::backwardSource(int flags, int blockSize, bool sliceGra
     std::string code = kl->findFile("qmlp/kernels/network_backward.h").value();
     fillEncodingsAndActivations(code);
     replaceAll(code, "$$BLOCK_SIZE$$", std::to_string(blockSize));
+    replaceAll(code, "$$HAS_OUTPUT_ORDER$$", trainsSortedBatches() ? "1" : "0");
     bool wideRegisters = false;
     (void)fusedWeightUpdateLayers(flags, sliceGradients, &wideRegisters);
     // (the pre-activations of all layers stay in registers beside the gradient tiles: 256 registers spilled 404 bytes
@@ -1432,6 +1433,7 @@ void FusedNetwork::compileBackwardKernel(int flags, bool sliceGradients, bool co
         ak.adjoint.sharedMemorySize = ldsGradientLayout(flags, ak.adjoint.blockSize, ldsGradients, sliceGradients, recompute);
     }
     ak.fusedLayers = fusedWeightUpdateLayers(flags, sliceGradients);
+    ak.outputOrder = trainsSortedBatches();
     ak.fusedWeightUpdate = false;
     for (bool f : ak.fusedLayers) ak.fusedWeightUpdate = ak.fusedWeightUpdate || f;
     if (ak.fusedWeightUpdate) {
@@ -1892,6 +1894,12 @@ void FusedNetwork::prepare(int numel, int adjointFlags)
     }
 }
 
+bool FusedNetwork::trainsSortedBatches() const
+{
+    kernel::PointOrderKey key{};
+    return compileOptions_.sortTraining && pointOrderFor(1 << 30, key);
+}
+
 bool FusedNetwork::sortsTraining(int numel) const
 {
     kernel::PointOrderKey key{};
@@ -2227,7 +2235,9 @@ void FusedNetwork::adjoint(const Tensor& input, const Tensor& adjOutput, Adjoint
         float* partialGradients = reinterpret_cast<float*>(static_cast<char*>(tmpMemoryAdjoint)
                                                            + static_cast<size_t>(ak.perEntryAdjointMemoryBytes) * static_cast<size_t>(numel64));
         std::vector<void*> args = {&numel, &inputAcc, &adjOutputAcc, &adjInputAcc, &networkParams,
-                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights, &partialGradients, &partialSlices, &adjOutputOrder};
+                                   &forwardTmpMemory, &adjointTmpMemory, &transposedWeights, &partialGradients, &partialSlices};
+        CHECK_ERROR(ak.outputOrder || adjOutputOrder == nullptr, "a batch trains in sorted order but the backward kernel does not take the order");
+        if (ak.outputOrder) args.push_back(&adjOutputOrder);
         std::vector<std::vector<char>> storage;
         encodingArguments(args, storage);
         ck.fun.launch(grid, ck.blockSize, ck.sharedMemorySize, stream, args.data());
